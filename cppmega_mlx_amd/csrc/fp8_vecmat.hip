@@ -1,0 +1,253 @@
+// FP8 (e4m3) block-scaled vecmat / skinny GEMM for decode projections (gfx950).
+//
+//   out[m, n] = sum_k dec(w[n, k]) * w_scale(n, k / 128) * x[m, k]
+//
+// The weight is read from HBM exactly once; everything else is sized so that
+// the weight stream is the only traffic that matters.
+//
+//  * M == 1  (gemv_kernel): no matrix cores.  A workgroup of 4 wavefronts owns
+//    a few output rows; wavefront w owns the 1 KiB K-chunks c with c % 4 == w,
+//    so the four wavefronts read 4 KiB of one row contiguously.  The activation
+//    slice a wavefront needs is converted to fp32 once and stays in registers
+//    for all rows.  Per row a lane issues 16-byte weight loads, converts two
+//    bytes per instruction, accumulates in fp32 per 128-wide scale block, and
+//    the row sum is a wavefront reduction followed by a 4-way LDS combine.
+//  * 2 <= M <= 16 (skinny_mfma_kernel): the activation rows are the 16-wide N
+//    side of v_mfma_f32_16x16x32_bf16 (e4m3 -> bf16 is exact), the weight rows
+//    the M side; K is split across workgroups, partial sums go to a workspace
+//    and the last workgroup to finish a row tile adds them in a fixed order.
+//  * anything else (odd K, misaligned rows): rowwise_kernel, one wavefront per
+//    output row, scalar byte loads.
+
+#include "common.h"
+
+namespace cm {
+namespace {
+
+struct VecmatParams {
+  const void* x;
+  const float* scale_x;
+  const unsigned char* w;
+  const float* scale_w;
+  void* out;
+  float* partial;          // [splits][M][N] fp32 (skinny kernel)
+  unsigned* counters;      // [row tiles]       (skinny kernel)
+  int m, n, k;
+  int x_dtype, out_dtype;
+  int srow_shift;          // scale row index = n >> srow_shift
+  int srow_stride;         // floats between scale rows
+  int scol_stride;         // floats between 128-wide K blocks (0 or 1)
+  int rows_per_wg;
+  int k_splits;
+};
+
+__device__ __forceinline__ float wscale(const VecmatParams& p, int n, int kb) {
+  return p.scale_w[(size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)kb * p.scol_stride];
+}
+
+// 16 consecutive activation values starting at element k -> fp32
+__device__ __forceinline__ void load_x16(const VecmatParams& p, size_t off, float (&o)[16]) {
+  if (p.x_dtype == CPPMEGA_MI355_F32) {
+    const float4* s = reinterpret_cast<const float4*>((const float*)p.x + off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { const float4 t = s[i]; o[4*i] = t.x; o[4*i+1] = t.y; o[4*i+2] = t.z; o[4*i+3] = t.w; }
+  } else if (p.x_dtype == CPPMEGA_MI355_E4M3) {
+    const uint4 t = *reinterpret_cast<const uint4*>((const unsigned char*)p.x + off);
+    const unsigned wds[4] = {t.x, t.y, t.z, t.w};
+    const float sx = p.scale_x ? p.scale_x[0] : 1.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x2 lo = e4m3x2_lo(wds[i]), hi = e4m3x2_hi(wds[i]);
+      o[4*i] = lo[0] * sx; o[4*i+1] = lo[1] * sx; o[4*i+2] = hi[0] * sx; o[4*i+3] = hi[1] * sx;
+    }
+  } else {
+    const uint4* s = reinterpret_cast<const uint4*>((const unsigned short*)p.x + off);
+    const bool bf = p.x_dtype == CPPMEGA_MI355_BF16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint4 t = s[h];
+      const unsigned wds[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const unsigned short a = (unsigned short)(wds[i] & 0xffffu), b = (unsigned short)(wds[i] >> 16);
+        o[8*h + 2*i] = bf ? bf16_bits_to_f32(a) : f16_bits_to_f32(a);
+        o[8*h + 2*i + 1] = bf ? bf16_bits_to_f32(b) : f16_bits_to_f32(b);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ float dot16(const uint4 wv, const float (&x)[16]) {
+  const unsigned wds[4] = {wv.x, wv.y, wv.z, wv.w};
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f32x2 lo = e4m3x2_lo(wds[i]), hi = e4m3x2_hi(wds[i]);
+    s = fmaf(lo[0], x[4*i], s);
+    s = fmaf(lo[1], x[4*i+1], s);
+    s = fmaf(hi[0], x[4*i+2], s);
+    s = fmaf(hi[1], x[4*i+3], s);
+  }
+  return s;
+}
+
+constexpr int kGemvWaves = 4;
+constexpr int kChunk = 1024;        // bytes of one row a wavefront reads per load instruction
+constexpr int kRowUnroll = 4;
+constexpr int kMaxRowsPerWg = 32;
+
+// M == 1.  CH = 1 KiB chunks per wavefront per pass over K.
+template <int CH>
+__global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const VecmatParams p) {
+  __shared__ float red[kGemvWaves][kMaxRowsPerWg];
+  const int lane = lane_id();
+  const int wave = (int)(threadIdx.x >> 6);
+  const int K = p.k;
+  const int row0 = (int)blockIdx.x * p.rows_per_wg;
+  const int nrows = min(p.rows_per_wg, p.n - row0);
+
+  float acc[kMaxRowsPerWg / kRowUnroll][kRowUnroll];
+#pragma unroll
+  for (int i = 0; i < kMaxRowsPerWg / kRowUnroll; ++i)
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) acc[i][u] = 0.0f;
+
+  for (int kpass = 0; kpass < K; kpass += kGemvWaves * CH * kChunk) {
+    float xr[CH][16];
+    int koff[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      koff[c] = kpass + (c * kGemvWaves + wave) * kChunk + lane * 16;
+      if (koff[c] < K) {
+        load_x16(p, (size_t)koff[c], xr[c]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xr[c][i] = 0.0f;
+      }
+    }
+#pragma unroll
+    for (int rg = 0; rg < kMaxRowsPerWg / kRowUnroll; ++rg) {
+      if (rg * kRowUnroll < nrows) {
+        uint4 wv[kRowUnroll][CH];
+        float sc[kRowUnroll][CH];
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+          const int n = row0 + min(rg * kRowUnroll + u, nrows - 1);
+          const unsigned char* wrow = p.w + (size_t)n * K;
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            if (koff[c] < K) {
+              wv[u][c] = *reinterpret_cast<const uint4*>(wrow + koff[c]);
+              sc[u][c] = wscale(p, n, koff[c] >> 7);
+            } else {
+              wv[u][c] = make_uint4(0, 0, 0, 0);
+              sc[u][c] = 0.0f;
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u)
+#pragma unroll
+          for (int c = 0; c < CH; ++c) acc[rg][u] = fmaf(sc[u][c], dot16(wv[u][c], xr[c]), acc[rg][u]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int rg = 0; rg < kMaxRowsPerWg / kRowUnroll; ++rg)
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const float s = wave_sum(acc[rg][u]);
+      if (lane == 0) red[wave][rg * kRowUnroll + u] = s;
+    }
+  __syncthreads();
+  if ((int)threadIdx.x < nrows) {
+    const int r = (int)threadIdx.x;
+    const float s = ((red[0][r] + red[1][r]) + red[2][r]) + red[3][r];
+    store_as(p.out, (size_t)(row0 + r), p.out_dtype, s);
+  }
+}
+
+// Any shape: one wavefront per output row, all M activations in turn.
+__global__ __launch_bounds__(256) void rowwise_kernel(const VecmatParams p) {
+  const int lane = lane_id();
+  const int n = (int)(blockIdx.x * 4 + (threadIdx.x >> 6));
+  if (n >= p.n) return;
+  const unsigned char* wrow = p.w + (size_t)n * p.k;
+  const float sx = (p.x_dtype == CPPMEGA_MI355_E4M3 && p.scale_x) ? p.scale_x[0] : 1.0f;
+  for (int m = 0; m < p.m; ++m) {
+    float acc = 0.0f;
+    for (int k = lane; k < p.k; k += 64) {
+      const float wv = e4m3_to_f32(wrow[k]) * wscale(p, n, k >> 7);
+      acc = fmaf(wv, load_as(p.x, (size_t)m * p.k + k, p.x_dtype) * sx, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) store_as(p.out, (size_t)m * p.n + n, p.out_dtype, acc);
+  }
+}
+
+}  // namespace
+
+static int fill_scale_layout(const cppmega_mi355_vecmat_args_t& a, VecmatParams& p) {
+  const int kb = (a.k + 127) / 128;
+  switch (a.scale_w_kind) {
+    case CPPMEGA_MI355_WSCALE_SCALAR: p.srow_shift = 0; p.srow_stride = 0; p.scol_stride = 0; return 0;
+    case CPPMEGA_MI355_WSCALE_PER_ROW: p.srow_shift = 0; p.srow_stride = 1; p.scol_stride = 0; return 0;
+    case CPPMEGA_MI355_WSCALE_ROW_BLOCK: p.srow_shift = 0; p.srow_stride = kb; p.scol_stride = 1; return 0;
+    case CPPMEGA_MI355_WSCALE_GRID_128: p.srow_shift = 7; p.srow_stride = kb; p.scol_stride = 1; return 0;
+    default: return fail(CPPMEGA_MI355_ERR_SHAPE, "vecmat: unknown scale_w_kind %d", a.scale_w_kind);
+  }
+}
+
+static int validate(const cppmega_mi355_vecmat_args_t& a) {
+  if (!a.x || !a.w || !a.scale_w || !a.out) return fail(CPPMEGA_MI355_ERR_NULL, "vecmat: x/w/scale_w/out is NULL");
+  if (a.m < 1 || a.n < 1 || a.k < 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "vecmat: M=%d N=%d K=%d", a.m, a.n, a.k);
+  if (a.x_dtype != CPPMEGA_MI355_F32 && a.x_dtype != CPPMEGA_MI355_F16 && a.x_dtype != CPPMEGA_MI355_BF16 &&
+      a.x_dtype != CPPMEGA_MI355_E4M3)
+    return fail(CPPMEGA_MI355_ERR_DTYPE, "vecmat: x dtype %d", a.x_dtype);
+  if (a.x_dtype == CPPMEGA_MI355_E4M3 && !a.scale_x)
+    return fail(CPPMEGA_MI355_ERR_NULL, "vecmat: e4m3 activation needs scale_x");
+  if (a.out_dtype != CPPMEGA_MI355_F32 && a.out_dtype != CPPMEGA_MI355_F16 && a.out_dtype != CPPMEGA_MI355_BF16)
+    return fail(CPPMEGA_MI355_ERR_DTYPE, "vecmat: out dtype %d", a.out_dtype);
+  return 0;
+}
+
+int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes) {
+  if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "vecmat: bytes is NULL");
+  *bytes = 0;
+  return 0;
+}
+
+int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) {
+  int rc = validate(a);
+  if (rc) return rc;
+  VecmatParams p;
+  p.x = a.x; p.scale_x = a.scale_x; p.w = a.w; p.scale_w = a.scale_w; p.out = a.out;
+  p.partial = nullptr; p.counters = nullptr;
+  p.m = a.m; p.n = a.n; p.k = a.k; p.x_dtype = a.x_dtype; p.out_dtype = a.out_dtype;
+  p.rows_per_wg = 0; p.k_splits = 1;
+  rc = fill_scale_layout(a, p);
+  if (rc) return rc;
+
+  const size_t xelt = (size_t)dtype_size(a.x_dtype);
+  const bool aligned = (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) &&
+                       (((size_t)a.k * xelt) % 16 == 0);
+  if (a.m == 1 && aligned) {
+    // rows per workgroup: keep at least ~3 workgroups per CU in the grid
+    int rows = 16;
+    while (rows > 4 && (a.n + rows - 1) / rows < 768) rows >>= 1;
+    p.rows_per_wg = rows;
+    const dim3 grid((unsigned)((a.n + rows - 1) / rows)), block(kGemvWaves * 64);
+    const int chunks = (a.k + kChunk - 1) / kChunk;
+    if (chunks <= kGemvWaves) hipLaunchKernelGGL(gemv_kernel<1>, grid, block, 0, stream, p);
+    else if (chunks <= 2 * kGemvWaves) hipLaunchKernelGGL(gemv_kernel<2>, grid, block, 0, stream, p);
+    else hipLaunchKernelGGL(gemv_kernel<4>, grid, block, 0, stream, p);
+  } else {
+    const dim3 grid((unsigned)((a.n + 3) / 4)), block(256);
+    hipLaunchKernelGGL(rowwise_kernel, grid, block, 0, stream, p);
+  }
+  CM_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+}  // namespace cm

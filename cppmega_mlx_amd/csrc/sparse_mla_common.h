@@ -1,0 +1,52 @@
+// Parameter block shared by the sparse-MLA kernels.
+#pragma once
+
+#include "common.h"
+
+namespace cm {
+
+struct MlaParams {
+  const void* q;
+  const void* q_scale;
+  const void* kv;
+  const void* kv_scale;
+  const void* rope;
+  const void* indices;
+  const float* sinks;
+  void* out;
+  float* lse;
+  void* workspace;
+  int q_dtype, q_scale_kind, q_scale_block;
+  int kv_dtype, kv_scale_kind, kv_scale_block;
+  int rope_dtype, rope_dim;
+  int index_dtype, out_dtype;
+  int B, S, H, G, Skv, topk;
+  int d_qk, d_kv, d_v;
+  int heads_per_group;
+  int num_splits;       // split-KV factor of the MFMA kernel
+  int keys_per_split;
+  float sm_scale;
+};
+
+__device__ __forceinline__ long long load_index(const MlaParams& p, size_t i) {
+  return p.index_dtype == CPPMEGA_MI355_I64 ? ((const long long*)p.indices)[i]
+                                            : (long long)((const int*)p.indices)[i];
+}
+
+// scale of element block `blk` of row `row` (row = flattened leading index)
+__device__ __forceinline__ float row_scale(const void* scale, int kind, size_t row, int nblk, int blk) {
+  switch (kind) {
+    case CPPMEGA_MI355_SCALE_PER_TOKEN: return ((const float*)scale)[row];
+    case CPPMEGA_MI355_SCALE_E8M0: return e8m0_to_f32(((const unsigned char*)scale)[row * nblk + blk]);
+    case CPPMEGA_MI355_SCALE_F32_BLOCK: return ((const float*)scale)[row * nblk + blk];
+    default: return 1.0f;
+  }
+}
+
+int sparse_mla_scalar_launch(const MlaParams& p, hipStream_t stream);
+int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream);
+bool sparse_mla_mfma_supported(const MlaParams& p);
+size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p);
+void sparse_mla_mfma_plan(MlaParams& p);
+
+}  // namespace cm

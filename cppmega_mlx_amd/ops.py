@@ -1,0 +1,261 @@
+"""Host-side launch helpers: torch tensors in, one C-ABI call out.
+
+These functions fill the argument structs of ``include/cppmega_mi355.h`` from
+dense device tensors and enqueue the kernel on torch's current HIP stream.
+They validate what the C side cannot see (tensor ranks, devices, contiguity)
+and leave value/shape contracts to the library, whose status codes come back as
+``ValueError`` / ``TypeError`` / ``NativeCallError``.  Outputs are caller-owned;
+the only tensor this module ever creates is the split-KV / split-K workspace,
+kept per device and reused, unless the caller passes ``workspace=``.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+_ws_lock = threading.Lock()
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int, stream: int) -> torch.Tensor | None:
+    """Per-(device, stream) scratch, grown geometrically, never shrunk."""
+    if nbytes <= 0:
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    with _ws_lock:
+        buf = _workspaces.get(key)
+        if buf is None or buf.numel() < nbytes:
+            size = max(nbytes, 1 << 20)
+            if buf is not None:
+                size = max(size, 2 * buf.numel())
+            buf = torch.zeros(size, dtype=torch.uint8, device=device)
+            _workspaces[key] = buf
+        return buf
+
+
+def _dtype_or_raise(t: torch.Tensor, name: str, allowed: tuple[int, ...]) -> int:
+    code = _lib.dtype_code(t)
+    if code is None or code not in allowed:
+        raise TypeError(f"{name}: unsupported dtype {t.dtype}")
+    return code
+
+
+# ---------------------------------------------------------------------------
+# top-k
+# ---------------------------------------------------------------------------
+
+def topk_select(
+    scores: torch.Tensor,
+    k: int,
+    *,
+    out: torch.Tensor,
+    starts: torch.Tensor | None = None,
+    ends: torch.Tensor | None = None,
+    order: str = "index",
+    neg_inf_is_masked: bool = False,
+) -> torch.Tensor:
+    """Write the per-row top-k indices of ``scores`` (rows, width) into ``out`` (rows, k)."""
+    _lib.require_device_tensor(scores, "scores")
+    _lib.require_device_tensor(out, "out", scores)
+    if scores.ndim != 2:
+        raise ValueError(f"topk_selector expects a (B, T) array; got shape {tuple(scores.shape)}")
+    rows, width = scores.shape
+    if out.dtype != torch.int32:
+        raise ValueError(f"topk_selector: out dtype must be torch.int32; got {out.dtype}")
+    if tuple(out.shape) != (rows, int(k)):
+        raise ValueError(f"topk_selector: out shape must be ({rows}, {int(k)}); got {tuple(out.shape)}")
+    if order not in ("index", "value"):
+        raise ValueError(f"unknown order {order!r}")
+    for name, bound in (("starts", starts), ("ends", ends)):
+        if bound is None:
+            continue
+        _lib.require_device_tensor(bound, name, scores)
+        if tuple(bound.shape) != (rows,) or bound.dtype != torch.int32:
+            raise ValueError(f"starts/ends must be int32 with shape ({rows},); got {name}={tuple(bound.shape)} {bound.dtype}")
+    args = _lib.TopkArgs()
+    args.struct_size = C.sizeof(args)
+    args.score_dtype = _dtype_or_raise(scores, "scores", (_lib.F32, _lib.F16, _lib.BF16))
+    args.scores = scores.data_ptr()
+    args.row_stride = width
+    args.rows, args.width, args.k = rows, width, int(k)
+    args.order = _lib.TOPK_ORDER_VALUE if order == "value" else _lib.TOPK_ORDER_INDEX
+    args.starts = _lib.ptr(starts)
+    args.ends = _lib.ptr(ends)
+    args.indices = out.data_ptr()
+    args.neg_inf_is_masked = 1 if neg_inf_is_masked else 0
+    lib = _lib.load()
+    with torch.cuda.device(scores.device):
+        rc = lib.cppmega_mi355_topk_select(C.byref(args), C.sizeof(args), _lib.current_stream(scores.device))
+    _lib.check(rc, "topk_select")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# sparse MLA
+# ---------------------------------------------------------------------------
+
+@dataclass
+class QuantSpec:
+    """How one operand of the attention is stored."""
+
+    kind: int = _lib.SCALE_NONE
+    scale: torch.Tensor | None = None
+    block: int = 0
+
+
+_KERNELS = {"auto": _lib.MLA_KERNEL_AUTO, "scalar": _lib.MLA_KERNEL_SCALAR, "mfma": _lib.MLA_KERNEL_MFMA}
+
+
+def _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel):
+    B, S, H, d_qk = q.shape
+    _, Skv, G, d_kv = kv.shape
+    rope_dim = 0 if kv_rope is None else kv_rope.shape[-1]
+    a = _lib.SparseMlaArgs()
+    a.struct_size = C.sizeof(a)
+    a.kernel = _KERNELS[kernel]
+    a.q = q.data_ptr()
+    a.q_scale = _lib.ptr(q_spec.scale)
+    a.q_dtype = _dtype_or_raise(q, "q", (_lib.F32, _lib.F16, _lib.BF16, _lib.E4M3))
+    a.q_scale_kind, a.q_scale_block = q_spec.kind, q_spec.block
+    a.kv = kv.data_ptr()
+    a.kv_scale = _lib.ptr(kv_spec.scale)
+    a.kv_dtype = _dtype_or_raise(kv, "kv", (_lib.F32, _lib.F16, _lib.BF16, _lib.E4M3))
+    a.kv_scale_kind, a.kv_scale_block = kv_spec.kind, kv_spec.block
+    a.kv_rope = _lib.ptr(kv_rope)
+    a.rope_dtype = _dtype_or_raise(kv_rope, "kv_rope", (_lib.F32, _lib.F16, _lib.BF16)) if kv_rope is not None else 0
+    a.rope_dim = rope_dim
+    a.indices = indices.data_ptr()
+    a.index_dtype = _dtype_or_raise(indices, "indices", (_lib.I32, _lib.I64))
+    a.batch, a.seq_q, a.heads, a.kv_groups, a.seq_kv, a.topk = B, S, H, G, Skv, indices.shape[-1]
+    a.d_qk, a.d_v = d_qk, int(d_v)
+    a.sm_scale = float(sm_scale)
+    a.sinks = _lib.ptr(sinks)
+    a.out = _lib.ptr(out)
+    a.lse = _lib.ptr(lse)
+    a.out_dtype = _dtype_or_raise(out, "out", (_lib.F32, _lib.F16, _lib.BF16)) if out is not None else _lib.BF16
+    return a
+
+
+def sparse_mla_forward(
+    q: torch.Tensor,
+    kv: torch.Tensor,
+    indices: torch.Tensor,
+    *,
+    sm_scale: float,
+    d_v: int,
+    out: torch.Tensor,
+    lse: torch.Tensor | None = None,
+    q_spec: QuantSpec | None = None,
+    kv_spec: QuantSpec | None = None,
+    kv_rope: torch.Tensor | None = None,
+    sinks: torch.Tensor | None = None,
+    kernel: str = "auto",
+    workspace: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Sparse MLA forward into caller-owned ``out`` [B,S,H,d_v] (and ``lse`` [B,S,H])."""
+    q_spec = q_spec or QuantSpec()
+    kv_spec = kv_spec or QuantSpec()
+    if kernel not in _KERNELS:
+        raise ValueError(f"unknown kernel {kernel!r}")
+    named = [("q", q), ("kv", kv), ("indices", indices), ("out", out), ("lse", lse), ("kv_rope", kv_rope),
+             ("sinks", sinks), ("q_scale", q_spec.scale), ("kv_scale", kv_spec.scale)]
+    for name, t in named:
+        if t is not None:
+            _lib.require_device_tensor(t, name, q if name != "q" else None)
+    if q.ndim != 4 or kv.ndim != 4 or indices.ndim != 4:
+        raise ValueError("sparse_mla: q, kv and indices must be rank 4")
+    B, S, H, _ = q.shape
+    if tuple(out.shape) != (B, S, H, int(d_v)):
+        raise ValueError(f"out must have shape {(B, S, H, int(d_v))}; got {tuple(out.shape)}")
+    if lse is not None and (tuple(lse.shape) != (B, S, H) or lse.dtype != torch.float32):
+        raise ValueError(f"lse must be float32 with shape {(B, S, H)}; got {lse.dtype} {tuple(lse.shape)}")
+    if sinks is not None and (tuple(sinks.shape) != (H,) or sinks.dtype != torch.float32):
+        raise ValueError(f"sinks must be float32 with shape ({H},), got {sinks.dtype} {tuple(sinks.shape)}")
+    a = _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel)
+    lib = _lib.load()
+    need = C.c_size_t(0)
+    _lib.check(lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)), "sparse_mla")
+    stream = _lib.current_stream(q.device)
+    if need.value:
+        if workspace is None:
+            workspace = _workspace(q.device, need.value, stream)
+        else:
+            _lib.require_device_tensor(workspace, "workspace", q)
+        a.workspace = workspace.data_ptr()
+        a.workspace_bytes = workspace.numel() * workspace.element_size()
+    with torch.cuda.device(q.device):
+        rc = lib.cppmega_mi355_sparse_mla_fwd(C.byref(a), C.sizeof(a), stream)
+    _lib.check(rc, "sparse_mla_fwd")
+    return out, lse
+
+
+def sparse_mla_workspace_bytes(q, kv, indices, *, d_v, q_spec=None, kv_spec=None, kv_rope=None, kernel="auto") -> int:
+    a = _fill_mla_args(q, q_spec or QuantSpec(), kv, kv_spec or QuantSpec(), kv_rope, indices, 1.0, d_v, None,
+                       None, None, kernel)
+    need = C.c_size_t(0)
+    _lib.check(_lib.load().cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)),
+               "sparse_mla")
+    return int(need.value)
+
+
+def sparse_mla_selected_kernel(q, kv, indices, *, d_v, q_spec=None, kv_spec=None, kv_rope=None, kernel="auto") -> str:
+    a = _fill_mla_args(q, q_spec or QuantSpec(), kv, kv_spec or QuantSpec(), kv_rope, indices, 1.0, d_v, None,
+                       None, None, kernel)
+    rc = _lib.load().cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a))
+    if rc < 0:
+        _lib.check(-rc, "sparse_mla_select_kernel")
+    return {v: k for k, v in _KERNELS.items()}[rc]
+
+
+# ---------------------------------------------------------------------------
+# FP8 vecmat
+# ---------------------------------------------------------------------------
+
+def fp8_vecmat(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    scale_w: torch.Tensor,
+    *,
+    out: torch.Tensor,
+    scale_x: torch.Tensor | None = None,
+    scale_w_kind: int,
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """out[m, n] = sum_k dec(w[n,k]) * scale_w(n,k) * x[m,k];  x is [M,K] or [K]."""
+    for name, t in (("x", x), ("w", w), ("scale_w", scale_w), ("out", out), ("scale_x", scale_x)):
+        if t is not None:
+            _lib.require_device_tensor(t, name, w if name != "w" else None)
+    if w.ndim != 2:
+        raise ValueError(f"W must be 2D [N, K]; got {tuple(w.shape)}")
+    n, k = w.shape
+    m = 1 if x.ndim == 1 else x.shape[0]
+    a = _lib.VecmatArgs()
+    a.struct_size = C.sizeof(a)
+    a.x_dtype = _dtype_or_raise(x, "x", (_lib.F32, _lib.F16, _lib.BF16, _lib.E4M3))
+    a.x = x.data_ptr()
+    a.scale_x = _lib.ptr(scale_x)
+    a.w = w.data_ptr()
+    a.scale_w = scale_w.data_ptr()
+    a.scale_w_kind = scale_w_kind
+    a.m, a.n, a.k = m, n, k
+    a.out_dtype = _dtype_or_raise(out, "out", (_lib.F32, _lib.F16, _lib.BF16))
+    a.out = out.data_ptr()
+    lib = _lib.load()
+    need = C.c_size_t(0)
+    _lib.check(lib.cppmega_mi355_fp8_vecmat_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)), "fp8_vecmat")
+    stream = _lib.current_stream(w.device)
+    if need.value:
+        if workspace is None:
+            workspace = _workspace(w.device, need.value, stream)
+        a.workspace = workspace.data_ptr()
+        a.workspace_bytes = workspace.numel() * workspace.element_size()
+    with torch.cuda.device(w.device):
+        rc = lib.cppmega_mi355_fp8_vecmat(C.byref(a), C.sizeof(a), stream)
+    _lib.check(rc, "fp8_vecmat")
+    return out

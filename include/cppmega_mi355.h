@@ -1,0 +1,242 @@
+/*
+ * cppmega_mi355.h -- C ABI of the MI355X (gfx950) sparse-attention hot path.
+ *
+ * One shared library, libcppmega_mi355.so, exports the entry points below.
+ * They are what a binding of the reference's kernel boundary would call in
+ * place of the TileLang/TVM-FFI artefacts it compiles today.  Conventions are
+ * taken from the reference's only native C ABI,
+ * cppmega_mlx/nn/_tilelang/native_bridge/tilelang_mlx_tvm_ffi_bridge.h:18-39:
+ *
+ *   - every call takes a pointer to a plain struct plus sizeof(struct); the
+ *     struct starts with `struct_size` so old callers keep working when fields
+ *     are appended;
+ *   - the return value is an int status, 0 = ok (1 = null argument,
+ *     2 = struct too small, as in tilelang_mlx_tvm_ffi_bridge.cpp:33-69);
+ *   - outputs are caller-owned ("owner-output", reference AGENTS.md:3-20):
+ *     the library never allocates, copies or casts a tensor.  The only device
+ *     memory beyond inputs and outputs is an optional caller-provided
+ *     workspace whose size the matching *_workspace_bytes() call reports;
+ *   - all pointers are device pointers unless stated; tensors are dense and
+ *     row-major with the shapes given per field; work is enqueued on `stream`
+ *     (a hipStream_t, passed as void*; NULL = the default stream) and the call
+ *     returns without synchronising.
+ */
+#ifndef CPPMEGA_MI355_H_
+#define CPPMEGA_MI355_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CPPMEGA_MI355_ABI_VERSION 1
+
+/* ---- status codes -------------------------------------------------------- */
+enum {
+  CPPMEGA_MI355_OK = 0,
+  CPPMEGA_MI355_ERR_NULL = 1,          /* a required pointer is NULL            */
+  CPPMEGA_MI355_ERR_STRUCT_SIZE = 2,   /* args_size smaller than this ABI needs  */
+  CPPMEGA_MI355_ERR_SHAPE = 3,         /* shape / value contract -> ValueError   */
+  CPPMEGA_MI355_ERR_DTYPE = 4,         /* unsupported dtype combo -> TypeError   */
+  CPPMEGA_MI355_ERR_UNSUPPORTED = 5,   /* valid request, no kernel for it        */
+  CPPMEGA_MI355_ERR_WORKSPACE = 6,     /* workspace missing or too small         */
+  CPPMEGA_MI355_ERR_LAUNCH = 7,        /* HIP reported a launch/runtime error    */
+  CPPMEGA_MI355_ERR_ALIGNMENT = 8      /* pointer or stride misaligned           */
+};
+
+/* ---- element types ------------------------------------------------------- */
+enum {
+  CPPMEGA_MI355_F32 = 0,
+  CPPMEGA_MI355_F16 = 1,
+  CPPMEGA_MI355_BF16 = 2,
+  CPPMEGA_MI355_E4M3 = 3,   /* OCP e4m3fn bytes (uint8 storage)                */
+  CPPMEGA_MI355_I32 = 4,
+  CPPMEGA_MI355_I64 = 5
+};
+
+/* ---- how a quantised operand is scaled ----------------------------------- */
+enum {
+  CPPMEGA_MI355_SCALE_NONE = 0,       /* float carrier, no scale                */
+  CPPMEGA_MI355_SCALE_PER_TOKEN = 1,  /* float32, one per row     [..rows]      */
+  CPPMEGA_MI355_SCALE_E8M0 = 2,       /* uint8 E8M0, one per `block` elements   */
+  CPPMEGA_MI355_SCALE_F32_BLOCK = 3   /* float32,    one per `block` elements   */
+};
+
+/* Probe: replaces cppmega_tilelang_mlx_tvm_ffi_bridge_probe
+ * (native_bridge/tilelang_mlx_tvm_ffi_bridge.h:18-39).  Host memory. */
+typedef struct cppmega_mi355_status {
+  uint32_t struct_size;
+  int32_t abi_version;
+  int32_t device_count;       /* HIP devices visible, 0 when none            */
+  int32_t gfx950_devices;     /* how many of them report gcnArchName gfx950  */
+  char built_for[32];         /* offload arch the kernels were compiled for  */
+  char message[160];
+} cppmega_mi355_status_t;
+
+int cppmega_mi355_status(cppmega_mi355_status_t* out, size_t out_size);
+
+/* Static text for a status code (host memory, never NULL). */
+const char* cppmega_mi355_error_string(int code);
+
+/* After a non-zero return: detail of the last failure on the calling thread. */
+const char* cppmega_mi355_last_error(void);
+
+/* ---- top-k selector --------------------------------------------------------
+ * Replaces the kernel compiled by _path_c_tvm_ffi_kernel_for and called as
+ * kernel(ends, indices, scores, starts)
+ * (cppmega_mlx/nn/_tilelang/topk_selector.py:522-629, 655-674, 771), and the
+ * masked rows that path sends to topk_selector_reference (:227-330, 728-733).
+ *
+ * Per row: the k largest of scores[row, clip(start) .. clip(end)), ties
+ * toward the lower index; slots past the number of selectable positions hold
+ * -1.  NaN scores are never selected.
+ */
+enum { CPPMEGA_MI355_TOPK_ORDER_INDEX = 0, CPPMEGA_MI355_TOPK_ORDER_VALUE = 1 };
+
+typedef struct cppmega_mi355_topk_args {
+  uint32_t struct_size;
+  int32_t score_dtype;        /* F32, F16 or BF16                              */
+  const void* scores;         /* [rows, width], row pitch = row_stride elems   */
+  int64_t row_stride;
+  int32_t rows;
+  int32_t width;
+  int32_t k;                  /* 1 <= k <= width                               */
+  int32_t order;              /* ORDER_INDEX: ascending index; ORDER_VALUE:
+                                 value descending, lower index first           */
+  const int32_t* starts;      /* [rows] or NULL (= 0)                          */
+  const int32_t* ends;        /* [rows] or NULL (= width)                      */
+  int32_t* indices;           /* out [rows, k], dense                          */
+  int32_t neg_inf_is_masked;  /* non-zero: an in-range -inf is unselectable    */
+  int32_t reserved;
+} cppmega_mi355_topk_args_t;
+
+int cppmega_mi355_topk_select(const cppmega_mi355_topk_args_t* args, size_t args_size, void* stream);
+
+/* ---- sparse MLA forward ----------------------------------------------------
+ * One entry point for the three prepared-buffer kernels of the reference and
+ * the float-carrier one:
+ *   blockscaled_sparse_mla_apply_kernel  (q_fp8,q_scale,kv_fp8,kv_scale,indices,
+ *       sm_scale_buf,out,lse)  sparse_mla_blockscaled_path_c.py:1054-1164
+ *   fp8_sparse_mla_apply_kernel (.., sinks, has_sinks, out, lse)
+ *       sparse_mla_fp8_path_c.py:1821-1956
+ *   sparse_mla_fwd_direct (indices,kv,lse,out,q,sm_scale_buf)
+ *       sparse_mla_path_c.py:2291-2382
+ * and for the pure-MLX fallback they are checked against
+ * (cppmega_mlx/nn/sparse_mla.py:125-210).
+ *
+ *   q        [B, S, H, d_qk]
+ *   kv       [B, Skv, G, d_kv]      d_kv = d_qk - rope_dim
+ *   kv_rope  [B, Skv, G, rope_dim]  optional tail of every key row (QK only)
+ *   indices  [B, S, G, topk]        entry < 0 or >= Skv is skipped
+ *   out      [B, S, H, d_v]         d_v <= d_kv: V = first d_v channels of kv
+ *   lse      [B, S, H] float32, natural log, includes sm_scale; 0 for a row
+ *            with nothing to attend to.  May be NULL.
+ *   sinks    [H] float32 or NULL: one extra logit per head that joins the
+ *            max and the denominator and carries no value row.
+ * Scales: *_scale_kind says how q / kv bytes are scaled; per-token scales are
+ * [B,S,H] / [B,Skv,G]; block scales are [.., d/block].
+ */
+enum {
+  CPPMEGA_MI355_MLA_KERNEL_AUTO = 0,
+  CPPMEGA_MI355_MLA_KERNEL_SCALAR = 1,   /* one wavefront per (b,s,h), fp32 VALU */
+  CPPMEGA_MI355_MLA_KERNEL_MFMA = 2      /* head-batched bf16 MFMA, split-KV     */
+};
+
+typedef struct cppmega_mi355_sparse_mla_args {
+  uint32_t struct_size;
+  int32_t kernel;             /* CPPMEGA_MI355_MLA_KERNEL_*                    */
+
+  const void* q;
+  const void* q_scale;        /* NULL when q_scale_kind == SCALE_NONE          */
+  int32_t q_dtype;            /* F32/F16/BF16/E4M3                             */
+  int32_t q_scale_kind;
+  int32_t q_scale_block;      /* elements per scale for the block kinds        */
+
+  int32_t kv_dtype;
+  const void* kv;
+  const void* kv_scale;
+  int32_t kv_scale_kind;
+  int32_t kv_scale_block;
+
+  const void* kv_rope;        /* NULL when rope_dim == 0                       */
+  int32_t rope_dtype;         /* F32/F16/BF16                                  */
+  int32_t rope_dim;
+
+  const void* indices;
+  int32_t index_dtype;        /* I32 or I64                                    */
+
+  int32_t batch, seq_q, heads, kv_groups, seq_kv, topk;
+  int32_t d_qk;               /* width of a q row                              */
+  int32_t d_v;
+  float sm_scale;
+
+  const float* sinks;
+  void* out;
+  float* lse;
+  int32_t out_dtype;          /* F32/F16/BF16                                  */
+  int32_t reserved;
+
+  void* workspace;            /* split-KV partials; see *_workspace_bytes      */
+  size_t workspace_bytes;
+} cppmega_mi355_sparse_mla_args_t;
+
+/* Bytes of workspace cppmega_mi355_sparse_mla_fwd needs for these shapes with
+ * the kernel it would pick (0 when none).  Only the shape / dtype / kernel
+ * fields are read.  Returns a status code; the size goes to *bytes. */
+int cppmega_mi355_sparse_mla_workspace_bytes(const cppmega_mi355_sparse_mla_args_t* args,
+                                             size_t args_size, size_t* bytes);
+
+int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size,
+                                 void* stream);
+
+/* Which kernel AUTO resolves to for these shapes (CPPMEGA_MI355_MLA_KERNEL_*),
+ * or a negative status code. */
+int cppmega_mi355_sparse_mla_select_kernel(const cppmega_mi355_sparse_mla_args_t* args,
+                                           size_t args_size);
+
+/* ---- FP8 vecmat / skinny GEMM ----------------------------------------------
+ * Replaces fp8_vecmat_reduce_direct, called as kernel(A, A_scale, B, B_scale, C)
+ * (cppmega_mlx/nn/_tilelang/fp8_vecmat_path_c.py:737-821, 1039-1046) and the
+ * inline kernel of fused_fp8_gemm (cppmega_v4/_tilelang/fused_fp8_gemm.py:83-142).
+ *
+ *   out[m, n] = sum_k dec(w[n, k]) * w_scale(n, k) * x(m, k)     fp32 accumulate
+ *   w        [N, K] e4m3 bytes ("already transposed" weight)
+ *   x        [M, K]: E4M3 bytes with one float32 scale_x (x(m,k) =
+ *            dec(x)*scale_x[0]), or F32/F16/BF16 with scale_x == NULL
+ *   out      [M, N] F32/F16/BF16
+ */
+enum {
+  CPPMEGA_MI355_WSCALE_SCALAR = 0,     /* float32 [1]                           */
+  CPPMEGA_MI355_WSCALE_PER_ROW = 1,    /* float32 [N]                           */
+  CPPMEGA_MI355_WSCALE_ROW_BLOCK = 2,  /* float32 [N, ceil(K/128)]              */
+  CPPMEGA_MI355_WSCALE_GRID_128 = 3    /* float32 [ceil(N/128), ceil(K/128)]    */
+};
+
+typedef struct cppmega_mi355_vecmat_args {
+  uint32_t struct_size;
+  int32_t x_dtype;
+  const void* x;
+  const float* scale_x;
+  const uint8_t* w;
+  const float* scale_w;
+  int32_t scale_w_kind;
+  int32_t m, n, k;
+  int32_t out_dtype;
+  int32_t reserved;
+  void* out;
+  void* workspace;            /* split-K partials for 2 <= M; may be NULL when
+                                 *_workspace_bytes reports 0                   */
+  size_t workspace_bytes;
+} cppmega_mi355_vecmat_args_t;
+
+int cppmega_mi355_fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t* args,
+                                             size_t args_size, size_t* bytes);
+
+int cppmega_mi355_fp8_vecmat(const cppmega_mi355_vecmat_args_t* args, size_t args_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CPPMEGA_MI355_H_ */

@@ -1,0 +1,29 @@
+"""CPU oracle for the sparse-attention hot path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the shipped package may import this directory: only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` use it,
+and only as the checker.  Every function restates, in NumPy, one function of the
+reference's pure-MLX fallback and cites the reference file:line it follows.
+
+Pinning status (what fixes each function besides its own formula):
+
+* ``fp8.e4m3_decode``            -- closed-form bit spec; pinned against the
+  reference's edge-byte known answers and against torch's independent
+  ``float8_e4m3fn`` decoder for all 254 non-NaN bytes.
+* ``fp8.e8m0_decode``            -- pinned against the reference-held table
+  rule (byte 0 or 255 -> 0, else 2**(b-127)).
+* ``fp8.e4m3_encode``, ``fp8.quantize_*`` -- producer side (input generation
+  only).  The reference delegates to MLX ``mx.to_fp8`` / ``mx.quantize`` whose
+  source is not in the tree: **parity unpinned** for the quantiser's rounding;
+  kernels consume prepared bytes + scales, so no kernel result depends on it.
+  Mathematically pinned here by round-trip exactness on the e4m3 grid and by
+  nearest-value brute force.
+* ``topk.topk_selector_oracle``  -- pinned by the reference tests' exact-order
+  known answers, sentinel cases and an O(T^2) brute-force ranker.
+* ``sparse_mla.sparse_mla_oracle`` -- pinned against a per-token loop
+  formulation, ``torch.softmax`` / ``torch.logsumexp`` closed forms and the
+  invariants the reference tests pin (all-invalid row -> zeros, duplicated
+  index = doubled weight, permutation invariance).
+* ``vecmat.*``                   -- pinned against float64 ``W_deq @ x`` with
+  torch's independent e4m3 decoder.
+"""
