@@ -1,0 +1,158 @@
+"""Per-token-scaled FP8 sparse-MLA forward over prepared buffers, with sinks.
+
+Surface of the reference's ``cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py``:
+``sparse_mla_fp8_path_c_apply_direct`` :2756-2869 and
+``sparse_mla_fp8_path_c_apply`` :2872-3004 with the kernel contract of
+:1821-1956: ``q_scale`` float32 ``[B,S,H]``, ``kv_scale`` float32 ``[B,Skv,G]``,
+score = (sum dec*dec) * qs * ks * sm_scale, optional attention ``sinks`` ``[H]``
+(one extra logit per head in the max and the denominator, no value row),
+``out`` float32/float16/bfloat16 (``output_dtype``), ``lse`` float32.
+
+A float32 ``kv_scale`` of rank 4 selects the block-128 latent layout described
+in ``sparse_mla_blockscaled_path_c`` (per-token is its one-block case), so the
+sink path is available for the latent KV cache as well.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from ... import _lib
+from . import _prepared
+
+__all__ = [
+    "SparseMLAFp8PathCDirectError",
+    "SparseMLAFp8PathCStatus",
+    "sparse_mla_fp8_path_c_apply",
+    "sparse_mla_fp8_path_c_apply_direct",
+    "sparse_mla_fp8_path_c_status",
+]
+
+_OP = "FP8 Sparse-MLA Path C apply"
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+class SparseMLAFp8PathCDirectError(RuntimeError):
+    """Raised when the prepared-buffer owner-output path cannot run."""
+
+
+@dataclass(frozen=True)
+class SparseMLAFp8PathCStatus:
+    available: bool
+    reason: str
+    target: str = "hip-gfx950"
+
+
+def sparse_mla_fp8_path_c_status() -> SparseMLAFp8PathCStatus:
+    try:
+        st = _lib.status()
+    except _lib.NativeLibraryError as exc:
+        return SparseMLAFp8PathCStatus(False, str(exc))
+    if st["gfx950_devices"] < 1:
+        return SparseMLAFp8PathCStatus(False, st["message"])
+    return SparseMLAFp8PathCStatus(True, "FP8 sparse-MLA HIP kernels (gfx950) are available")
+
+
+def _float_dtype(dtype, *, name: str = "dtype"):
+    if dtype not in _FLOATS:
+        raise TypeError(f"{name} must be float32, float16, or bfloat16; got {dtype}")
+    return dtype
+
+
+def _check_sinks(sinks, heads: int):
+    if sinks is None:
+        return None
+    if not isinstance(sinks, torch.Tensor):
+        raise TypeError("sinks must be a torch.Tensor")
+    if tuple(sinks.shape) != (heads,):
+        raise ValueError(f"sinks must have shape ({heads},), got {tuple(sinks.shape)}")
+    if sinks.dtype != torch.float32:
+        raise ValueError("sinks must be float32")
+    return sinks
+
+
+def sparse_mla_fp8_path_c_apply_direct(
+    q_fp8: torch.Tensor,
+    q_scale: torch.Tensor | None,
+    kv_fp8: torch.Tensor,
+    kv_scale: torch.Tensor,
+    indices: torch.Tensor,
+    *,
+    sm_scale: float,
+    out: torch.Tensor,
+    lse: torch.Tensor,
+    d_v: int | None = None,
+    sinks: torch.Tensor | None = None,
+    output_dtype: torch.dtype | None = None,
+    kv_rope: torch.Tensor | None = None,
+    kernel: str = "auto",
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Forward into caller-owned ``out``/``lse``; returns those same objects."""
+    status = sparse_mla_fp8_path_c_status()
+    if not status.available:
+        raise SparseMLAFp8PathCDirectError(status.reason)
+    plan = _prepared.plan_prepared(q_fp8, q_scale, kv_fp8, kv_scale, indices, d_v=d_v, kv_rope=kv_rope,
+                                   op_name=_OP, family="fp8")
+    want = _float_dtype(out.dtype if output_dtype is None else output_dtype, name="output_dtype") \
+        if isinstance(out, torch.Tensor) else None
+    _prepared.validate_owner_outputs(out, lse, plan, out_dtype=want)
+    sinks = _check_sinks(sinks, plan.heads)
+    try:
+        _prepared.launch_prepared(q_fp8, kv_fp8, indices, plan, sm_scale=sm_scale, out=out, lse=lse,
+                                  kv_rope=kv_rope, sinks=sinks, kernel=kernel)
+    except (_lib.NativeCallError, _lib.NativeLibraryError) as exc:
+        raise SparseMLAFp8PathCDirectError(
+            f"FP8 Sparse-MLA forward dispatch failed: {type(exc).__name__}: {exc}"
+        ) from exc
+    return out, lse
+
+
+def sparse_mla_fp8_path_c_apply(
+    q_fp8: torch.Tensor,
+    q_scale: torch.Tensor | None,
+    kv_fp8: torch.Tensor,
+    kv_scale: torch.Tensor,
+    indices: torch.Tensor,
+    *,
+    sm_scale: float,
+    d_v: int | None = None,
+    sinks: torch.Tensor | None = None,
+    return_lse: bool = False,
+    force_path_c: bool = False,
+    out: torch.Tensor | None = None,
+    lse: torch.Tensor | None = None,
+    output_dtype: torch.dtype | None = None,
+    kv_rope: torch.Tensor | None = None,
+    kernel: str = "auto",
+):
+    """Fused FP8 sparse-MLA forward over prepared GPU buffers."""
+    if (out is None) != (lse is None):
+        raise ValueError("sparse_mla_fp8_path_c_apply owner-output route requires both out and lse buffers")
+    if out is not None and lse is not None:
+        direct_out, direct_lse = sparse_mla_fp8_path_c_apply_direct(
+            q_fp8, q_scale, kv_fp8, kv_scale, indices, sm_scale=sm_scale, out=out, lse=lse, d_v=d_v, sinks=sinks,
+            output_dtype=output_dtype, kv_rope=kv_rope, kernel=kernel)
+        return (direct_out, direct_lse) if return_lse else direct_out
+
+    status = sparse_mla_fp8_path_c_status()
+    if not status.available:
+        if force_path_c:
+            raise RuntimeError(f"sparse_mla_fp8_path_c_apply: {status.reason}")
+        return None
+    plan = _prepared.plan_prepared(q_fp8, q_scale, kv_fp8, kv_scale, indices, d_v=d_v, kv_rope=kv_rope,
+                                   op_name=_OP, family="fp8")
+    default = torch.float16 if q_fp8.dtype == torch.uint8 else q_fp8.dtype
+    out_dtype = _float_dtype(default if output_dtype is None else output_dtype, name="output_dtype")
+    sinks = _check_sinks(sinks, plan.heads)
+    out = torch.empty((plan.batch, plan.seq_len, plan.heads, plan.d_v), dtype=out_dtype, device=q_fp8.device)
+    lse = torch.empty((plan.batch, plan.seq_len, plan.heads), dtype=torch.float32, device=q_fp8.device)
+    try:
+        _prepared.launch_prepared(q_fp8, kv_fp8, indices, plan, sm_scale=sm_scale, out=out, lse=lse,
+                                  kv_rope=kv_rope, sinks=sinks, kernel=kernel)
+    except (_lib.NativeCallError, _lib.NativeLibraryError) as exc:
+        raise RuntimeError(
+            f"sparse_mla_fp8_path_c_apply: kernel dispatch failed: {type(exc).__name__}: {exc}"
+        ) from exc
+    return (out, lse) if return_lse else out

@@ -1,0 +1,128 @@
+"""The C-ABI library: loads, exports what the header declares, lays structs out
+as the Python binding expects, and rejects bad calls before touching the GPU."""
+
+import ctypes as C
+import re
+import shutil
+import subprocess
+from pathlib import Path
+
+import pytest
+
+from cppmega_mlx_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "cppmega_mi355.h"
+
+
+def _declared_functions() -> list[str]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(cppmega_mi355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_functions()
+    assert set(declared) == set(_lib.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_status_probe_reports_abi_and_arch():
+    st = _lib.status()
+    assert st["abi_version"] == _lib.ABI_VERSION == 1
+    assert st["built_for"] == "gfx950"
+    assert st["device_count"] >= 0
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="gcc not available")
+def test_struct_layouts_match_the_header(tmp_path):
+    fields = {
+        "cppmega_mi355_topk_args_t": (_lib.TopkArgs, ["scores", "row_stride", "k", "starts", "indices", "neg_inf_is_masked"]),
+        "cppmega_mi355_sparse_mla_args_t": (_lib.SparseMlaArgs, ["q", "kv_dtype", "kv", "kv_rope", "indices", "batch", "d_qk", "sm_scale", "sinks", "out", "lse", "out_dtype", "workspace", "workspace_bytes"]),
+        "cppmega_mi355_vecmat_args_t": (_lib.VecmatArgs, ["x", "scale_w", "scale_w_kind", "k", "out", "workspace_bytes"]),
+        "cppmega_mi355_status_t": (_lib.StatusStruct, ["abi_version", "built_for", "message"]),
+    }
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void){"]
+    for ctype, (_, names) in fields.items():
+        lines.append(f'printf("{ctype} size %zu\\n", sizeof({ctype}));')
+        for n in names:
+            lines.append(f'printf("{ctype} {n} %zu\\n", offsetof({ctype}, {n}));')
+    lines.append("return 0;}")
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    for line in out.strip().splitlines():
+        ctype, name, value = line.split()
+        struct = fields[ctype][0]
+        got = C.sizeof(struct) if name == "size" else getattr(struct, name).offset
+        assert got == int(value), f"{ctype}.{name}: ctypes {got} != C {value}"
+
+
+def test_null_and_short_struct_are_rejected_with_the_bridge_codes():
+    lib = _lib.load()
+    assert lib.cppmega_mi355_status(None, 0) == _lib.ERR_NULL
+    st = _lib.StatusStruct()
+    assert lib.cppmega_mi355_status(C.byref(st), 4) == _lib.ERR_STRUCT_SIZE
+    assert lib.cppmega_mi355_topk_select(None, 0, None) == _lib.ERR_NULL
+    args = _lib.TopkArgs()
+    args.struct_size = 8
+    assert lib.cppmega_mi355_topk_select(C.byref(args), C.sizeof(args), None) == _lib.ERR_STRUCT_SIZE
+    assert lib.cppmega_mi355_fp8_vecmat(None, 0, None) == _lib.ERR_NULL
+    assert lib.cppmega_mi355_sparse_mla_fwd(None, 0, None) == _lib.ERR_NULL
+    assert b"NULL" in lib.cppmega_mi355_error_string(_lib.ERR_NULL)
+
+
+def test_contract_violations_return_shape_and_dtype_codes_without_a_gpu():
+    lib = _lib.load()
+    fake = 0x1000  # never dereferenced: validation fails first
+    t = _lib.TopkArgs()
+    t.struct_size = C.sizeof(t)
+    t.scores, t.indices, t.rows, t.width, t.row_stride, t.k = fake, fake, 2, 16, 16, 17
+    assert lib.cppmega_mi355_topk_select(C.byref(t), C.sizeof(t), None) == _lib.ERR_SHAPE
+    assert b"topk must be in [1, 16]" in lib.cppmega_mi355_last_error()
+    t.k, t.score_dtype = 4, _lib.I32
+    assert lib.cppmega_mi355_topk_select(C.byref(t), C.sizeof(t), None) == _lib.ERR_DTYPE
+    t.score_dtype, t.width, t.row_stride, t.k = _lib.F32, 20000, 20000, 4
+    assert lib.cppmega_mi355_topk_select(C.byref(t), C.sizeof(t), None) == _lib.ERR_UNSUPPORTED
+
+    m = _lib.SparseMlaArgs()
+    m.struct_size = C.sizeof(m)
+    m.q = m.kv = m.indices = m.out = fake
+    m.q_dtype = m.kv_dtype = m.out_dtype = _lib.BF16
+    m.index_dtype = _lib.I32
+    m.batch, m.seq_q, m.heads, m.kv_groups, m.seq_kv, m.topk, m.d_qk, m.d_v = 1, 1, 6, 4, 8, 4, 64, 64
+    assert lib.cppmega_mi355_sparse_mla_fwd(C.byref(m), C.sizeof(m), None) == _lib.ERR_SHAPE
+    assert b"not divisible by kv_group" in lib.cppmega_mi355_last_error()
+    m.kv_groups, m.d_v = 2, 65
+    assert lib.cppmega_mi355_sparse_mla_fwd(C.byref(m), C.sizeof(m), None) == _lib.ERR_SHAPE
+    m.d_v, m.index_dtype = 64, _lib.F32
+    assert lib.cppmega_mi355_sparse_mla_fwd(C.byref(m), C.sizeof(m), None) == _lib.ERR_DTYPE
+
+    v = _lib.VecmatArgs()
+    v.struct_size = C.sizeof(v)
+    v.x = v.w = v.scale_w = v.out = fake
+    v.m, v.n, v.k, v.x_dtype, v.out_dtype = 1, 8, 0, _lib.BF16, _lib.BF16
+    assert lib.cppmega_mi355_fp8_vecmat(C.byref(v), C.sizeof(v), None) == _lib.ERR_SHAPE
+    v.k, v.x_dtype = 16, _lib.E4M3
+    assert lib.cppmega_mi355_fp8_vecmat(C.byref(v), C.sizeof(v), None) == _lib.ERR_NULL  # scale_x missing
+
+
+def test_check_maps_codes_to_python_errors():
+    with pytest.raises(ValueError):
+        _lib.check(_lib.ERR_SHAPE, "op")
+    with pytest.raises(TypeError):
+        _lib.check(_lib.ERR_DTYPE, "op")
+    with pytest.raises(_lib.NativeCallError) as info:
+        _lib.check(_lib.ERR_LAUNCH, "op")
+    assert info.value.code == _lib.ERR_LAUNCH
+    _lib.check(_lib.OK, "op")
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(_lib.NativeLibraryError, match="no fallback"):
+        _lib.load()
