@@ -1,0 +1,378 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode,vecmat,topk,prefill]
+
+Prints ONE JSON line.  The headline (`metric`/`value`) is sparse-MLA decode
+throughput on the B=32, H=128, topk=2048, 64K-token FP8 latent-cache
+configuration; `vecmat` and `topk` carry the two HBM-bound kernels of the same
+path with their own roofline objects, `prefill` the causal prefill
+configuration when asked for.
+
+A "step" is one pass of the kernel(s) over one synthetic batch that is already
+resident in HBM.  Steps are captured into a HIP graph (launch-bound at these
+kernel lengths otherwise) and the K timed steps are one graph replay bracketed
+by HIP events on the launch stream and host synchronisation.  Input sets
+rotate between steps so the HBM-bound kernels cannot be served by the 256 MB
+Infinity Cache.
+
+`cpu_baseline` times the NumPy oracle (a port of the reference's pure-MLX
+fallback, which cannot be installed here) on a bounded sample of the same
+workload on this machine's host cores.  It is a reported baseline only.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+# --------------------------------------------------------------------------- inputs (device side, torch only)
+
+def quantize_block_pow2(x: torch.Tensor, block: int = 128):
+    """x [..., K] fp32 -> (e4m3 bytes [..., K], fp32 scale [..., K/block]), scale = 2^ceil(log2(amax/448))."""
+    shp = x.shape
+    xb = x.reshape(*shp[:-1], shp[-1] // block, block)
+    amax = xb.abs().amax(dim=-1)
+    scale = torch.where(amax > 0, torch.exp2(torch.ceil(torch.log2(amax / 448.0))), torch.ones_like(amax))
+    codes = (xb / scale[..., None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    return codes.reshape(shp).contiguous(), scale.contiguous()
+
+
+def make_latent_cache(gen, B, Skv, device):
+    codes = torch.empty((B, Skv, 1, 512), dtype=torch.uint8, device=device)
+    scale = torch.empty((B, Skv, 1, 4), dtype=torch.float32, device=device)
+    rope = torch.empty((B, Skv, 1, 64), dtype=torch.bfloat16, device=device)
+    for b in range(B):
+        lat = torch.randn((Skv, 1, 512), generator=gen, device=device, dtype=torch.float32)
+        c, s = quantize_block_pow2(lat)
+        codes[b], scale[b] = c, s
+        rope[b] = torch.randn((Skv, 1, 64), generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16)
+    return codes, scale, rope
+
+
+def uniform_indices(gen, B, S, Skv, topk, device):
+    """Uniform without replacement per (b, s): top-k of random keys."""
+    out = torch.empty((B, S, 1, topk), dtype=torch.int32, device=device)
+    for b in range(B):
+        for s0 in range(0, S, 256):
+            s1 = min(S, s0 + 256)
+            r = torch.rand((s1 - s0, Skv), generator=gen, device=device)
+            out[b, s0:s1, 0] = r.topk(topk, dim=-1).indices.to(torch.int32)
+    return out
+
+
+def timed_graph(step_fns, steps: int, warmup: int):
+    """Run `warmup` eager steps, capture `steps` steps into a HIP graph, replay once timed.
+
+    step_fns: list of zero-argument callables (rotated).  Returns (seconds for
+    the K steps by HIP events, seconds by host clock)."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for i in range(max(warmup, 1)):
+            step_fns[i % len(step_fns)]()
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for i in range(steps):
+            step_fns[i % len(step_fns)]()
+    graph.replay()                      # untimed replay: first replay pays upload costs
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return e0.elapsed_time(e1) * 1e-3, t1 - t0
+
+
+# --------------------------------------------------------------------------- workloads
+
+def bench_decode(args, device):
+    from cppmega_mlx_amd import ops
+    from cppmega_mlx_amd.nn._tilelang import sparse_mla_blockscaled_path_c as bs
+
+    B, H, Skv, topk, d_qk, d_v = 32, 128, 65536, 2048, 576, 512
+    gen = torch.Generator(device=device).manual_seed(1234)
+    codes, scale, rope = make_latent_cache(gen, B, Skv, device)
+    n_sets = 3
+    qs = [torch.randn((B, 1, H, d_qk), generator=gen, device=device).to(torch.bfloat16) for _ in range(n_sets)]
+    idxs = [uniform_indices(gen, B, 1, Skv, topk, device) for _ in range(n_sets)]
+    outs = [torch.empty((B, 1, H, d_v), dtype=torch.bfloat16, device=device) for _ in range(n_sets)]
+    lses = [torch.empty((B, 1, H), dtype=torch.float32, device=device) for _ in range(n_sets)]
+    sm_scale = d_qk ** -0.5
+    kernel = ops.sparse_mla_selected_kernel(qs[0], codes, idxs[0], d_v=d_v, kv_rope=rope,
+                                            kv_spec=ops.QuantSpec(3, scale, 128))
+
+    def make(i):
+        return lambda: bs.sparse_mla_blockscaled_path_c_apply_direct(
+            qs[i], None, codes, scale, idxs[i], sm_scale=sm_scale, out=outs[i], lse=lses[i], d_v=d_v, kv_rope=rope)
+
+    steps = args.steps
+    secs, host_secs = timed_graph([make(i) for i in range(n_sets)], steps, args.warmup)
+    flops = 2.0 * B * H * topk * (d_qk + d_v)
+    bytes_alg = B * topk * 656 + B * H * d_qk * 2 + B * H * d_v * 2 + B * topk * 4 + B * H * 4
+    per_step = secs / steps
+    res = {
+        "workload": "sparse_mla_decode B=32 S_q=1 H=128 topk=2048 Skv=65536 latent e4m3[512]+fp32/128 +bf16 rope[64]",
+        "kernel": kernel,
+        "ms_per_step": per_step * 1e3,
+        "host_ms_per_step": host_secs / steps * 1e3,
+        "tflops": flops / per_step / 1e12,
+        "flops_per_step": flops,
+        "algorithmic_bytes_per_step": bytes_alg,
+        "hbm_gbs": bytes_alg / per_step / 1e9,
+    }
+    sample = (qs[0], codes, scale, rope, idxs[0], outs[0], lses[0], sm_scale)
+    return res, sample
+
+
+def cpu_baseline_decode(sample, budget_s: float = 15.0):
+    """Oracle on the first few sequences of the decode batch (compacted to their gathered rows)."""
+    from oracle import fp8, sparse_mla as om
+
+    q, codes, scale, rope, idx, out, lse, sm_scale = sample
+    H, topk = q.shape[2], idx.shape[-1]
+    done, t_total, errs = 0, 0.0, []
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    for b in range(q.shape[0]):
+        ids = idx[b, 0, 0].long()
+        rows = om.dequant_block_latent(codes[b, ids, 0].cpu().numpy(), scale[b, ids, 0].cpu().numpy(),
+                                       rope[b, ids, 0].float().cpu().numpy())[None, :, None, :]
+        qb = q[b:b + 1].float().cpu().numpy()
+        ar = np.arange(topk, dtype=np.int64)[None, None, None, :]
+        t0 = time.perf_counter()
+        want, _ = om.sparse_mla_oracle(qb, rows, ar, sm_scale=sm_scale, d_v=512)
+        t_total += time.perf_counter() - t0
+        got = out[b:b + 1].float().cpu().numpy()
+        errs.append(float(np.abs(got - want).max() / np.abs(want).max()))
+        done += 1
+        if t_total > budget_s or done >= 8:
+            break
+    flops = 2.0 * done * H * topk * (576 + 512)
+    return {
+        "value": flops / t_total / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"NumPy float64 oracle on {done} of 32 sequences (H=128, topk=2048 gathered rows), {t_total:.2f} s",
+    }, max(errs)
+
+
+def bench_vecmat(args, device, M: int):
+    from cppmega_mlx_amd.nn._tilelang import fp8_vecmat_path_c as vm
+
+    N, K = 7168, 16384
+    gen = torch.Generator(device=device).manual_seed(77 + M)
+    n_sets = 3
+    ws, ss = [], []
+    for _ in range(n_sets):
+        w = torch.randn((N, K), generator=gen, device=device, dtype=torch.float32)
+        c, s = quantize_block_pow2(w)
+        ws.append(c)
+        ss.append(s)
+        del w
+    xs = [torch.randn((M, K), generator=gen, device=device).to(torch.bfloat16) for _ in range(n_sets)]
+    outs = [torch.empty((M, N), dtype=torch.bfloat16, device=device) for _ in range(n_sets)]
+
+    def make(i):
+        return lambda: vm.fp8_scaled_vecmat_path_c_direct(xs[i], ws[i], scale_x=None, scale_w=ss[i], out=outs[i])
+
+    steps = max(args.steps, 30)
+    secs, _ = timed_graph([make(i) for i in range(n_sets)], steps, args.warmup)
+    per = secs / steps
+    bytes_alg = N * K + N * (K // 128) * 4 + M * K * 2 + M * N * 2
+    res = {
+        "workload": f"fp8_vecmat W e4m3[7168,16384] + fp32 scale/1x128, x bf16[{M},16384] -> bf16[{M},7168]",
+        "us_per_launch": per * 1e6,
+        "algorithmic_bytes": bytes_alg,
+        "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+    }
+    return res, (xs[0], ws[0], ss[0], outs[0])
+
+
+def cpu_baseline_vecmat(sample, rows: int = 1024):
+    from oracle import vecmat as ov
+
+    x, w, s, out = sample
+    wn, sn, xn = w[:rows].cpu().numpy(), s[:rows].cpu().numpy(), x.float().cpu().numpy()
+    t0 = time.perf_counter()
+    want = ov.fused_fp8_gemm_oracle(wn, sn, xn)
+    dt = time.perf_counter() - t0
+    err = float(np.abs(out[:, :rows].float().cpu().numpy() - want).max() / np.abs(want).max())
+    nbytes = rows * w.shape[1] * (1 + 4 / 128)
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": os.cpu_count() or 1, "kind": "port",
+            "sample": f"NumPy float64 dequant+matmul on the first {rows} of 7168 weight rows, {dt:.2f} s"}, err
+
+
+def bench_topk(args, device):
+    from cppmega_mlx_amd.nn._tilelang import topk_selector as tk
+
+    B, S, T, k = 4, 1024, 8192, 2048
+    gen = torch.Generator(device=device).manual_seed(99)
+    n_sets = 3
+    ends = (T - S + torch.arange(S, device=device, dtype=torch.int32) + 1).repeat(B)
+    col = torch.arange(T, device=device)[None, :]
+    scores, outs = [], []
+    for _ in range(n_sets):
+        s = torch.randn((B * S, T), generator=gen, device=device)
+        n_dup = T // 20
+        dst = torch.randint(0, T, (B * S, n_dup), generator=gen, device=device)
+        src = torch.randint(0, T, (B * S, n_dup), generator=gen, device=device)
+        s.scatter_(1, dst, s.gather(1, src))
+        s.masked_fill_(col >= ends[:, None], float("-inf"))
+        scores.append(s)
+        outs.append(torch.empty((B * S, k), dtype=torch.int32, device=device))
+
+    def make(i):
+        return lambda: tk.topk_selector_tilelang_direct(scores[i], k, out=outs[i], ends=ends, order="index")
+
+    steps = max(args.steps, 30)
+    secs, _ = timed_graph([make(i) for i in range(n_sets)], steps, args.warmup)
+    per = secs / steps
+    bytes_alg = B * S * T * 4 + B * S * k * 4
+    res = {
+        "workload": "topk_selector scores fp32[4,1024,8192] (5% ties, causal bounds) -> int32[4,1024,2048]",
+        "us_per_launch": per * 1e6,
+        "algorithmic_bytes": bytes_alg,
+        "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+    }
+    return res, (scores[0], ends, outs[0], k)
+
+
+def cpu_baseline_topk(sample, rows: int = 512):
+    from oracle import topk as ot
+
+    scores, ends, out, k = sample
+    sn, en = scores[:rows].cpu().numpy(), ends[:rows].cpu().numpy()
+    t0 = time.perf_counter()
+    want = ot.topk_selector_oracle(sn, k, ends=en)
+    dt = time.perf_counter() - t0
+    exact = bool(np.array_equal(out[:rows].cpu().numpy(), want))
+    nbytes = rows * (scores.shape[1] * 4 + k * 4)
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"NumPy stable-argsort oracle on the first {rows} of 4096 rows, {dt:.2f} s"}, exact
+
+
+def bench_prefill(args, device):
+    from cppmega_mlx_amd.nn._tilelang import sparse_mla_blockscaled_path_c as bs, topk_selector as tk
+
+    S, H, topk = 8192, 128, 2048
+    gen = torch.Generator(device=device).manual_seed(555)
+    codes, scale, rope = make_latent_cache(gen, 1, S, device)
+    q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.bfloat16)
+    idx_scores = torch.randn((S, S), generator=gen, device=device)
+    ends = torch.arange(1, S + 1, device=device, dtype=torch.int32)
+    idx = torch.empty((S, topk), dtype=torch.int32, device=device)
+    tk.topk_selector_tilelang_direct(idx_scores, topk, out=idx, ends=ends, order="index")
+    idx = idx.view(1, S, 1, topk)
+    out = torch.empty((1, S, H, 512), dtype=torch.bfloat16, device=device)
+    lse = torch.empty((1, S, H), dtype=torch.float32, device=device)
+    fn = lambda: bs.sparse_mla_blockscaled_path_c_apply_direct(q, None, codes, scale, idx, sm_scale=576 ** -0.5, out=out,
+                                                               lse=lse, d_v=512, kv_rope=rope)
+    steps = max(1, min(args.steps, 5))
+    secs, _ = timed_graph([fn], steps, 1)
+    per = secs / steps
+    pairs = int(torch.minimum(ends.long(), torch.tensor(topk, device=device)).sum().item())
+    flops = 2.0 * H * pairs * (576 + 512)
+    return {"workload": "sparse_mla_prefill B=1 S=8192 H=128 topk=2048 causal", "ms_per_step": per * 1e3,
+            "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", type=str, default="decode,vecmat,topk")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU; the path shards without communication "
+              "(rows / sequences / queries per GPU), so --gpus N>1 is not run here.", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels have no CPU path.", file=sys.stderr)
+        return 3
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    from cppmega_mlx_amd import native_status
+    native_status()
+    parts = set(args.only.split(","))
+
+    line = {
+        "metric": "sparse_mla_decode_tflops",
+        "value": None,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": None,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 MFMA over e4m3 KV (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {},
+    }
+    if "decode" in parts:
+        res, sample = bench_decode(args, device)
+        line["value"] = res["tflops"]
+        line["ms_per_step"] = res["ms_per_step"]
+        line["config"] = {"workload": res["workload"], "kernel": res["kernel"],
+                          "flops_per_step": res["flops_per_step"],
+                          "algorithmic_bytes_per_step": res["algorithmic_bytes_per_step"],
+                          "host_ms_per_step": res["host_ms_per_step"], "hbm_gbs": res["hbm_gbs"]}
+        line["roofline"] = {"bound": "mfma", "achieved": res["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                            "frac": res["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
+        if not args.no_cpu_baseline:
+            cpu, rel_err = cpu_baseline_decode(sample)
+            line["cpu_baseline"] = cpu
+            line["config"]["max_rel_err_vs_oracle_on_sample"] = rel_err
+        del sample
+        torch.cuda.empty_cache()
+    if "vecmat" in parts:
+        line["vecmat"] = {}
+        for M in (1, 4, 16):
+            res, sample = bench_vecmat(args, device, M)
+            if not args.no_cpu_baseline and M == 1:
+                res["cpu_baseline"], res["max_rel_err_vs_oracle_on_sample"] = cpu_baseline_vecmat(sample)
+            line["vecmat"][f"M{M}"] = res
+            del sample
+            torch.cuda.empty_cache()
+    if "topk" in parts:
+        res, sample = bench_topk(args, device)
+        if not args.no_cpu_baseline:
+            res["cpu_baseline"], res["bit_exact_vs_oracle_on_sample"] = cpu_baseline_topk(sample)
+        line["topk"] = res
+        del sample
+        torch.cuda.empty_cache()
+    if "prefill" in parts:
+        line["prefill"] = bench_prefill(args, device)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -195,8 +195,14 @@ def load() -> C.CDLL:
         return lib
 
 
-def status() -> dict[str, Any]:
-    """Probe the library (and the HIP runtime under it)."""
+_status_cache: dict[str, Any] | None = None
+
+
+def status(refresh: bool = False) -> dict[str, Any]:
+    """Probe the library (and the HIP runtime under it); the answer is cached."""
+    global _status_cache
+    if _status_cache is not None and not refresh:
+        return dict(_status_cache)
     lib = load()
     st = StatusStruct()
     rc = lib.cppmega_mi355_status(C.byref(st), C.sizeof(st))
@@ -204,13 +210,14 @@ def status() -> dict[str, Any]:
         raise NativeLibraryError(f"cppmega_mi355_status returned {rc}")
     if st.abi_version != ABI_VERSION:
         raise NativeLibraryError(f"ABI version {st.abi_version} != expected {ABI_VERSION}; rebuild the library")
-    return {
+    _status_cache = {
         "abi_version": st.abi_version,
         "device_count": st.device_count,
         "gfx950_devices": st.gfx950_devices,
         "built_for": st.built_for.decode(),
         "message": st.message.decode(),
     }
+    return dict(_status_cache)
 
 
 def check(rc: int, op: str) -> None:
