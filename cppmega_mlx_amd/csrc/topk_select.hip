@@ -1,15 +1,21 @@
-// Wavefront radix-select top-k over indexer scores (gfx950).
+// Radix-select top-k over indexer scores (gfx950).
 //
-// One 64-lane wavefront owns one score row.  The row is read from HBM exactly
-// once, with 16-byte loads, and stays in registers (up to 128 values per lane)
-// for the rest of the kernel.  A 4096-bin histogram in LDS, private to the
-// wavefront, is filled by LDS atomics and scanned by the same wavefront, so the
-// kernel needs no cross-wavefront barrier.
+// One workgroup owns one score row.  The row is read from HBM exactly once,
+// with 16-byte loads, and stays in registers for the rest of the kernel; a
+// 4096-bin histogram of the row lives in LDS.
+//
+// Rows of up to 8192 columns (topk_tile_kernel) are staged through LDS once so
+// that every thread ends up owning a contiguous run of columns: a thread's
+// selected columns are then a bit mask, one block-wide prefix sum of the
+// popcounts gives every thread its output offset, and the indices come out in
+// ascending order.  Wider rows (topk_row_kernel, up to 65536 columns) do not
+// fit in LDS; they keep the interleaved ownership of the coalesced loads and
+// compact with per-chunk ballots.
 //
 // Selection (k largest, ties toward the lower index):
-//   pass 1  histogram of bits[31:20] (sign, exponent, 3 mantissa bits) over the
-//           selectable positions; a two-level scan, walking the bins from the
-//           largest value down, finds the bin where the running count reaches k
+//   pass 1  LDS-atomic histogram of bits[31:20] (sign, exponent, 3 mantissa
+//           bits); a two-level scan over the bins, walking from the largest
+//           value down, finds the bin where the running count reaches k
 //   pass 2  the same over bits[19:8] of the elements that fell in that bin
 //   pass 3  the same over bits[7:0]
 // A pass ends the search early when the bin it found has to be taken whole;
@@ -17,11 +23,15 @@
 // the threshold value itself is duplicated beyond what is needed does the
 // emission count equal elements and keep the first `rem` of them by index.
 //
-// Emission is a ballot/mbcnt compaction in ascending index order; the optional
-// value-descending order sorts the selected (value, index) pairs in LDS.
+// Emission is a ballot/mbcnt compaction in ascending index order, staged in
+// LDS and copied out with coalesced stores; the optional value-descending
+// order sorts the selected (value, index) pairs in LDS first.
 //
 // Float compares give the ordering: -0.0 == +0.0, and NaN (which also stands
 // for "outside [start,end)") never compares true, so it is never selected.
+// After `x + 0.0f` every NaN is quiet, so NaNs fall into histogram bins no
+// real number can reach (0x7f9..0x7ff, 0xff9..0xfff); those bins are cleared
+// before the scan instead of testing every element.
 
 #include "common.h"
 
@@ -40,20 +50,20 @@ struct TopkParams {
   int sort_len;  // power of two >= k, used by the value-descending order
 };
 
-template <typename T>
-struct ScoreLoad;
-template <>
-struct ScoreLoad<float> {
+struct Half {};   // tag types: 16-bit storage
+struct BHalf {};
+template <typename T> struct Storage { typedef unsigned short type; };
+template <> struct Storage<float> { typedef float type; };
+
+template <typename T> struct ScoreLoad;
+template <> struct ScoreLoad<float> {
   static __device__ __forceinline__ void vec4(const float* p, float (&o)[4]) {
     const float4 t = *reinterpret_cast<const float4*>(p);
     o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
   }
   static __device__ __forceinline__ float one(const float* p) { return *p; }
 };
-struct Half {};   // tag types: 16-bit storage
-struct BHalf {};
-template <>
-struct ScoreLoad<Half> {
+template <> struct ScoreLoad<Half> {
   static __device__ __forceinline__ void vec4(const unsigned short* p, float (&o)[4]) {
     const uint2 t = *reinterpret_cast<const uint2*>(p);
     o[0] = f16_bits_to_f32((unsigned short)(t.x & 0xffffu));
@@ -63,8 +73,7 @@ struct ScoreLoad<Half> {
   }
   static __device__ __forceinline__ float one(const unsigned short* p) { return f16_bits_to_f32(*p); }
 };
-template <>
-struct ScoreLoad<BHalf> {
+template <> struct ScoreLoad<BHalf> {
   static __device__ __forceinline__ void vec4(const unsigned short* p, float (&o)[4]) {
     const uint2 t = *reinterpret_cast<const uint2*>(p);
     o[0] = __uint_as_float(t.x << 16);
@@ -74,15 +83,6 @@ struct ScoreLoad<BHalf> {
   }
   static __device__ __forceinline__ float one(const unsigned short* p) { return bf16_bits_to_f32(*p); }
 };
-template <typename T> struct Storage { typedef unsigned short type; };
-template <> struct Storage<float> { typedef float type; };
-
-struct BinHit {
-  unsigned bin;    // raw bin index in the histogram
-  unsigned above;  // elements in bins that rank before it
-  unsigned cnt;    // elements in it
-  unsigned total;  // elements in all bins
-};
 
 // Walk order of the bins, largest value first:
 //   kSigned      bin = bits[31:20]: non-negative bins 2047..0, then negative bins 2048..4095
@@ -90,59 +90,108 @@ struct BinHit {
 //   kAscending   larger digit = smaller value (negative prefix)
 enum { kSigned = 0, kDescending = 1, kAscending = 2 };
 
-template <int NB>
-__device__ __forceinline__ void lane_block(int lane, int mode, int& blk, bool& rev) {
-  // NB/64 consecutive walk positions per lane map to one aligned block in memory.
-  if (mode == kSigned) {
-    if (lane < 32) { blk = 31 - lane; rev = true; } else { blk = lane; rev = false; }
-  } else if (mode == kDescending) {
-    blk = 63 - lane; rev = true;
-  } else {
-    blk = lane; rev = false;
-  }
-}
+// LDS layout (unsigned words) after the histogram
+constexpr int kWaveTot = kHistBins;        // [16] per-wave totals of a scan
+constexpr int kHit = kHistBins + 16;       // [4]  bin, above, cnt
+
+struct BinHit {
+  unsigned bin, above, cnt, total;
+};
 
 // Finds the bin at which the running count, walking from the largest value
-// down, first reaches `need` (1 <= need <= total is the caller's business; if
-// need > total the hit is meaningless and only `total` may be used).
-template <int NB>
-__device__ BinHit find_bin(const unsigned* hist, unsigned need, int mode) {
-  constexpr int L = NB / 64;
-  static_assert(L >= 1 && L <= 64 && (L % 4 == 0), "bins per lane");
-  const int lane = lane_id();
-  int blk; bool rev;
-  lane_block<NB>(lane, mode, blk, rev);
-  unsigned sum = 0;
-  const uint4* src = reinterpret_cast<const uint4*>(hist + blk * L);
+// down, first reaches `need`.  All THREADS threads call it.  The NB bins are
+// read as NB/4 aligned quads, thread t taking quads t, t+THREADS, ... so that
+// the 16-byte LDS reads of a wavefront are consecutive (no bank conflicts).
+// Quads [s*THREADS, (s+1)*THREADS) form "segment" s; the walk visits whole
+// segments in a mode-dependent order, ascending or descending inside each.
+template <int NB, int THREADS>
+__device__ BinHit find_bin(unsigned* smem, unsigned need, int mode) {
+  constexpr int SEGS = NB / 4 / THREADS;
+  constexpr int WAVES = THREADS / 64;
+  static_assert(SEGS >= 1 && SEGS <= 4 && NB == SEGS * 4 * THREADS, "segments");
+  static_assert(SEGS * WAVES <= 16, "scan scratch");
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  uint4 quad[SEGS];
+  unsigned qsum[SEGS], incl[SEGS];
 #pragma unroll
-  for (int i = 0; i < L / 4; ++i) {
-    const uint4 t = src[i];
-    sum += t.x + t.y + t.z + t.w;
+  for (int s = 0; s < SEGS; ++s) {
+    quad[s] = reinterpret_cast<const uint4*>(smem)[s * THREADS + tid];
+    qsum[s] = quad[s].x + quad[s].y + quad[s].z + quad[s].w;
+    incl[s] = wave_inclusive_sum_dpp(qsum[s]);
+    if (lane == 63) smem[kWaveTot + s * WAVES + wave] = incl[s];
   }
-  const unsigned incl = wave_inclusive_sum(sum);
+  __syncthreads();
+  unsigned wtot[SEGS][WAVES], segtot[SEGS], total = 0;
+#pragma unroll
+  for (int s = 0; s < SEGS; ++s) {
+    segtot[s] = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      wtot[s][w] = smem[kWaveTot + s * WAVES + w];
+      segtot[s] += wtot[s][w];
+    }
+    total += segtot[s];
+  }
+  // walk step m visits segment seg(m), descending (larger quad index first) when desc(m)
+  unsigned walked = 0;   // elements in segments the walk has finished
+#pragma unroll
+  for (int m = 0; m < SEGS; ++m) {
+    int s; bool desc;
+    if (mode == kAscending) { s = m; desc = false; }
+    else if (mode == kDescending) { s = SEGS - 1 - m; desc = true; }
+    else {  // kSigned: bins 2047..0 then 2048..4095 (SEGS is even here)
+      if (m < SEGS / 2) { s = SEGS / 2 - 1 - m; desc = true; } else { s = m; desc = false; }
+    }
+    // (the loop is unrolled and `s` selects among registers: keep it branch-free over s)
+    unsigned my_sum = 0, my_incl = 0, my_wave_tot = 0, waves_before = 0;
+    uint4 my_quad = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int ss = 0; ss < SEGS; ++ss) {
+      if (ss == s) {
+        my_sum = qsum[ss]; my_incl = incl[ss]; my_quad = quad[ss]; my_wave_tot = wtot[ss][0];
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+          if (w == wave) my_wave_tot = wtot[ss][w];
+          if (desc ? (w > wave) : (w < wave)) waves_before += wtot[ss][w];
+        }
+      }
+    }
+    const unsigned lanes_before = desc ? (my_wave_tot - my_incl) : (my_incl - my_sum);
+    const unsigned before = walked + waves_before + lanes_before;
+    if (before < need && need <= before + my_sum) {      // exactly one (thread, m) when need <= total
+      const unsigned cs[4] = {my_quad.x, my_quad.y, my_quad.z, my_quad.w};
+      unsigned run = before;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int slot = desc ? 3 - i : i;
+        const unsigned c = cs[slot];
+        if (run < need && need <= run + c) {
+          smem[kHit + 0] = (unsigned)((s * THREADS + tid) * 4 + slot);
+          smem[kHit + 1] = run;
+          smem[kHit + 2] = c;
+        }
+        run += c;
+      }
+    }
+    walked += (s == 0 ? segtot[0] : 0);
+#pragma unroll
+    for (int ss = 1; ss < SEGS; ++ss) walked += (s == ss ? segtot[ss] : 0);
+  }
+  __syncthreads();
   BinHit hit;
-  hit.total = __shfl(incl, 63, 64);
-  const unsigned long long m1 = __ballot(incl >= need);
-  const int lx = m1 ? __builtin_ctzll(m1) : 63;
-  const unsigned above_lane = __shfl(incl - sum, lx, 64);
-  int blkx; bool revx;
-  lane_block<NB>(lx, mode, blkx, revx);
-  const int slot = revx ? (L - 1 - lane) : lane;
-  const unsigned c = (lane < L) ? hist[blkx * L + slot] : 0u;
-  const unsigned incl2 = wave_inclusive_sum(c);
-  const unsigned long long m2 = __ballot(lane < L && above_lane + incl2 >= need);
-  const int ix = m2 ? __builtin_ctzll(m2) : 0;
-  hit.bin = (unsigned)(blkx * L + (revx ? (L - 1 - ix) : ix));
-  hit.above = above_lane + __shfl(incl2 - c, ix, 64);
-  hit.cnt = __shfl(c, ix, 64);
+  hit.bin = smem[kHit + 0];
+  hit.above = smem[kHit + 1];
+  hit.cnt = smem[kHit + 2];
+  hit.total = total;
   return hit;
 }
 
-__device__ __forceinline__ void zero_hist(unsigned* hist, int lane) {
+template <int THREADS>
+__device__ __forceinline__ void zero_hist(unsigned* hist, int nbins) {
   uint4* dst = reinterpret_cast<uint4*>(hist);
   const uint4 z = make_uint4(0, 0, 0, 0);
-#pragma unroll
-  for (int i = 0; i < kHistBins / 4 / 64; ++i) dst[i * 64 + lane] = z;
+  for (int i = (int)threadIdx.x; i < nbins / 4; i += THREADS) dst[i] = z;
 }
 
 // Monotone key of a float: larger value <=> larger key.
@@ -151,67 +200,25 @@ __device__ __forceinline__ unsigned order_key(float x) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// Compaction of the selected elements, ascending by index.
-//   TIE == false: selected <=> x >= thr
-//   TIE == true : selected <=> x > thr, or x == thr and fewer than `rem`
-//                 equal elements precede it
-// SORTED == false: out_row[pos] = index.   SORTED == true: pairs[pos] = key.
-template <int ITEMS, int VEC, bool TIE, bool SORTED>
-__device__ __forceinline__ unsigned emit(const float (&v)[ITEMS][VEC], float thr, unsigned rem,
-                                         int* out_row, unsigned long long* pairs) {
-  const int lane = lane_id();
-  unsigned base_g = 0, base_e = 0;
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    bool g[VEC], e[VEC];
-    unsigned pre_g = 0, pre_e = 0, tot_g = 0, tot_e = 0;
-#pragma unroll
-    for (int c = 0; c < VEC; ++c) {
-      const float x = v[j][c];
-      g[c] = TIE ? (x > thr) : (x >= thr);
-      const unsigned long long mg = __ballot(g[c]);
-      pre_g += mbcnt(mg);
-      tot_g += (unsigned)__popcll(mg);
-      if (TIE) {
-        e[c] = (x == thr);
-        const unsigned long long me = __ballot(e[c]);
-        pre_e += mbcnt(me);
-        tot_e += (unsigned)__popcll(me);
-      } else {
-        e[c] = false;
-      }
-    }
-    if (tot_g + tot_e) {
-      unsigned run_g = base_g + pre_g, run_e = base_e + pre_e;
-#pragma unroll
-      for (int c = 0; c < VEC; ++c) {
-        const bool sel = g[c] || (TIE && e[c] && run_e < rem);
-        const unsigned pos = run_g + (TIE ? min(run_e, rem) : 0u);
-        if (sel) {
-          const unsigned idx = (unsigned)((j * 64 + lane) * VEC + c);
-          if (SORTED) {
-            pairs[pos] = ((unsigned long long)order_key(v[j][c]) << 32) | (0xffffffffu - idx);
-          } else {
-            out_row[pos] = (int)idx;
-          }
-        }
-        run_g += g[c] ? 1u : 0u;
-        if (TIE) run_e += e[c] ? 1u : 0u;
-      }
-    }
-    base_g += tot_g;
-    base_e += tot_e;
-  }
-  return base_g + (TIE ? min(base_e, rem) : 0u);
-}
+// ---------------------------------------------------------------------------
+// Rows of up to 8192 columns: 256 threads, thread t owns columns [t*E, (t+1)*E).
+// ---------------------------------------------------------------------------
+constexpr int kTileThreads = 256;
+constexpr int kTileScratch = kHistBins + 64;            // words: histogram + scan scratch
+__host__ __device__ constexpr int tile_pad(int E) { return E == 4 ? 0 : 4; }
 
-template <typename ScoreT, int ITEMS, int VEC>
-__global__ __launch_bounds__(64) void topk_wave_kernel(const TopkParams p) {
+template <typename ScoreT, int E, int VEC>
+__global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParams p) {
+  constexpr int THREADS = kTileThreads;
+  constexpr int ITEMS = E / VEC;                        // loads per thread
+  constexpr int CHUNK = THREADS * VEC;                  // columns covered by one load per thread
+  constexpr int PITCH = E + tile_pad(E);                // words between the runs of consecutive threads
   extern __shared__ __align__(16) unsigned smem[];
+  float* tile = reinterpret_cast<float*>(smem);
   unsigned* hist = smem;
   typedef typename Storage<ScoreT>::type St;
 
-  const int lane = lane_id();
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int row = (int)blockIdx.x;
   const int T = p.width;
   int start = p.starts ? p.starts[row] : 0;
@@ -222,60 +229,60 @@ __global__ __launch_bounds__(64) void topk_wave_kernel(const TopkParams p) {
   int* out_row = p.out + (long long)row * p.k;
   const float kNaN = __uint_as_float(0x7fc00000u);
   const float kNegInf = __uint_as_float(0xff800000u);
+  const unsigned k = (unsigned)p.k;
 
-  // ---- the row: HBM -> registers, once -----------------------------------
-  float v[ITEMS][VEC];
+  // ---- HBM -> LDS, coalesced; chunks with nothing selectable are not read ----------
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
-    const int chunk_lo = j * 64 * VEC;
-    const int base = chunk_lo + lane * VEC;
-    if (chunk_lo >= end || chunk_lo + 64 * VEC <= start) {   // uniform: nothing selectable here
-#pragma unroll
-      for (int c = 0; c < VEC; ++c) v[j][c] = kNaN;
-    } else if constexpr (VEC == 4) {
-      if (base < T) {
-        ScoreLoad<ScoreT>::vec4(src + base, v[j]);
-      } else {
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) v[j][c] = kNaN;
-      }
+    const int chunk_lo = j * CHUNK;
+    const int col = chunk_lo + tid * VEC;
+    if (chunk_lo >= end || chunk_lo + CHUNK <= start || col >= T) continue;
+    float* dst = tile + col + (col / E) * tile_pad(E);
+    if constexpr (VEC == 4) {
+      float t4[4];
+      ScoreLoad<ScoreT>::vec4(src + col, t4);
+      *reinterpret_cast<float4*>(dst) = make_float4(t4[0], t4[1], t4[2], t4[3]);
     } else {
-      v[j][0] = (base < T) ? ScoreLoad<ScoreT>::one(src + base) : kNaN;
-    }
-  }
-  zero_hist(hist, lane);
-
-  // ---- canonicalise: -0 -> +0, signalling NaN -> quiet NaN, mask -> NaN -----
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    const int chunk_lo = j * 64 * VEC;
-    const bool inside = chunk_lo >= start && chunk_lo + 64 * VEC <= end;   // uniform
-#pragma unroll
-    for (int c = 0; c < VEC; ++c) {
-      float x = v[j][c] + 0.0f;
-      if (!inside) {
-        const int idx = chunk_lo + lane * VEC + c;
-        x = (idx >= start && idx < end) ? x : kNaN;
-      }
-      if (p.neg_inf_masked) x = (x == kNegInf) ? kNaN : x;
-      v[j][c] = x;
+      *dst = ScoreLoad<ScoreT>::one(src + col);
     }
   }
   __syncthreads();
+  // ---- LDS -> registers: my contiguous run ------------------------------------------
+  float v[E];
+#pragma unroll
+  for (int i = 0; i < E / 4; ++i) {
+    const float4 t4 = *reinterpret_cast<const float4*>(tile + tid * PITCH + 4 * i);
+    v[4 * i] = t4.x; v[4 * i + 1] = t4.y; v[4 * i + 2] = t4.z; v[4 * i + 3] = t4.w;
+  }
+  __syncthreads();
+  zero_hist<THREADS>(hist, kHistBins);
+  __syncthreads();
 
-  // ---- pass 1: bits[31:20] ---------------------------------------------------
+  // ---- canonicalise (-0 -> +0, NaN -> quiet NaN, masked -> NaN) + pass 1 -------------
+  const int col0 = tid * E;
+  if (col0 >= start && col0 + E <= end && !p.neg_inf_masked) {
 #pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
+    for (int i = 0; i < E; ++i) {
+      const float x = v[i] + 0.0f;
+      v[i] = x;
+      atomicAdd(&hist[__float_as_uint(x) >> 20], 1u);
+    }
+  } else {
 #pragma unroll
-    for (int c = 0; c < VEC; ++c) {
-      const float x = v[j][c];
+    for (int i = 0; i < E; ++i) {
+      float x = v[i] + 0.0f;
+      const int idx = col0 + i;
+      x = (idx >= start && idx < end) ? x : kNaN;
+      if (p.neg_inf_masked) x = (x == kNegInf) ? kNaN : x;
+      v[i] = x;
       if (x == x) atomicAdd(&hist[__float_as_uint(x) >> 20], 1u);
     }
   }
   __syncthreads();
+  if (tid < 7) { hist[0x7f9 + tid] = 0u; hist[0xff9 + tid] = 0u; }   // bins only NaN patterns reach
+  __syncthreads();
 
-  const unsigned k = (unsigned)p.k;
-  BinHit h1 = find_bin<kHistBins>(hist, k, kSigned);
+  BinHit h1 = find_bin<kHistBins, THREADS>(smem, k, kSigned);
   float thr;
   unsigned rem = 0;
   bool tie = false;
@@ -288,70 +295,98 @@ __global__ __launch_bounds__(64) void topk_wave_kernel(const TopkParams p) {
     if (rem == h1.cnt) {
       lo_bits = (h1.bin << 20) | (neg ? 0x000fffffu : 0u);
     } else {
-      // ---- pass 2: bits[19:8] of the elements in bin h1 --------------------
-      __syncthreads();
-      zero_hist(hist, lane);
+      // ---- pass 2: bits[19:8] of the elements in bin h1 -----------------------------
+      zero_hist<THREADS>(hist, kHistBins);
       __syncthreads();
       const unsigned p1 = h1.bin;
 #pragma unroll
-      for (int j = 0; j < ITEMS; ++j) {
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) {
-          const unsigned u = __float_as_uint(v[j][c]);
-          if ((u >> 20) == p1) atomicAdd(&hist[(u >> 8) & 0xfffu], 1u);
-        }
+      for (int i = 0; i < E; ++i) {
+        const unsigned u = __float_as_uint(v[i]);
+        if ((u >> 20) == p1) atomicAdd(&hist[(u >> 8) & 0xfffu], 1u);
       }
       __syncthreads();
-      const BinHit h2 = find_bin<kHistBins>(hist, rem, neg ? kAscending : kDescending);
+      const BinHit h2 = find_bin<kHistBins, THREADS>(smem, rem, neg ? kAscending : kDescending);
       rem -= h2.above;
       const unsigned p2 = (p1 << 12) | h2.bin;     // bits[31:8]
       if (rem == h2.cnt) {
         lo_bits = (p2 << 8) | (neg ? 0xffu : 0u);
       } else {
-        // ---- pass 3: bits[7:0] ------------------------------------------------
-        __syncthreads();
-        if (lane < 64) reinterpret_cast<uint4*>(hist)[lane] = make_uint4(0, 0, 0, 0);
+        // ---- pass 3: bits[7:0] (256 of 1024 cleared slots are used) ------------------
+        zero_hist<THREADS>(hist, 1024);
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < ITEMS; ++j) {
-#pragma unroll
-          for (int c = 0; c < VEC; ++c) {
-            const unsigned u = __float_as_uint(v[j][c]);
-            if ((u >> 8) == p2) atomicAdd(&hist[u & 0xffu], 1u);
-          }
+        for (int i = 0; i < E; ++i) {
+          const unsigned u = __float_as_uint(v[i]);
+          if ((u >> 8) == p2) atomicAdd(&hist[u & 0xffu], 1u);
         }
         __syncthreads();
-        const BinHit h3 = find_bin<256>(hist, rem, neg ? kAscending : kDescending);
+        const BinHit h3 = find_bin<1024, THREADS>(smem, rem, neg ? kAscending : kDescending);
         rem -= h3.above;
         lo_bits = (p2 << 8) | h3.bin;
         tie = rem != h3.cnt;
       }
     }
-    // bins above 0xff800000 hold only NaN patterns: the lowest real value is -inf
-    if (lo_bits > 0xff800000u) lo_bits = 0xff800000u;
+    if (lo_bits > 0xff800000u) lo_bits = 0xff800000u;   // below -inf there are only NaN patterns
     thr = __uint_as_float(lo_bits);
   }
-  __syncthreads();   // the histogram memory is reused by the sorted emission
 
-  // ---- emission ---------------------------------------------------------------
-  unsigned n_sel;
-  unsigned long long* pairs = reinterpret_cast<unsigned long long*>(smem);
-  if (p.order == CPPMEGA_MI355_TOPK_ORDER_INDEX) {
-    n_sel = tie ? emit<ITEMS, VEC, true, false>(v, thr, rem, out_row, pairs)
-                : emit<ITEMS, VEC, false, false>(v, thr, rem, out_row, pairs);
-    for (unsigned i = n_sel + lane; i < k; i += 64) out_row[i] = -1;
+  // ---- emission: bit masks, one block-wide prefix sum, ascending indices --------------
+  unsigned gmask = 0, emask = 0;
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    const float x = v[i];
+    gmask |= ((tie ? (x > thr) : (x >= thr)) ? 1u : 0u) << i;
+    if (tie) emask |= ((x == thr) ? 1u : 0u) << i;
+  }
+  const unsigned cg = (unsigned)__popc(gmask), ce = (unsigned)__popc(emask);
+  const unsigned packed = cg | (ce << 16);               // both counts fit in 16 bits (<= 8192)
+  const unsigned incl = wave_inclusive_sum_dpp(packed);
+  if (lane == 63) smem[kWaveTot + wave] = incl;
+  __syncthreads();
+  unsigned before = incl - packed, totals = 0;
+#pragma unroll
+  for (int w = 0; w < THREADS / 64; ++w) {
+    const unsigned t = smem[kWaveTot + w];
+    if (w < wave) before += t;
+    totals += t;
+  }
+  unsigned run_g = before & 0xffffu, run_e = before >> 16;
+  const unsigned n_sel = (totals & 0xffffu) + min(totals >> 16, rem);
+  const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
+  int* stage = reinterpret_cast<int*>(smem + kTileScratch);
+  unsigned long long* pairs = reinterpret_cast<unsigned long long*>(smem + kTileScratch);
+  if (!sorted && !tie) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      if ((gmask >> i) & 1u) stage[run_g++] = col0 + i;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      const bool g = (gmask >> i) & 1u, e = (emask >> i) & 1u;
+      const bool sel = g || (e && run_e < rem);
+      const unsigned pos = run_g + min(run_e, rem);
+      if (sel) {
+        const unsigned idx = (unsigned)(col0 + i);
+        if (sorted) pairs[pos] = ((unsigned long long)order_key(v[i]) << 32) | (0xffffffffu - idx);
+        else stage[pos] = (int)idx;
+      }
+      run_g += g ? 1u : 0u;
+      run_e += e ? 1u : 0u;
+    }
+  }
+  if (!sorted) {
+    __syncthreads();
+    for (unsigned i = tid; i < k; i += THREADS) out_row[i] = (i < n_sel) ? stage[i] : -1;
     return;
   }
-
-  n_sel = tie ? emit<ITEMS, VEC, true, true>(v, thr, rem, out_row, pairs)
-              : emit<ITEMS, VEC, false, true>(v, thr, rem, out_row, pairs);
   const unsigned P = (unsigned)p.sort_len;
-  for (unsigned i = n_sel + lane; i < P; i += 64) pairs[i] = 0ull;   // sorts last
+  for (unsigned i = n_sel + tid; i < P; i += THREADS) pairs[i] = 0ull;   // sorts last
   __syncthreads();
   // bitonic sort, descending: larger value first, then lower index
   for (unsigned size = 2; size <= P; size <<= 1) {
     for (unsigned stride = size >> 1; stride > 0; stride >>= 1) {
-      for (unsigned t = lane; t < P / 2; t += 64) {
+      for (unsigned t = tid; t < P / 2; t += THREADS) {
         const unsigned i = 2 * t - (t & (stride - 1));
         const unsigned jx = i + stride;
         const bool desc = (i & size) == 0;
@@ -361,29 +396,251 @@ __global__ __launch_bounds__(64) void topk_wave_kernel(const TopkParams p) {
       __syncthreads();
     }
   }
-  for (unsigned i = lane; i < k; i += 64)
+  for (unsigned i = tid; i < k; i += THREADS)
     out_row[i] = (i < n_sel) ? (int)(0xffffffffu - (unsigned)(pairs[i] & 0xffffffffull)) : -1;
 }
 
-template <typename ScoreT>
-int launch_for_type(const TopkParams& p, bool vec4, size_t smem, hipStream_t stream) {
-  const dim3 grid((unsigned)p.rows), block(64);
+// ---------------------------------------------------------------------------
+// Wider rows (up to 65536 columns): 1024 threads, interleaved ownership as loaded
+// (column = (j*THREADS + tid)*VEC + c).  Bins come from the monotone key of the
+// value, so every walk is "larger digit first".
+// ---------------------------------------------------------------------------
+constexpr int kWideThreads = 1024;
+constexpr int kWideWaves = kWideThreads / 64;
+constexpr int kWideEmit = kHistBins + 64;               // [ITEMS*16*2] per (chunk, wave) counts
+constexpr int kWideScratch = kHistBins + 64 + 2 * 32 * kWideWaves;
+
+template <typename ScoreT, int ITEMS, int VEC>
+__global__ __launch_bounds__(kWideThreads) void topk_wide_kernel(const TopkParams p) {
+  constexpr int THREADS = kWideThreads, WAVES = kWideWaves;
+  constexpr int CHUNK = THREADS * VEC;
+  extern __shared__ __align__(16) unsigned smem[];
+  unsigned* hist = smem;
+  typedef typename Storage<ScoreT>::type St;
+
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int row = (int)blockIdx.x;
   const int T = p.width;
-#define CM_TOPK_LAUNCH(ITEMS, VEC)                                                        \
-  do {                                                                                    \
-    hipLaunchKernelGGL((topk_wave_kernel<ScoreT, ITEMS, VEC>), grid, block, smem, stream, p); \
-    return 0;                                                                             \
-  } while (0)
-  if (vec4) {
-    if (T <= 512) CM_TOPK_LAUNCH(2, 4);
-    if (T <= 2048) CM_TOPK_LAUNCH(8, 4);
-    if (T <= 8192) CM_TOPK_LAUNCH(32, 4);
-  } else {
-    if (T <= 512) CM_TOPK_LAUNCH(8, 1);
-    if (T <= 2048) CM_TOPK_LAUNCH(32, 1);
-    if (T <= 8192) CM_TOPK_LAUNCH(128, 1);
+  int start = p.starts ? p.starts[row] : 0;
+  int end = p.ends ? p.ends[row] : T;
+  start = min(max(start, 0), T);
+  end = min(max(end, 0), T);
+  const St* src = reinterpret_cast<const St*>(p.scores) + (long long)row * p.row_stride;
+  int* out_row = p.out + (long long)row * p.k;
+  const float kNaN = __uint_as_float(0x7fc00000u);
+  const float kNegInf = __uint_as_float(0xff800000u);
+  const unsigned k = (unsigned)p.k;
+
+  float v[ITEMS][VEC];
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const int chunk_lo = j * CHUNK;
+    const int base = chunk_lo + tid * VEC;
+    if (chunk_lo >= end || chunk_lo + CHUNK <= start || base >= T) {
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) v[j][c] = kNaN;
+    } else if constexpr (VEC == 4) {
+      ScoreLoad<ScoreT>::vec4(src + base, v[j]);
+    } else {
+      v[j][0] = ScoreLoad<ScoreT>::one(src + base);
+    }
   }
-#undef CM_TOPK_LAUNCH
+  zero_hist<THREADS>(hist, kHistBins);
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+      float x = v[j][c] + 0.0f;
+      const int idx = j * CHUNK + tid * VEC + c;
+      x = (idx >= start && idx < end) ? x : kNaN;
+      if (p.neg_inf_masked) x = (x == kNegInf) ? kNaN : x;
+      v[j][c] = x;
+      if (x == x) atomicAdd(&hist[order_key(x) >> 20], 1u);
+    }
+  }
+  __syncthreads();
+
+  BinHit h1 = find_bin<kHistBins, THREADS>(smem, k, kDescending);
+  float thr;
+  unsigned rem = 0;
+  bool tie = false;
+  if (h1.total <= k) {
+    thr = kNegInf;
+  } else {
+    unsigned lo_key;
+    rem = k - h1.above;
+    if (rem == h1.cnt) {
+      lo_key = h1.bin << 20;
+    } else {
+      zero_hist<THREADS>(hist, kHistBins);
+      __syncthreads();
+      const unsigned p1 = h1.bin;
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j)
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+          const float x = v[j][c];
+          const unsigned key = order_key(x);
+          if (x == x && (key >> 20) == p1) atomicAdd(&hist[(key >> 8) & 0xfffu], 1u);
+        }
+      __syncthreads();
+      const BinHit h2 = find_bin<kHistBins, THREADS>(smem, rem, kDescending);
+      rem -= h2.above;
+      const unsigned p2 = (p1 << 12) | h2.bin;
+      if (rem == h2.cnt) {
+        lo_key = p2 << 8;
+      } else {
+        zero_hist<THREADS>(hist, kHistBins);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j)
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) {
+            const float x = v[j][c];
+            const unsigned key = order_key(x);
+            if (x == x && (key >> 8) == p2) atomicAdd(&hist[key & 0xffu], 1u);
+          }
+        __syncthreads();
+        const BinHit h3 = find_bin<kHistBins, THREADS>(smem, rem, kDescending);
+        rem -= h3.above;
+        lo_key = (p2 << 8) | h3.bin;
+        tie = rem != h3.cnt;
+      }
+    }
+    if (lo_key < 0x007fffffu) lo_key = 0x007fffffu;       // the key of -inf; below it only NaN patterns
+    thr = __uint_as_float((lo_key & 0x80000000u) ? (lo_key ^ 0x80000000u) : ~lo_key);
+  }
+
+  // ---- emission: per-chunk ballots ------------------------------------------------------
+  unsigned long long gflags = 0, eflags = 0;   // bit j*VEC+c
+  unsigned short pre_g[ITEMS], pre_e[ITEMS];
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    unsigned pg = 0, pe = 0, tg = 0, te = 0;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+      const float x = v[j][c];
+      const bool g = tie ? (x > thr) : (x >= thr);
+      const unsigned long long mg = __ballot(g);
+      pg += mbcnt(mg);
+      tg += (unsigned)__popcll(mg);
+      gflags |= (g ? 1ull : 0ull) << (j * VEC + c);
+      if (tie) {
+        const bool e = (x == thr);
+        const unsigned long long me = __ballot(e);
+        pe += mbcnt(me);
+        te += (unsigned)__popcll(me);
+        eflags |= (e ? 1ull : 0ull) << (j * VEC + c);
+      }
+    }
+    pre_g[j] = (unsigned short)pg;
+    pre_e[j] = (unsigned short)pe;
+    if (lane == 0) {
+      smem[kWideEmit + (j * WAVES + wave) * 2 + 0] = tg;
+      smem[kWideEmit + (j * WAVES + wave) * 2 + 1] = te;
+    }
+  }
+  __syncthreads();
+  const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
+  int* stage = reinterpret_cast<int*>(smem + kWideScratch);
+  unsigned long long* pairs = reinterpret_cast<unsigned long long*>(smem + kWideScratch);
+  unsigned base_g = 0, base_e = 0;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    unsigned run_g = base_g, run_e = base_e;
+    for (int w = 0; w < WAVES; ++w) {
+      const unsigned tg = smem[kWideEmit + (j * WAVES + w) * 2 + 0];
+      const unsigned te = smem[kWideEmit + (j * WAVES + w) * 2 + 1];
+      if (w < wave) { run_g += tg; run_e += te; }
+      base_g += tg;
+      base_e += te;
+    }
+    run_g += pre_g[j];
+    run_e += pre_e[j];
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+      const bool g = (gflags >> (j * VEC + c)) & 1ull;
+      const bool e = (eflags >> (j * VEC + c)) & 1ull;
+      const bool sel = g || (e && run_e < rem);
+      const unsigned pos = run_g + min(run_e, rem);
+      if (sel) {
+        const unsigned idx = (unsigned)(j * CHUNK + tid * VEC + c);
+        if (sorted) pairs[pos] = ((unsigned long long)order_key(v[j][c]) << 32) | (0xffffffffu - idx);
+        else stage[pos] = (int)idx;
+      }
+      run_g += g ? 1u : 0u;
+      run_e += e ? 1u : 0u;
+    }
+  }
+  const unsigned n_sel = base_g + min(base_e, rem);
+  if (!sorted) {
+    __syncthreads();
+    for (unsigned i = tid; i < k; i += THREADS) out_row[i] = (i < n_sel) ? stage[i] : -1;
+    return;
+  }
+  const unsigned P = (unsigned)p.sort_len;
+  for (unsigned i = n_sel + tid; i < P; i += THREADS) pairs[i] = 0ull;
+  __syncthreads();
+  for (unsigned size = 2; size <= P; size <<= 1) {
+    for (unsigned stride = size >> 1; stride > 0; stride >>= 1) {
+      for (unsigned t = tid; t < P / 2; t += THREADS) {
+        const unsigned i = 2 * t - (t & (stride - 1));
+        const unsigned jx = i + stride;
+        const bool desc = (i & size) == 0;
+        const unsigned long long a = pairs[i], b = pairs[jx];
+        if ((a < b) == desc) { pairs[i] = b; pairs[jx] = a; }
+      }
+      __syncthreads();
+    }
+  }
+  for (unsigned i = tid; i < k; i += THREADS)
+    out_row[i] = (i < n_sel) ? (int)(0xffffffffu - (unsigned)(pairs[i] & 0xffffffffull)) : -1;
+}
+
+template <typename K>
+int launch_kernel(K kernel, const TopkParams& p, int threads, size_t smem, hipStream_t stream) {
+  if (smem > 64 * 1024 &&
+      hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    return -2;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)p.rows), dim3((unsigned)threads), smem, stream, p);
+  return 0;
+}
+
+template <typename ScoreT>
+int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* smem_out) {
+  const int T = p.width;
+  const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
+  const size_t out_words = sorted ? (size_t)p.sort_len * 2 : (size_t)p.k;
+  if (T <= 8192) {
+    auto tile_smem = [&](int E) {
+      const size_t tile_words = (size_t)kTileThreads * (E + tile_pad(E));
+      const size_t need = (size_t)kTileScratch + out_words;
+      return (need > tile_words ? need : tile_words) * 4;
+    };
+#define CM_TOPK_TILE(E)                                                                   \
+  do {                                                                                    \
+    const size_t smem = tile_smem(E);                                                     \
+    *smem_out = smem;                                                                     \
+    if (smem > 160 * 1024) return -3;                                                     \
+    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4>, p, kTileThreads, smem, stream) \
+                : launch_kernel(topk_tile_kernel<ScoreT, E, 1>, p, kTileThreads, smem, stream); \
+  } while (0)
+    if (T <= 1024) CM_TOPK_TILE(4);
+    if (T <= 2048) CM_TOPK_TILE(8);
+    if (T <= 4096) CM_TOPK_TILE(16);
+    CM_TOPK_TILE(32);
+#undef CM_TOPK_TILE
+  }
+  const size_t smem = ((size_t)kWideScratch + out_words) * 4;
+  *smem_out = smem;
+  if (smem > 160 * 1024) return -3;
+  if (vec4) {
+    if (T <= 32768) return launch_kernel(topk_wide_kernel<ScoreT, 8, 4>, p, kWideThreads, smem, stream);
+    if (T <= 65536) return launch_kernel(topk_wide_kernel<ScoreT, 16, 4>, p, kWideThreads, smem, stream);
+  } else {
+    if (T <= 32768) return launch_kernel(topk_wide_kernel<ScoreT, 32, 1>, p, kWideThreads, smem, stream);
+  }
   return -1;
 }
 
@@ -397,14 +654,14 @@ int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream) {
   if (a.row_stride < a.width) return fail(CPPMEGA_MI355_ERR_SHAPE, "topk: row_stride %lld < width %d", (long long)a.row_stride, a.width);
   if (a.order != CPPMEGA_MI355_TOPK_ORDER_INDEX && a.order != CPPMEGA_MI355_TOPK_ORDER_VALUE)
     return fail(CPPMEGA_MI355_ERR_SHAPE, "topk: unknown order %d", a.order);
-  if (a.width > 8192)
-    return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "topk: width %d exceeds the 8192 a wavefront keeps in registers", a.width);
-  if (a.rows == 0) return 0;
-
-  const int esz = dtype_size(a.score_dtype);
   if (a.score_dtype != CPPMEGA_MI355_F32 && a.score_dtype != CPPMEGA_MI355_F16 && a.score_dtype != CPPMEGA_MI355_BF16)
     return fail(CPPMEGA_MI355_ERR_DTYPE, "topk: scores must be float32, float16 or bfloat16");
+  const int esz = dtype_size(a.score_dtype);
   const bool vec4 = (a.width % 4 == 0) && (a.row_stride % 4 == 0) && (((uintptr_t)a.scores) % (size_t)(4 * esz) == 0);
+  if (a.width > (vec4 ? 65536 : 32768))
+    return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "topk: width %d exceeds what one workgroup keeps in registers (%d)",
+                a.width, vec4 ? 65536 : 32768);
+  if (a.rows == 0) return 0;
 
   TopkParams p;
   p.scores = a.scores; p.row_stride = a.row_stride; p.starts = a.starts; p.ends = a.ends; p.out = a.indices;
@@ -412,14 +669,15 @@ int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream) {
   int sort_len = 2;
   while (sort_len < a.k) sort_len <<= 1;
   p.sort_len = sort_len;
-  size_t smem = (size_t)kHistBins * 4;
-  if (a.order == CPPMEGA_MI355_TOPK_ORDER_VALUE && (size_t)sort_len * 8 > smem) smem = (size_t)sort_len * 8;
 
   int rc;
-  if (a.score_dtype == CPPMEGA_MI355_F32) rc = launch_for_type<float>(p, vec4, smem, stream);
-  else if (a.score_dtype == CPPMEGA_MI355_F16) rc = launch_for_type<Half>(p, vec4, smem, stream);
-  else rc = launch_for_type<BHalf>(p, vec4, smem, stream);
-  if (rc != 0) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "topk: no kernel for width %d", a.width);
+  size_t smem = 0;
+  if (a.score_dtype == CPPMEGA_MI355_F32) rc = launch_for_type<float>(p, vec4, stream, &smem);
+  else if (a.score_dtype == CPPMEGA_MI355_F16) rc = launch_for_type<Half>(p, vec4, stream, &smem);
+  else rc = launch_for_type<BHalf>(p, vec4, stream, &smem);
+  if (rc == -3)
+    return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "topk: k=%d with this order needs %zu bytes of LDS (limit 160 KiB)", a.k, smem);
+  if (rc != 0) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "topk: no kernel for width %d (rc %d)", a.width, rc);
   CM_HIP_CHECK(hipGetLastError());
   return 0;
 }

@@ -45,7 +45,7 @@ __all__ = [
     "topk_selector_tilelang_direct",
 ]
 
-MAX_WIDTH = 8192  # columns one wavefront keeps in registers
+MAX_WIDTH = 65536  # columns one workgroup keeps in registers
 _SCORE_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
 

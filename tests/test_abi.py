@@ -85,7 +85,7 @@ def test_contract_violations_return_shape_and_dtype_codes_without_a_gpu():
     assert b"topk must be in [1, 16]" in lib.cppmega_mi355_last_error()
     t.k, t.score_dtype = 4, _lib.I32
     assert lib.cppmega_mi355_topk_select(C.byref(t), C.sizeof(t), None) == _lib.ERR_DTYPE
-    t.score_dtype, t.width, t.row_stride, t.k = _lib.F32, 20000, 20000, 4
+    t.score_dtype, t.width, t.row_stride, t.k = _lib.F32, 70000, 70000, 4
     assert lib.cppmega_mi355_topk_select(C.byref(t), C.sizeof(t), None) == _lib.ERR_UNSUPPORTED
 
     m = _lib.SparseMlaArgs()

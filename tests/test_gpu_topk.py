@@ -38,7 +38,7 @@ def test_reference_known_answers(device, golden_dir):
 
 
 @pytest.mark.parametrize("rows,width,k", [(4, 64, 8), (3, 512, 64), (5, 2048, 256), (6, 8192, 2048), (2, 8192, 1),
-                                          (2, 8192, 8192), (3, 100, 7), (2, 1001, 500), (2, 4096, 2048), (1, 4, 4)])
+                                          (2, 8192, 8192), (3, 100, 7), (2, 1001, 500), (2, 4096, 2048), (1, 4, 4), (2, 20000, 3000), (1, 65536, 2048), (2, 9001, 100)])
 @pytest.mark.parametrize("masked", [False, True])
 @pytest.mark.parametrize("order", ["index", "value"])
 def test_random_rows_bit_exact(device, rows, width, k, masked, order):
