@@ -255,7 +255,9 @@ __global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParam
     v[4 * i] = t4.x; v[4 * i + 1] = t4.y; v[4 * i + 2] = t4.z; v[4 * i + 3] = t4.w;
   }
   __syncthreads();
-  zero_hist<THREADS>(hist, kHistBins);
+  // two cleared histograms: pass 1 uses the first, pass 2 the second (no clear + barrier in between)
+  constexpr int kHist2 = (kTileThreads * PITCH >= 2 * kHistBins + 64) ? kHistBins + 64 : 0;
+  zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
   __syncthreads();
 
   // ---- canonicalise (-0 -> +0, NaN -> quiet NaN, masked -> NaN) + pass 1 -------------
@@ -296,16 +298,19 @@ __global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParam
       lo_bits = (h1.bin << 20) | (neg ? 0x000fffffu : 0u);
     } else {
       // ---- pass 2: bits[19:8] of the elements in bin h1 -----------------------------
-      zero_hist<THREADS>(hist, kHistBins);
-      __syncthreads();
+      unsigned* hist2 = smem + kHist2;
+      if (!kHist2) {
+        zero_hist<THREADS>(hist, kHistBins);
+        __syncthreads();
+      }
       const unsigned p1 = h1.bin;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
         const unsigned u = __float_as_uint(v[i]);
-        if ((u >> 20) == p1) atomicAdd(&hist[(u >> 8) & 0xfffu], 1u);
+        if ((u >> 20) == p1) atomicAdd(&hist2[(u >> 8) & 0xfffu], 1u);
       }
       __syncthreads();
-      const BinHit h2 = find_bin<kHistBins, THREADS>(smem, rem, neg ? kAscending : kDescending);
+      const BinHit h2 = find_bin<kHistBins, THREADS>(hist2, rem, neg ? kAscending : kDescending);
       rem -= h2.above;
       const unsigned p2 = (p1 << 12) | h2.bin;     // bits[31:8]
       if (rem == h2.cnt) {
