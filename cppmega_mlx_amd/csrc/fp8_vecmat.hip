@@ -168,6 +168,120 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const VecmatParam
   }
 }
 
+// M <= 4 bf16 activations, K a multiple of 4096 up to 16384: the streaming kernel.
+//   * activations stay in registers as packed bf16 pairs;
+//   * weights go e4m3 -> bf16 pairs two bytes per instruction (exact) and meet
+//     the activations in v_dot2_f32_bf16, fp32 accumulation;
+//   * rows are processed in groups of U with the loads of the next group issued
+//     before the arithmetic of the current one (two register buffers);
+//   * per row: DPP wavefront reduction, then a fixed-order 4-way LDS combine.
+constexpr int kStreamRows = 16;
+
+__device__ __forceinline__ float wave_total_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+template <int M, int CH, int U>
+struct StreamBuf {
+  uint4 w[U][CH];
+  float sc[U][CH];
+};
+
+template <int M, int CH, int U>
+__global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const VecmatParams p) {
+  constexpr int R = kStreamRows, G = R / U;
+  static_assert(G % 2 == 0, "row groups come in pairs");
+  __shared__ float red[kGemvWaves][R][M];
+  const int lane = lane_id();
+  const int wave = (int)(threadIdx.x >> 6);
+  const int K = p.k;
+  const int row0 = (int)blockIdx.x * R;
+  const int last_row = p.n - 1;
+
+  int koff[CH];
+  bf16x2 xp[M][CH][8];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    koff[c] = (c * kGemvWaves + wave) * kChunk + lane * 16;
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + koff[c]);
+      const uint4 a = src[0], b = src[1];
+      const unsigned wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xp[m][c][i] = __builtin_bit_cast(bf16x2, wds[i]);
+    }
+  }
+
+  auto load = [&](StreamBuf<M, CH, U>& buf, int g) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int n = min(row0 + g * U + u, last_row);
+      const unsigned char* wrow = p.w + (size_t)n * K;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        buf.w[u][c] = *reinterpret_cast<const uint4*>(wrow + koff[c]);
+        buf.sc[u][c] = wscale(p, n, koff[c] >> 7);
+      }
+    }
+  };
+  auto compute = [&](const StreamBuf<M, CH, U>& buf, int g) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float acc[M];
+#pragma unroll
+      for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const unsigned wds[4] = {buf.w[u][c].x, buf.w[u][c].y, buf.w[u][c].z, buf.w[u][c].w};
+        bf16x2 wp[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          wp[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, false);
+          wp[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, true);
+        }
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          float part = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) part = __builtin_amdgcn_fdot2_f32_bf16(wp[i], xp[m][c][i], part, false);
+          acc[m] = fmaf(buf.sc[u][c], part, acc[m]);
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const float s = wave_total_dpp(acc[m]);
+        if (lane == 0) red[wave][g * U + u][m] = s;
+      }
+    }
+  };
+
+  StreamBuf<M, CH, U> a, b;
+  load(a, 0);
+#pragma unroll
+  for (int g = 0; g < G; g += 2) {
+    load(b, g + 1);
+    compute(a, g);
+    if (g + 2 < G) load(a, g + 2);
+    compute(b, g + 1);
+  }
+  __syncthreads();
+  const int t = (int)threadIdx.x;
+  if (t < R * M) {
+    const int r = t / M, m = t % M;
+    if (row0 + r <= last_row) {
+      const float s = ((red[0][r][m] + red[1][r][m]) + red[2][r][m]) + red[3][r][m];
+      store_as(p.out, (size_t)m * p.n + row0 + r, p.out_dtype, s);
+    }
+  }
+}
+
 // Any shape: one wavefront per output row, all M activations in turn.
 __global__ __launch_bounds__(256) void rowwise_kernel(const VecmatParams p) {
   const int lane = lane_id();
@@ -232,7 +346,23 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   const size_t xelt = (size_t)dtype_size(a.x_dtype);
   const bool aligned = (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) &&
                        (((size_t)a.k * xelt) % 16 == 0);
-  if (a.m == 1 && aligned) {
+  const bool stream_ok = aligned && a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 4096 == 0) && a.k <= 16384;
+  if (stream_ok) {
+    const dim3 grid((unsigned)((a.n + kStreamRows - 1) / kStreamRows)), block(kGemvWaves * 64);
+    const int ch = a.k / 4096;
+#define CM_STREAM(M, U)                                                                             \
+  do {                                                                                              \
+    if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, U>), grid, block, 0, stream, p);      \
+    else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, U>), grid, block, 0, stream, p); \
+    else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, U>), grid, block, 0, stream, p); \
+    else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, U>), grid, block, 0, stream, p);              \
+  } while (0)
+    if (a.m == 1) CM_STREAM(1, 4);
+    else if (a.m == 2) CM_STREAM(2, 2);
+    else if (a.m == 3) CM_STREAM(3, 2);
+    else CM_STREAM(4, 2);
+#undef CM_STREAM
+  } else if (a.m == 1 && aligned) {
     // rows per workgroup: keep at least ~3 workgroups per CU in the grid
     int rows = 16;
     while (rows > 4 && (a.n + rows - 1) / rows < 768) rows >>= 1;
