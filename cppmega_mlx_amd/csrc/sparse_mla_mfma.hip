@@ -1,10 +1,604 @@
-// Head-batched MFMA sparse-MLA kernel (placeholder until the kernel lands).
+// Sparse MLA forward on the matrix cores (gfx950): 32 heads share one gathered
+// latent KV stream.
+//
+// Shapes served: d_qk = 576 = 512 latent + 64 rope, d_v = 512, bf16 queries;
+// the latent is e4m3 with one fp32 scale per 128 channels (or per row) plus a
+// bf16 rope tail, or a packed bf16 row of 576.  Everything else goes to the
+// scalar kernel.
+//
+// Decomposition
+//   workgroup = (batch*query, group of 32 heads, key split); 4 wavefronts.
+//   Each wavefront owns all 32 heads for its own interleaved stream of 16-key
+//   tiles, so wavefronts never synchronise inside the key loop; their partial
+//   results are merged once at the end through LDS, and the key splits of a
+//   query are merged by a second, small kernel.
+//
+// Per tile (16 gathered keys)
+//   stage   the 16 rows (fetched one tile ahead into registers) go e4m3 -> bf16
+//           with their block scale (two bytes per instruction when the scale is
+//           a power of two, an fp32 multiply otherwise) into a swizzled
+//           [16][576] bf16 tile private to the wavefront;
+//   QK^T    S^T[16 keys x 32 heads] = K . Q^T as 2 x 18 v_mfma_f32_16x16x32_bf16;
+//           K fragments are 16-byte LDS reads, Q^T fragments stay in registers
+//           for the whole kernel (144 VGPRs);
+//   softmax base-2, running max updated lazily (only when it grows by more
+//           than 2^8), so the 256 accumulator registers are rescaled rarely;
+//   P.V     O^T[512 x 32 heads] += V^T . P^T as 16 v_mfma_f32_32x32x16_bf16;
+//           V^T fragments come from the same tile through the LDS transpose
+//           read (ds_read_b64_tr_b16); P^T goes from the S^T accumulators to
+//           the B operand with one v_permlane16_swap, never through memory.
+
 #include "sparse_mla_common.h"
+
 namespace cm {
-bool sparse_mla_mfma_supported(const MlaParams&) { return false; }
-size_t sparse_mla_mfma_workspace_bytes(const MlaParams&) { return 0; }
-void sparse_mla_mfma_plan(MlaParams&) {}
-int sparse_mla_mfma_launch(const MlaParams&, hipStream_t) {
-  return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla: MFMA kernel not built");
+namespace {
+
+constexpr int kLat = 512;          // latent channels (= d_v)
+constexpr int kRope = 64;
+constexpr int kDqk = kLat + kRope; // 576
+constexpr int kTile = 16;          // keys per tile
+constexpr int kRowBytes = kDqk * 2;             // 1152: one bf16 key row in LDS
+constexpr int kTileBytes = kTile * kRowBytes;   // 18432: the bf16 tile of a wavefront
+constexpr int kRawLat = kTile * kLat;           // 8192: the same 16 rows as fetched (e4m3)
+constexpr int kRawRope = kTile * kRope * 2;     // 2048
+constexpr int kMaxBlocks = 8;                   // scale blocks per row the raw area holds
+constexpr int kRawScale = kTile * kMaxBlocks * 4;   // 512
+constexpr int kWaveBytes = kTileBytes + kRawLat + kRawRope + kRawScale;   // 29184 per wavefront
+constexpr int kHeads = 32;         // heads per workgroup
+constexpr int kWaves = 4;
+constexpr int kKSteps = kDqk / 32; // 18 MFMA k-steps of 32 channels
+constexpr int kXPitch = 260;       // floats per head row of the merge buffer (256 + 4 pad)
+constexpr int kXBytes = kWaves * kHeads * kXPitch * 4;    // 133120
+constexpr int kStatOff = kXBytes;                         // [4 waves][32 heads][2] floats
+constexpr int kSmemBytes = kXBytes + kWaves * kHeads * 2 * 4;
+static_assert(kWaves * kWaveBytes <= kXBytes, "the merge buffer reuses the tile area");
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kLazy = 8.0f;      // rescale when the running max grows by more than 2^8
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void glb_void;
+
+// 16-byte chunk q of row r lives at chunk (q with its low 3 bits xor f(r)):
+// 8 consecutive rows hit 8 different bank groups for the same q (16-byte
+// fragment reads), and 4 consecutive rows x 2 adjacent chunks hit all 8
+// (transpose reads).
+__device__ __forceinline__ int swz(int q, int r) {
+  const int f = ((r & 3) << 1) | ((r >> 2) & 1);
+  return (q & ~7) | ((q & 7) ^ f);
 }
+
+__device__ __forceinline__ bf16x8 lds_read_b128(const unsigned char* base, int byte_off) {
+  return *reinterpret_cast<const bf16x8*>(base + byte_off);
+}
+
+__device__ __forceinline__ bf16x4 lds_read_tr16_b64(const unsigned char* addr) {
+  typedef __attribute__((ext_vector_type(4))) short s16x4;
+  const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)addr);
+  return __builtin_bit_cast(bf16x4, v);
+}
+
+__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
+  // round-to-nearest-even; inputs are finite and non-negative probabilities or dequantised values
+  typedef __attribute__((ext_vector_type(2))) __bf16 v2;
+  v2 r;
+  r[0] = (__bf16)a;
+  r[1] = (__bf16)b;
+  return __builtin_bit_cast(unsigned, r);
+}
+
+__device__ __forceinline__ bool scale_is_pow2(float s) {
+  const unsigned u = __float_as_uint(s);
+  const unsigned e = u >> 23;                 // sign + exponent
+  return (u & 0x007fffffu) == 0u && e >= 1u && e <= 254u;
+}
+
+// 16 e4m3 bytes * scale -> 16 bf16 (two 16-byte LDS chunks)
+__device__ __forceinline__ void dequant16(const uint4 raw, float scale, uint4& lo, uint4& hi) {
+  const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+  unsigned o[8];
+  if (scale_is_pow2(scale)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[i], scale, false));
+      o[2 * i + 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[i], scale, true));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x2 a = e4m3x2_lo(w[i]), b = e4m3x2_hi(w[i]);
+      o[2 * i] = pack_bf16(a[0] * scale, a[1] * scale);
+      o[2 * i + 1] = pack_bf16(b[0] * scale, b[1] * scale);
+    }
+  }
+  lo = make_uint4(o[0], o[1], o[2], o[3]);
+  hi = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+// KV_FP8: latent e4m3 + fp32 scales (+ bf16 rope tail); otherwise a bf16 row of 576 (or 512 + rope tail)
+template <bool KV_FP8>
+__global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const MlaParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  unsigned char* tile = smem + wave * kWaveBytes;
+  unsigned char* raw_lat = tile + kTileBytes;
+  unsigned char* raw_rope = raw_lat + kRawLat;
+  unsigned char* raw_sc = raw_rope + kRawRope;
+
+  // ---- which (query, head group, split) ------------------------------------
+  const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
+  const int hg = (int)blockIdx.x % (p.G * groups_per_kv);
+  const size_t bs = blockIdx.x / (p.G * groups_per_kv);          // b*S + s
+  const int split = (int)blockIdx.y;
+  const int g = hg / groups_per_kv;
+  const int head0 = g * p.heads_per_group + (hg % groups_per_kv) * kHeads;
+  const int heads_here = min(kHeads, (g + 1) * p.heads_per_group - head0);
+  const int b = (int)(bs / p.S);
+  const size_t idx_base = (bs * p.G + g) * (size_t)p.topk;
+  const int key_begin = split * p.keys_per_split;
+  const int key_end = min(p.topk, key_begin + p.keys_per_split);
+  const int n_tiles = (key_end - key_begin + kTile - 1) / kTile;  // tiles of this split
+
+  // ---- Q^T fragments: lane (head n = lane%16, kq = lane/16) for both head halves ----
+  bf16x8 qf[2][kKSteps];
+  {
+    const int n = lane & 15, kq = lane >> 4;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int h = hh * 16 + n;
+      const bool live = h < heads_here;
+      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (live ? h : 0)) * (size_t)kDqk;
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        uint4 t = make_uint4(0, 0, 0, 0);
+        if (live) t = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * kq);
+        qf[hh][ks] = __builtin_bit_cast(bf16x8, t);
+      }
+    }
+  }
+
+  f32x16 o[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) o[i][j] = 0.0f;
+  float m_run[2] = {-INFINITY, -INFINITY};   // base-2 running reference of heads (lane%16) and 16+(lane%16)
+  float l_run[2] = {0.0f, 0.0f};             // this lane's share of the denominators
+  const float qk_scale = p.sm_scale * kLog2e;
+
+  // ---- staging ---------------------------------------------------------------------
+  // The gathered rows travel HBM -> LDS by the load unit itself (no registers are held
+  // while they are in flight): lane l of a 16-byte load instruction lands at base + 16*l.
+  //   latent : instruction it (0..7) carries rows 2it, 2it+1  (32 lanes x 16 bytes each)
+  //   rope   : instruction it (0..1) carries rows 8it .. 8it+7 (8 lanes x 16 bytes each)
+  //   scales : one 4-byte load per (row, block)
+  // A lane whose row is invalid issues nothing; what the raw area holds there is finite
+  // (zeroed at start, later only real rows) and meets a zero probability.
+  const int nblk = KV_FP8 ? (p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK ? kLat / p.kv_scale_block : 1) : 1;
+  const bool has_scale = KV_FP8 && p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;
+
+  auto key_row = [&](int key_pos) -> int {       // cache row of list position key_pos, or -1
+    if (key_pos >= key_end) return -1;
+    const long long k = load_index(p, idx_base + key_pos);
+    return (k >= 0 && k < p.Skv) ? (int)k : -1;
+  };
+  const int my_tiles = n_tiles > wave ? (n_tiles - wave + kWaves - 1) / kWaves : 0;
+  auto tile_key = [&](int t) -> int {            // lane l reports key (l % 16) of tile t
+    return t < my_tiles ? key_row(key_begin + (t * kWaves + wave) * kTile + (lane & 15)) : -1;
+  };
+  auto issue_dma = [&](int keyv) {                // keyv: this lane's tile_key() of the tile to fetch
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int r = __shfl(keyv, 2 * it + (lane >> 5), 64);
+      if (r >= 0) {
+        const size_t krow = ((size_t)b * p.Skv + (size_t)r) * p.G + g;
+        const unsigned char* src = (const unsigned char*)p.kv + krow * kLat + (lane & 31) * 16;
+        __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_lat + it * 1024), 16, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int r = __shfl(keyv, 8 * it + (lane >> 3), 64);
+      if (r >= 0) {
+        const size_t krow = ((size_t)b * p.Skv + (size_t)r) * p.G + g;
+        const unsigned short* src = (const unsigned short*)p.rope + krow * kRope + (lane & 7) * 8;
+        __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_rope + it * 1024), 16, 0, 0);
+      }
+    }
+    if (has_scale) {
+      for (int e0 = 0; e0 < kTile * nblk; e0 += 64) {   // uniform trip count (1 or 2)
+        const int e = e0 + lane;
+        const int r = __shfl(keyv, (e / nblk) & 15, 64);
+        if (e < kTile * nblk && r >= 0) {
+          const size_t krow = ((size_t)b * p.Skv + (size_t)r) * p.G + g;
+          const float* src = (const float*)p.kv_scale + krow * nblk + (e % nblk);
+          __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_sc + e0 * 4), 4, 0, 0);
+        }
+      }
+    }
+  };
+  auto stage = [&]() {                            // raw rows -> swizzled bf16 tile
+    const int c = lane & 31;
+    const int blk = (c * 16) / (kLat / nblk);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int r = 2 * it + (lane >> 5);
+      const uint4 raw = *reinterpret_cast<const uint4*>(raw_lat + it * 1024 + lane * 16);
+      const float sc = has_scale ? *reinterpret_cast<const float*>(raw_sc + (r * nblk + blk) * 4) : 1.0f;
+      uint4 lo, hi;
+      dequant16(raw, sc, lo, hi);
+      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c, r) * 16) = lo;
+      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c + 1, r) * 16) = hi;
+    }
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int r = 8 * it + (lane >> 3);
+      const uint4 v = *reinterpret_cast<const uint4*>(raw_rope + it * 1024 + lane * 16);
+      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + (lane & 7), r) * 16) = v;
+    }
+  };
+  // bf16 carrier rows are copied through registers (16 rows x 1152 bytes), not pipelined
+  auto stage_bf16 = [&](int keyv) {
+#pragma unroll 1
+    for (int r = 0; r < kTile; ++r) {
+      const int row = __shfl(keyv, r, 64);
+      const size_t krow = row >= 0 ? ((size_t)b * p.Skv + (size_t)row) * p.G + g : 0;
+      const unsigned short* src = (const unsigned short*)p.kv + krow * (size_t)p.d_kv;
+      for (int c = lane; c < kDqk / 8; c += 64) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (row >= 0) {
+          if (c * 8 < p.d_kv) v = *reinterpret_cast<const uint4*>(src + c * 8);
+          else v = *reinterpret_cast<const uint4*>((const unsigned short*)p.rope + krow * kRope + (c * 8 - p.d_kv));
+        }
+        *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(c, r) * 16) = v;
+      }
+    }
+  };
+
+  if (KV_FP8) {                                   // the raw area starts out as zeros
+    for (int i = lane; i < (kRawLat + kRawRope + kRawScale) / 16; i += 64)
+      reinterpret_cast<uint4*>(raw_lat)[i] = make_uint4(0, 0, 0, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  // software pipeline: tile t+1 is in flight to the raw area, and the keys of tile t+2
+  // are being read, while tile t computes
+  int key_cur = tile_key(0);
+  int key_nxt = tile_key(1);
+  if (KV_FP8 && my_tiles > 0) issue_dma(key_cur);
+
+  for (int t = 0; t < my_tiles; ++t) {
+    const unsigned vmask = (unsigned)(__ballot(key_cur >= 0) & 0xffffull);
+    if (KV_FP8) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // tile t has landed in the raw area
+      stage();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // raw area fully read before it is refilled
+      if (t + 1 < my_tiles) issue_dma(key_nxt);
+    } else {
+      stage_bf16(key_cur);
+    }
+    key_cur = key_nxt;
+    key_nxt = tile_key(t + 2);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (vmask == 0u) continue;                    // nothing to attend to in this tile (uniform)
+
+    // ---- S^T = K . Q^T ------------------------------------------------------------
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    {
+      const int m = lane & 15, kq = lane >> 4;
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        const bf16x8 a = lds_read_b128(tile, m * kRowBytes + swz(4 * ks + kq, m) * 16);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[0][ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[1][ks], s1, 0, 0, 0);
+      }
+    }
+    // lane (n = lane%16, gq = lane/16) holds keys 4*gq + i of heads n (s0) and 16+n (s1)
+    const int gq = lane >> 4;
+    float sv[2][4];
+    float mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = (vmask >> (4 * gq + i)) & 1u;
+      sv[0][i] = ok ? s0[i] * qk_scale : -INFINITY;
+      sv[1][i] = ok ? s1[i] * qk_scale : -INFINITY;
+      mx[0] = fmaxf(mx[0], sv[0][i]);
+      mx[1] = fmaxf(mx[1], sv[1][i]);
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      mx[hh] = fmaxf(mx[hh], __shfl_xor(mx[hh], 16, 64));
+      mx[hh] = fmaxf(mx[hh], __shfl_xor(mx[hh], 32, 64));
+    }
+    // lazy running reference: move it only when the tile maximum exceeds it by more than kLazy
+    const bool grow = (mx[0] > m_run[0] + kLazy) || (mx[1] > m_run[1] + kLazy);
+    if (__ballot(grow) != 0ull) {
+      float fac[2];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const float m_new = (mx[hh] > m_run[hh] + kLazy) ? mx[hh] : m_run[hh];
+        fac[hh] = (m_run[hh] == -INFINITY) ? 0.0f : exp2f(m_run[hh] - m_new);
+        l_run[hh] *= fac[hh];
+        m_run[hh] = m_new;
+      }
+      // accumulator lane l carries head l%32: half (l & 16)
+      const float fo = (lane & 16) ? fac[1] : fac[0];
+      if (__ballot(fo != 1.0f) != 0ull) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) o[i][j] *= fo;
+      }
+    }
+    unsigned pk[2][2];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      float pr[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pr[i] = exp2f(sv[hh][i] - m_run[hh]);      // -inf -> 0; m_run is finite once any key was valid
+        l_run[hh] += pr[i];
+      }
+      pk[hh][0] = pack_bf16(pr[0], pr[1]);
+      pk[hh][1] = pack_bf16(pr[2], pr[3]);
+    }
+    // P^T as the B operand of 32x32x16: lane (head = lane%32, kq = lane/32) needs keys 8kq..8kq+7
+    bf16x8 pb;
+    {
+      const u32x2 w0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
+      const u32x2 w1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
+      const uint4 packed = make_uint4(w0[0], w1[0], w0[1], w1[1]);
+      pb = __builtin_bit_cast(bf16x8, packed);
+    }
+    // ---- O^T += V^T . P^T ---------------------------------------------------------
+    {
+      const int i16 = lane & 15;
+      const int col_half = (lane >> 4) & 1;       // columns +0..15 or +16..31 of the 32-wide block
+      const int kq = lane >> 5;
+      const int r0 = 8 * kq + (i16 >> 2);         // first transpose read: rows 8kq .. 8kq+3
+      const int r1 = r0 + 4;                      // second: rows 8kq+4 .. 8kq+7
+      const int cin = (i16 & 3) * 4;              // 4 columns of the 16 this lane group covers
+#pragma unroll
+      for (int db = 0; db < 16; ++db) {
+        const int col = 32 * db + 16 * col_half + cin;   // bf16 column of the value
+        const int q = col >> 3, inner = (col & 7) * 2;
+        const bf16x4 a0 = lds_read_tr16_b64(tile + r0 * kRowBytes + swz(q, r0) * 16 + inner);
+        const bf16x4 a1 = lds_read_tr16_b64(tile + r1 * kRowBytes + swz(q, r1) * 16 + inner);
+        bf16x8 a;
+        a[0] = a0[0]; a[1] = a0[1]; a[2] = a0[2]; a[3] = a0[3];
+        a[4] = a1[0]; a[5] = a1[1]; a[6] = a1[2]; a[7] = a1[3];
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, o[db], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- merge the four wavefronts ----------------------------------------------------
+  // denominators: a head's share is spread over lanes n, n+16, n+32, n+48
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {
+    l_run[hh] += __shfl_xor(l_run[hh], 16, 64);
+    l_run[hh] += __shfl_xor(l_run[hh], 32, 64);
+  }
+  __syncthreads();                               // every wavefront is done with its tile
+  float* stats = reinterpret_cast<float*>(smem + kStatOff);
+  if (lane < 16) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      stats[(wave * kHeads + hh * 16 + lane) * 2 + 0] = m_run[hh];
+      stats[(wave * kHeads + hh * 16 + lane) * 2 + 1] = l_run[hh];
+    }
+  }
+  __syncthreads();
+  // accumulator lane carries head hd = lane%32
+  const int hd = lane & 31;
+  float m_all = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) m_all = fmaxf(m_all, stats[(w * kHeads + hd) * 2]);
+  float l_all = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    const float mw = stats[(w * kHeads + hd) * 2];
+    l_all += (mw == -INFINITY) ? 0.0f : stats[(w * kHeads + hd) * 2 + 1] * exp2f(mw - m_all);
+  }
+  {
+    const float mine = stats[(wave * kHeads + hd) * 2];
+    const float f = (mine == -INFINITY) ? 0.0f : exp2f(mine - m_all);
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) o[i][j] *= f;
+  }
+
+  // final scale for a single-split launch: fold the sink in and normalise
+  float out_scale = 1.0f, lse_val = 0.0f;
+  const bool direct = p.num_splits == 1;
+  if (direct) {
+    float m_fin = m_all, l_fin = l_all;
+    if (p.sinks && hd < heads_here) {
+      const float sk = p.sinks[head0 + hd] * kLog2e;
+      const float m2 = fmaxf(m_fin, sk);
+      const float keep = (m_fin == -INFINITY) ? 0.0f : exp2f(m_fin - m2);
+      l_fin = l_fin * keep + exp2f(sk - m2);
+      out_scale = keep;
+      m_fin = m2;
+    }
+    if (l_fin > 0.0f) {
+      out_scale = out_scale / l_fin;
+      lse_val = (m_fin + log2f(l_fin)) * kLn2;
+    } else {
+      out_scale = 0.0f;
+    }
+  }
+
+  float* xbuf = reinterpret_cast<float*>(smem);
+  const size_t q_index = bs;                     // b*S + s
+  // two rounds of 256 value channels each
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    __syncthreads();
+    // writer: lane (head hd, gq = lane/32) holds channels 32*db + 8*j + 4*gq + (0..3) in o[db][4j..4j+3]
+    {
+      const int gq2 = lane >> 5;
+#pragma unroll
+      for (int dbl = 0; dbl < 8; ++dbl) {
+        const int db = half * 8 + dbl;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int ch = 32 * dbl + 8 * j + 4 * gq2;      // channel within this half
+          float4 v = make_float4(o[db][4 * j], o[db][4 * j + 1], o[db][4 * j + 2], o[db][4 * j + 3]);
+          *reinterpret_cast<float4*>(xbuf + (wave * kHeads + hd) * kXPitch + ch) = v;
+        }
+      }
+    }
+    __syncthreads();
+    // reader: wavefront w sums heads 8w..8w+7; lane = 4 consecutive channels
+#pragma unroll
+    for (int hh = 0; hh < 8; ++hh) {
+      const int h = wave * 8 + hh;
+      if (h >= heads_here) break;                // uniform
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float4 v = *reinterpret_cast<const float4*>(xbuf + (w * kHeads + h) * kXPitch + lane * 4);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+      }
+      const int ch = half * 256 + lane * 4;
+      if (direct) {
+        const float sc = __shfl(out_scale, h, 64);   // lane h carries head h
+        const size_t off = (q_index * p.H + head0 + h) * (size_t)kLat + ch;
+        if (p.out_dtype == CPPMEGA_MI355_F32) {
+          *reinterpret_cast<float4*>((float*)p.out + off) = make_float4(acc.x * sc, acc.y * sc, acc.z * sc, acc.w * sc);
+        } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
+          *reinterpret_cast<uint2*>((unsigned short*)p.out + off) =
+              make_uint2(pack_bf16(acc.x * sc, acc.y * sc), pack_bf16(acc.z * sc, acc.w * sc));
+        } else {
+          unsigned short* dst = (unsigned short*)p.out + off;
+          dst[0] = f32_to_f16_bits(acc.x * sc); dst[1] = f32_to_f16_bits(acc.y * sc);
+          dst[2] = f32_to_f16_bits(acc.z * sc); dst[3] = f32_to_f16_bits(acc.w * sc);
+        }
+      } else {
+        // partial: [query][head][split][512] fp32
+        float* part = (float*)p.workspace + ((q_index * p.H + head0 + h) * (size_t)p.num_splits + split) * kLat + ch;
+        *reinterpret_cast<float4*>(part) = acc;
+      }
+    }
+  }
+  if (wave == 0 && lane < heads_here) {
+    if (direct) {
+      if (p.lse) p.lse[q_index * p.H + head0 + lane] = lse_val;
+    } else {
+      float* ml = (float*)p.workspace + (size_t)p.B * p.S * p.H * p.num_splits * kLat +
+                  ((q_index * p.H + head0 + lane) * (size_t)p.num_splits + split) * 2;
+      ml[0] = m_all;
+      ml[1] = l_all;
+    }
+  }
+}
+
+// Merges the key splits of every (query, head): one wavefront per (query, head).
+__global__ __launch_bounds__(256) void sparse_mla_combine_kernel(const MlaParams p) {
+  const int lane = lane_id();
+  const size_t qh = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (qh >= (size_t)p.B * p.S * p.H) return;
+  const int h = (int)(qh % p.H);
+  const float* part = (const float*)p.workspace + qh * (size_t)p.num_splits * kLat;
+  const float* ml = (const float*)p.workspace + (size_t)p.B * p.S * p.H * p.num_splits * kLat + qh * (size_t)p.num_splits * 2;
+  float m_all = -INFINITY;
+  for (int s = 0; s < p.num_splits; ++s) m_all = fmaxf(m_all, ml[2 * s]);
+  float m_fin = m_all;
+  float sink_term = 0.0f;
+  if (p.sinks) {
+    const float sk = p.sinks[h] * kLog2e;
+    m_fin = fmaxf(m_all, sk);
+    sink_term = exp2f(sk - m_fin);
+  }
+  float l_fin = sink_term;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+  for (int s = 0; s < p.num_splits; ++s) {
+    const float ms = ml[2 * s];
+    if (ms == -INFINITY) continue;
+    const float f = exp2f(ms - m_fin);
+    l_fin += ml[2 * s + 1] * f;
+    const float4 a = *reinterpret_cast<const float4*>(part + (size_t)s * kLat + lane * 8);
+    const float4 c = *reinterpret_cast<const float4*>(part + (size_t)s * kLat + lane * 8 + 4);
+    acc[0] += a.x * f; acc[1] += a.y * f; acc[2] += a.z * f; acc[3] += a.w * f;
+    acc[4] += c.x * f; acc[5] += c.y * f; acc[6] += c.z * f; acc[7] += c.w * f;
+  }
+  const float inv = l_fin > 0.0f ? 1.0f / l_fin : 0.0f;
+  const size_t off = qh * (size_t)kLat + lane * 8;
+  if (p.out_dtype == CPPMEGA_MI355_BF16) {
+    *reinterpret_cast<uint4*>((unsigned short*)p.out + off) =
+        make_uint4(pack_bf16(acc[0] * inv, acc[1] * inv), pack_bf16(acc[2] * inv, acc[3] * inv),
+                   pack_bf16(acc[4] * inv, acc[5] * inv), pack_bf16(acc[6] * inv, acc[7] * inv));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) store_as(p.out, off + i, p.out_dtype, acc[i] * inv);
+  }
+  if (p.lse && lane == 0) p.lse[qh] = l_fin > 0.0f ? (m_fin + log2f(l_fin)) * kLn2 : 0.0f;
+}
+
+}  // namespace
+
+bool sparse_mla_mfma_supported(const MlaParams& p) {
+  if (p.q_dtype != CPPMEGA_MI355_BF16 || p.q_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
+  if (p.d_qk != kDqk || p.d_v != kLat) return false;
+  if (p.rope_dim != 0 && (p.rope_dim != kRope || p.rope_dtype != CPPMEGA_MI355_BF16)) return false;
+  if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
+    if (p.rope_dim != kRope || p.d_kv != kLat) return false;
+    if (p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK) {
+      if (p.kv_scale_block < kLat / kMaxBlocks || kLat % p.kv_scale_block != 0) return false;
+    } else if (p.kv_scale_kind != CPPMEGA_MI355_SCALE_PER_TOKEN && p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE) {
+      return false;
+    }
+  } else if (p.kv_dtype == CPPMEGA_MI355_BF16) {
+    if (p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
+    if (p.d_kv + p.rope_dim != kDqk) return false;
+  } else {
+    return false;
+  }
+  if (p.topk < 1 || (size_t)p.B * p.S == 0) return false;
+  // pointers must allow 16-byte loads
+  if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
+  return true;
+}
+
+// Chooses the key-split factor: enough workgroups to cover the 256 CUs, at least 64 keys per wavefront.
+void sparse_mla_mfma_plan(MlaParams& p) {
+  const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
+  const long long base = (long long)p.B * p.S * p.G * groups_per_kv;
+  int splits = 1;
+  while (base * splits < 256 && p.topk / (splits * 2) >= kWaves * 64 && splits < 16) splits *= 2;
+  p.num_splits = splits;
+  const int tiles = (p.topk + kTile - 1) / kTile;
+  const int tiles_per_split = (tiles + splits - 1) / splits;
+  p.keys_per_split = tiles_per_split * kTile;
+}
+
+size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p) {
+  if (p.num_splits <= 1) return 0;
+  return (size_t)p.B * p.S * p.H * p.num_splits * (kLat + 2) * sizeof(float);
+}
+
+int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
+  const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
+  const dim3 grid((unsigned)((size_t)p.B * p.S * p.G * groups_per_kv), (unsigned)p.num_splits), block(kWaves * 64);
+  if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_mfma_kernel<true>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
+    hipLaunchKernelGGL(sparse_mla_mfma_kernel<true>, grid, block, kSmemBytes, stream, p);
+  } else {
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_mfma_kernel<false>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
+    hipLaunchKernelGGL(sparse_mla_mfma_kernel<false>, grid, block, kSmemBytes, stream, p);
+  }
+  CM_HIP_CHECK(hipGetLastError());
+  if (p.num_splits > 1) {
+    const size_t qh = (size_t)p.B * p.S * p.H;
+    hipLaunchKernelGGL(sparse_mla_combine_kernel, dim3((unsigned)((qh + 3) / 4)), dim3(256), 0, stream, p);
+    CM_HIP_CHECK(hipGetLastError());
+  }
+  return 0;
+}
+
 }  // namespace cm
