@@ -78,6 +78,28 @@ __device__ __forceinline__ bf16x4 lds_read_tr16_b64(const unsigned char* addr) {
   return __builtin_bit_cast(bf16x4, v);
 }
 
+// The two MFMA shapes as inline assembly with fixed register classes.  The
+// 32 x 512 fp32 output accumulators fill all 256 accumulation registers (AGPRs);
+// the small score accumulators therefore have to live in ordinary VGPRs, which
+// the builtin form of the instruction cannot express once a kernel uses AGPRs.
+// Dependent MFMAs on the same accumulator are interlocked by the hardware; a
+// VALU read of a result is not, hence mfma_settle().
+__device__ __forceinline__ void mfma_qk(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_pv(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// wait states between the last MFMA writing these registers and the first non-MFMA use
+__device__ __forceinline__ void mfma_settle(f32x4& s0, f32x4& s1) {
+  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(s0), "+v"(s1));
+}
+__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[16]) {
+  asm volatile("s_nop 15\n\ts_nop 7"
+               : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]),
+                 "+a"(o[8]), "+a"(o[9]), "+a"(o[10]), "+a"(o[11]), "+a"(o[12]), "+a"(o[13]), "+a"(o[14]), "+a"(o[15]));
+}
+
 __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
   // round-to-nearest-even; inputs are finite and non-negative probabilities or dequantised values
   typedef __attribute__((ext_vector_type(2))) __bf16 v2;
@@ -187,7 +209,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     return t < my_tiles ? key_row(key_begin + (t * kWaves + wave) * kTile + (lane & 15)) : -1;
   };
   auto issue_dma = [&](int keyv) {                // keyv: this lane's tile_key() of the tile to fetch
-#pragma unroll
+#pragma unroll 1
     for (int it = 0; it < 8; ++it) {
       const int r = __shfl(keyv, 2 * it + (lane >> 5), 64);
       if (r >= 0) {
@@ -196,7 +218,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_lat + it * 1024), 16, 0, 0);
       }
     }
-#pragma unroll
+#pragma unroll 1
     for (int it = 0; it < 2; ++it) {
       const int r = __shfl(keyv, 8 * it + (lane >> 3), 64);
       if (r >= 0) {
@@ -220,7 +242,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   auto stage = [&]() {                            // raw rows -> swizzled bf16 tile
     const int c = lane & 31;
     const int blk = (c * 16) / (kLat / nblk);
-#pragma unroll
+#pragma unroll 1
     for (int it = 0; it < 8; ++it) {
       const int r = 2 * it + (lane >> 5);
       const uint4 raw = *reinterpret_cast<const uint4*>(raw_lat + it * 1024 + lane * 16);
@@ -230,7 +252,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c, r) * 16) = lo;
       *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c + 1, r) * 16) = hi;
     }
-#pragma unroll
+#pragma unroll 1
     for (int it = 0; it < 2; ++it) {
       const int r = 8 * it + (lane >> 3);
       const uint4 v = *reinterpret_cast<const uint4*>(raw_rope + it * 1024 + lane * 16);
@@ -260,6 +282,24 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       reinterpret_cast<uint4*>(raw_lat)[i] = make_uint4(0, 0, 0, 0);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
+  // lane-constant LDS offsets of the operand fragments (the swizzle leaves two variants each)
+  int qk_base0, qk_base1, pv_base0a, pv_base0b, pv_base1a, pv_base1b;
+  {
+    const int m = lane & 15, kq = lane >> 4;
+    qk_base0 = m * kRowBytes + swz(kq, m) * 16;
+    qk_base1 = m * kRowBytes + swz(4 + kq, m) * 16;
+    // transpose reads: 16-lane group g16 covers columns 16*(g16&1)..+15 of a 32-wide block and
+    // rows 8*(lane/32) + {0..3} (first read) / {4..7} (second); lane i of the group supplies
+    // row i/4, columns 4*(i%4)..+3
+    const int i16 = lane & 15, col_half = (lane >> 4) & 1, kq2 = lane >> 5;
+    const int r0 = 8 * kq2 + (i16 >> 2), r1 = r0 + 4;
+    const int col = 16 * col_half + (i16 & 3) * 4;          // column within the block
+    const int lp = col >> 3, inner = (col & 7) * 2;
+    pv_base0a = r0 * kRowBytes + swz(lp, r0) * 16 + inner;
+    pv_base0b = r0 * kRowBytes + swz(4 + lp, r0) * 16 + inner;
+    pv_base1a = r1 * kRowBytes + swz(lp, r1) * 16 + inner;
+    pv_base1b = r1 * kRowBytes + swz(4 + lp, r1) * 16 + inner;
+  }
   // software pipeline: tile t+1 is in flight to the raw area, and the keys of tile t+2
   // are being read, while tile t computes
   int key_cur = tile_key(0);
@@ -284,13 +324,14 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     // ---- S^T = K . Q^T ------------------------------------------------------------
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
     {
-      const int m = lane & 15, kq = lane >> 4;
+      // chunk 4ks+kq of row m: 128 bytes per pair of k-steps, low bits swizzled -> two lane bases
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
-        const bf16x8 a = lds_read_b128(tile, m * kRowBytes + swz(4 * ks + kq, m) * 16);
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[0][ks], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[1][ks], s1, 0, 0, 0);
+        const bf16x8 a = lds_read_b128(tile, ((ks & 1) ? qk_base1 : qk_base0) + 128 * (ks >> 1));
+        mfma_qk(s0, a, qf[0][ks]);
+        mfma_qk(s1, a, qf[1][ks]);
       }
+      mfma_settle(s0, s1);
     }
     // lane (n = lane%16, gq = lane/16) holds keys 4*gq + i of heads n (s0) and 16+n (s1)
     const int gq = lane >> 4;
@@ -323,10 +364,18 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       // accumulator lane l carries head l%32: half (l & 16)
       const float fo = (lane & 16) ? fac[1] : fac[0];
       if (__ballot(fo != 1.0f) != 0ull) {
+        mfma_settle_acc(o);
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
+        for (int i = 0; i < 16; ++i) {
+          // one 16-register block at a time: the accumulators pass through ordinary
+          // VGPRs for the multiply and only a few of those are free
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int j = 0; j < 16; ++j) o[i][j] *= fo;
+          asm volatile("" : "+a"(o[i]));      // back into the accumulation registers right away
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_settle_acc(o);
       }
     }
     unsigned pk[2][2];
@@ -350,28 +399,23 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       pb = __builtin_bit_cast(bf16x8, packed);
     }
     // ---- O^T += V^T . P^T ---------------------------------------------------------
-    {
-      const int i16 = lane & 15;
-      const int col_half = (lane >> 4) & 1;       // columns +0..15 or +16..31 of the 32-wide block
-      const int kq = lane >> 5;
-      const int r0 = 8 * kq + (i16 >> 2);         // first transpose read: rows 8kq .. 8kq+3
-      const int r1 = r0 + 4;                      // second: rows 8kq+4 .. 8kq+7
-      const int cin = (i16 & 3) * 4;              // 4 columns of the 16 this lane group covers
 #pragma unroll
-      for (int db = 0; db < 16; ++db) {
-        const int col = 32 * db + 16 * col_half + cin;   // bf16 column of the value
-        const int q = col >> 3, inner = (col & 7) * 2;
-        const bf16x4 a0 = lds_read_tr16_b64(tile + r0 * kRowBytes + swz(q, r0) * 16 + inner);
-        const bf16x4 a1 = lds_read_tr16_b64(tile + r1 * kRowBytes + swz(q, r1) * 16 + inner);
-        bf16x8 a;
-        a[0] = a0[0]; a[1] = a0[1]; a[2] = a0[2]; a[3] = a0[3];
-        a[4] = a1[0]; a[5] = a1[1]; a[6] = a1[2]; a[7] = a1[3];
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, o[db], 0, 0, 0);
-      }
+    for (int db = 0; db < 16; ++db) {
+      const int off = 128 * (db >> 1);
+      const bf16x4 a0 = lds_read_tr16_b64(tile + ((db & 1) ? pv_base0b : pv_base0a) + off);
+      const bf16x4 a1 = lds_read_tr16_b64(tile + ((db & 1) ? pv_base1b : pv_base1a) + off);
+      bf16x8 a;
+      a[0] = a0[0]; a[1] = a0[1]; a[2] = a0[2]; a[3] = a0[3];
+      a[4] = a1[0]; a[5] = a1[1]; a[6] = a1[2]; a[7] = a1[3];
+      mfma_pv(o[db], a, pb);
+      // keep the scheduler from hoisting every fragment read of the loop to its top: the
+      // query fragments need the registers
+      if ((db & 3) == 3) __builtin_amdgcn_sched_barrier(0);
     }
   }
 
   // ---- merge the four wavefronts ----------------------------------------------------
+  mfma_settle_acc(o);
   // denominators: a head's share is spread over lanes n, n+16, n+32, n+48
 #pragma unroll
   for (int hh = 0; hh < 2; ++hh) {
@@ -403,9 +447,13 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     const float mine = stats[(wave * kHeads + hd) * 2];
     const float f = (mine == -INFINITY) ? 0.0f : exp2f(mine - m_all);
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 16; ++j) o[i][j] *= f;
+      asm volatile("" : "+a"(o[i]));
+    }
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // final scale for a single-split launch: fold the sink in and normalise
