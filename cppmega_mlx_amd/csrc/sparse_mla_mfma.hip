@@ -115,19 +115,19 @@ __device__ __forceinline__ bool scale_is_pow2(float s) {
   return (u & 0x007fffffu) == 0u && e >= 1u && e <= 254u;
 }
 
-// 16 e4m3 bytes * scale -> 16 bf16 (two 16-byte LDS chunks)
+// 16 e4m3 bytes * scale -> 16 bf16 (two 16-byte LDS chunks).  POW2: the scale is a
+// normal power of two, which the converter applies exactly (it only looks at the
+// exponent of its scale operand); otherwise convert unscaled and multiply in fp32.
+template <bool POW2>
 __device__ __forceinline__ void dequant16(const uint4 raw, float scale, uint4& lo, uint4& hi) {
   const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
   unsigned o[8];
-  if (scale_is_pow2(scale)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 4; ++i) {
+    if (POW2) {
       o[2 * i] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[i], scale, false));
       o[2 * i + 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[i], scale, true));
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    } else {
       const f32x2 a = e4m3x2_lo(w[i]), b = e4m3x2_hi(w[i]);
       o[2 * i] = pack_bf16(a[0] * scale, a[1] * scale);
       o[2 * i + 1] = pack_bf16(b[0] * scale, b[1] * scale);
@@ -135,6 +135,18 @@ __device__ __forceinline__ void dequant16(const uint4 raw, float scale, uint4& l
   }
   lo = make_uint4(o[0], o[1], o[2], o[3]);
   hi = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+// value of lane (lane ^ 16) / (lane ^ 32), VALU only
+__device__ __forceinline__ float xor16(float v) {
+  const unsigned u = __float_as_uint(v);
+  const u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float((lane_id() & 16) ? r[0] : r[1]);
+}
+__device__ __forceinline__ float xor32(float v) {
+  const unsigned u = __float_as_uint(v);
+  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float((lane_id() & 32) ? r[0] : r[1]);
 }
 
 // KV_FP8: latent e4m3 + fp32 scales (+ bf16 rope tail); otherwise a bf16 row of 576 (or 512 + rope tail)
@@ -209,20 +221,28 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     return t < my_tiles ? key_row(key_begin + (t * kWaves + wave) * kTile + (lane & 15)) : -1;
   };
   auto issue_dma = [&](int keyv) {                // keyv: this lane's tile_key() of the tile to fetch
-#pragma unroll 1
+    const bool upper = lane >= 32;
+    int rows[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {              // rows 2it (lanes 0..31) and 2it+1 (lanes 32..63)
+      const int ra = __builtin_amdgcn_readlane(keyv, 2 * it), rb = __builtin_amdgcn_readlane(keyv, 2 * it + 1);
+      rows[it] = upper ? rb : ra;
+    }
+    const int rope_r0 = __shfl(keyv, lane >> 3, 64), rope_r1 = __shfl(keyv, 8 + (lane >> 3), 64);
+    const size_t row_base = (size_t)b * p.Skv;
+#pragma unroll
     for (int it = 0; it < 8; ++it) {
-      const int r = __shfl(keyv, 2 * it + (lane >> 5), 64);
-      if (r >= 0) {
-        const size_t krow = ((size_t)b * p.Skv + (size_t)r) * p.G + g;
+      if (rows[it] >= 0) {
+        const size_t krow = (row_base + (size_t)rows[it]) * p.G + g;
         const unsigned char* src = (const unsigned char*)p.kv + krow * kLat + (lane & 31) * 16;
         __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_lat + it * 1024), 16, 0, 0);
       }
     }
-#pragma unroll 1
+#pragma unroll
     for (int it = 0; it < 2; ++it) {
-      const int r = __shfl(keyv, 8 * it + (lane >> 3), 64);
+      const int r = it ? rope_r1 : rope_r0;
       if (r >= 0) {
-        const size_t krow = ((size_t)b * p.Skv + (size_t)r) * p.G + g;
+        const size_t krow = (row_base + (size_t)r) * p.G + g;
         const unsigned short* src = (const unsigned short*)p.rope + krow * kRope + (lane & 7) * 8;
         __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_rope + it * 1024), 16, 0, 0);
       }
@@ -232,7 +252,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         const int e = e0 + lane;
         const int r = __shfl(keyv, (e / nblk) & 15, 64);
         if (e < kTile * nblk && r >= 0) {
-          const size_t krow = ((size_t)b * p.Skv + (size_t)r) * p.G + g;
+          const size_t krow = (row_base + (size_t)r) * p.G + g;
           const float* src = (const float*)p.kv_scale + krow * nblk + (e % nblk);
           __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_sc + e0 * 4), 4, 0, 0);
         }
@@ -242,17 +262,31 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   auto stage = [&]() {                            // raw rows -> swizzled bf16 tile
     const int c = lane & 31;
     const int blk = (c * 16) / (kLat / nblk);
-#pragma unroll 1
-    for (int it = 0; it < 8; ++it) {
-      const int r = 2 * it + (lane >> 5);
-      const uint4 raw = *reinterpret_cast<const uint4*>(raw_lat + it * 1024 + lane * 16);
-      const float sc = has_scale ? *reinterpret_cast<const float*>(raw_sc + (r * nblk + blk) * 4) : 1.0f;
-      uint4 lo, hi;
-      dequant16(raw, sc, lo, hi);
-      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c, r) * 16) = lo;
-      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c + 1, r) * 16) = hi;
+    const int hi_row = lane >> 5;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint4 raw[4];
+      float sc[4];
+      bool all_pow2 = true;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int it = half * 4 + i;
+        raw[i] = *reinterpret_cast<const uint4*>(raw_lat + it * 1024 + lane * 16);
+        sc[i] = has_scale ? *reinterpret_cast<const float*>(raw_sc + ((2 * it + hi_row) * nblk + blk) * 4) : 1.0f;
+        all_pow2 = all_pow2 && scale_is_pow2(sc[i]);
+      }
+      const bool fast = __ballot(!all_pow2) == 0ull;      // uniform
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 2 * (half * 4 + i) + hi_row;
+        uint4 lo, hi;
+        if (fast) dequant16<true>(raw[i], sc[i], lo, hi);
+        else dequant16<false>(raw[i], sc[i], lo, hi);
+        *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c, r) * 16) = lo;
+        *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c + 1, r) * 16) = hi;
+      }
     }
-#pragma unroll 1
+#pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int r = 8 * it + (lane >> 3);
       const uint4 v = *reinterpret_cast<const uint4*>(raw_rope + it * 1024 + lane * 16);
@@ -347,8 +381,8 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     }
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
-      mx[hh] = fmaxf(mx[hh], __shfl_xor(mx[hh], 16, 64));
-      mx[hh] = fmaxf(mx[hh], __shfl_xor(mx[hh], 32, 64));
+      mx[hh] = fmaxf(mx[hh], xor16(mx[hh]));
+      mx[hh] = fmaxf(mx[hh], xor32(mx[hh]));
     }
     // lazy running reference: move it only when the tile maximum exceeds it by more than kLazy
     const bool grow = (mx[0] > m_run[0] + kLazy) || (mx[1] > m_run[1] + kLazy);
@@ -410,7 +444,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       mfma_pv(o[db], a, pb);
       // keep the scheduler from hoisting every fragment read of the loop to its top: the
       // query fragments need the registers
-      if ((db & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+      if ((db & 7) == 7) __builtin_amdgcn_sched_barrier(0);
     }
   }
 
