@@ -206,7 +206,8 @@ def bench_vecmat(args, device, M: int):
         "us_per_launch": per * 1e6,
         "algorithmic_bytes": bytes_alg,
         "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS,
+                     "traffic": measured_traffic({1: "fp8_vecmat", 4: "fp8_vecmat_m4", 16: "fp8_vecmat_m16"}.get(M, ""))},
     }
     return res, (xs[0], ws[0], ss[0], outs[0])
 
@@ -256,7 +257,7 @@ def bench_topk(args, device):
         "us_per_launch": per * 1e6,
         "algorithmic_bytes": bytes_alg,
         "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic("topk_selector")},
     }
     return res, (scores[0], ends, outs[0], k)
 
@@ -300,6 +301,28 @@ def bench_prefill(args, device):
             "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
 
 
+def bench_copy(args, device):
+    """A plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
+    counters of the other kernels are scaled by."""
+    n = 256 << 20
+    src = torch.full((n,), 7, dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    secs, _ = timed_graph([lambda: dst.copy_(src)], args.steps, args.warmup)
+    per = secs / args.steps
+    return {"workload": "torch copy_ of 256 MiB (u8)", "bytes_read": n, "bytes_written": n, "us_per_launch": per * 1e6,
+            "gbs": 2.0 * n / per / 1e9}
+
+
+def measured_traffic(name):
+    """HBM bytes per launch from the committed rocprofv3 counter runs, or None."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
+    try:
+        with open(path) as fh:
+            return json.load(fh)["workloads"][name]["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -332,7 +355,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 MFMA over e4m3 KV (fp32 accumulate)",
+        "dtype": "bf16",
         "data": "synthetic",
         "config": {},
     }
@@ -345,7 +368,7 @@ def main() -> int:
                           "algorithmic_bytes_per_step": res["algorithmic_bytes_per_step"],
                           "host_ms_per_step": res["host_ms_per_step"], "hbm_gbs": res["hbm_gbs"]}
         line["roofline"] = {"bound": "mfma", "achieved": res["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                            "frac": res["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
+                            "frac": res["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic("sparse_mla_decode")}
         if not args.no_cpu_baseline:
             cpu, rel_err = cpu_baseline_decode(sample)
             line["cpu_baseline"] = cpu
@@ -370,6 +393,8 @@ def main() -> int:
         torch.cuda.empty_cache()
     if "prefill" in parts:
         line["prefill"] = bench_prefill(args, device)
+    if "copy" in parts:
+        line["copy"] = bench_copy(args, device)
     print(json.dumps(line))
     return 0
 
