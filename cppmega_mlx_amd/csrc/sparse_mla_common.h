@@ -25,6 +25,7 @@ struct MlaParams {
   int heads_per_group;
   int num_splits;       // split-KV factor of the MFMA kernel
   int keys_per_split;
+  int heads_per_wg;     // 0: 32-head tile kernel; 64 / 128: shared-tile latent kernel
   float sm_scale;
 };
 
@@ -48,5 +49,10 @@ int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream);
 bool sparse_mla_mfma_supported(const MlaParams& p);
 size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p);
 void sparse_mla_mfma_plan(MlaParams& p);
+
+// shared-tile kernel for FP8 latent caches (sparse_mla_latent.hip); dispatched by the *_mfma_* functions
+bool sparse_mla_latent_supported(const MlaParams& p);
+void sparse_mla_latent_plan(MlaParams& p);
+int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream);
 
 }  // namespace cm

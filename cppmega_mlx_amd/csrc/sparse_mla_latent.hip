@@ -1,0 +1,630 @@
+// Sparse MLA forward over an FP8 latent KV cache on the matrix cores (gfx950):
+// 64 or 128 heads share every gathered key row.
+//
+// Shapes served: bf16 queries of 576 = 512 latent + 64 rope channels, d_v = 512,
+// keys as e4m3 latent [512] with fp32 scales (per 128 / 256 / 512 channels, or
+// per row, or none) plus a bf16 rope tail [64]; at least 33 heads per KV group.
+//
+// Workgroup = (query, KV group, chunk of 32*HG heads, key split), 4 wavefronts,
+// key tiles of 32 rows.
+//
+//   HBM -> LDS   Rows travel as raw bytes (e4m3 latent, bf16 rope, fp32 scales)
+//                straight into a ring of four LDS tile slots by the load unit
+//                (global_load_lds), three tiles ahead.  Nothing is ever
+//                rewritten in LDS: both matrix products dequantise in the
+//                operand path, in registers.  The 16-byte chunk c of row r lives
+//                at chunk c ^ (r & 7), which makes both access patterns below
+//                conflict-free; the swizzle costs nothing because each lane of
+//                a load instruction picks which source chunk it fetches.
+//   S^T = K.Q^T  Wavefront w owns 32 heads (their Q^T fragments stay in 144
+//                VGPRs) and HG/2 sub-tiles of 16 keys.  A K fragment is one
+//                16-byte LDS read of e4m3 bytes, converted to bf16 by
+//                v_cvt_scalef32_pk_bf16_fp8 with the power-of-two part of the
+//                block scale (exact); the mantissa part of the scale multiplies
+//                the fp32 partial sum of that 128-channel block.  The contraction
+//                order inside a 64-channel step is permuted (the same way for K
+//                and Q) so that one 16-byte read feeds two MFMA k-steps.
+//   softmax      base 2, running maximum per (wavefront, head) moved lazily.
+//                P is written to LDS as bf16 in the B-operand layout of the
+//                second product, once per scale block with V's block scale
+//                folded in (so V itself is converted unscaled, exactly).
+//   O^T += V^T.P^T  Wavefront w owns value channels 128w..128w+127 for all heads
+//                of the workgroup: V^T fragments are transposing 8-byte LDS reads
+//                (ds_read_b64_tr_b8) of the raw tile.  Accumulators are kept per
+//                producing wavefront (its running maximum is private), 256 AGPRs
+//                in all, so the key loop needs one barrier per tile and no
+//                agreement on maxima; the two accumulator sets of a head (HG = 2)
+//                are merged once at the end, in registers.
+//   pipeline     iteration t: barrier; issue tile t+3; QK + softmax of tile t+1;
+//                PV of tile t.
+//
+// Key splits write fp32 partials and (max, sum) per head to the workspace; the
+// combine kernel of sparse_mla_mfma.hip finishes them.
+
+#include <cstdlib>
+
+#include "sparse_mla_common.h"
+#include "mfma_util.h"
+
+namespace cm {
+namespace {
+
+constexpr int kLat = 512;
+constexpr int kRope = 64;
+constexpr int kDqk = kLat + kRope;
+constexpr int kTK = 32;                         // keys per tile
+constexpr int kRing = 4;                        // tile slots
+constexpr int kLatBytes = kTK * kLat;           // 16384
+constexpr int kRopeBytes = kTK * kRope * 2;     // 4096
+constexpr int kScaleBytes = kTK * 4 * 4;        // 512: up to four fp32 scales per row
+constexpr int kSlotBytes = kLatBytes + kRopeBytes + kScaleBytes;   // 20992
+constexpr int kRingBytes = kRing * kSlotBytes;  // 83968
+constexpr int kMaxKeys = 2048;                  // keys of one split (their rows are staged in LDS)
+constexpr int kKeyInts = kMaxKeys + 4 * kTK;    // + the tiles the pipeline prefetches past the end
+constexpr int kXPitch = 132;                    // floats per head row of the output transpose (128 + 4)
+constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
+
+template <int HG>
+struct Geo {
+  static constexpr int kSpw = HG / 2;                       // 16-key sub-tiles per wavefront and tile
+  static constexpr int kSlots = 2 * HG;                     // (k-step, head group) pairs of a tile
+  static constexpr int kPBytes = 4 * kSlots * 1024;         // one parity: 4 scale variants
+  static constexpr int kPOff = kRingBytes;
+  static constexpr int kFacOff = kPOff + 2 * kPBytes;       // [parity][4 producers][32 heads] fp32
+  static constexpr int kFlagOff = kFacOff + 2 * 4 * 32 * 4; // [parity][4 producers] int
+  static constexpr int kStatOff = kFlagOff + 2 * 4 * 4;     // [4 producers][32 heads][2] fp32
+  static constexpr int kKeyOff = kStatOff + 4 * 32 * 2 * 4;
+  static constexpr int kSmem = kKeyOff + kKeyInts * 4;
+  static_assert(kSmem <= 160 * 1024, "LDS budget");
+  static_assert(4 * 32 * kXPitch * 4 <= kRingBytes, "the output transpose reuses the ring");
+};
+
+__device__ __forceinline__ bf16x8 cvt8(unsigned w0, unsigned w1, float pow2_scale) {
+  const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, pow2_scale, false));
+  const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, pow2_scale, true));
+  const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, pow2_scale, false));
+  const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, pow2_scale, true));
+  return __builtin_bit_cast(bf16x8, make_uint4(o0, o1, o2, o3));
+}
+
+// scale = pow2 * mant: pow2 keeps the exponent field (what the converter applies, exactly),
+// mant the sign and mantissa.  A zero or denormal scale comes out as ~2^-127 (its products
+// vanish either way); inf / nan scales stay non-finite.
+__device__ __forceinline__ float scale_pow2(float s) { return __uint_as_float(__float_as_uint(s) & 0x7f800000u); }
+__device__ __forceinline__ float scale_mant(float s) {
+  return __uint_as_float((__float_as_uint(s) & 0x807fffffu) | 0x3f800000u);
+}
+
+__device__ __forceinline__ void settle4(f32x4& a, f32x4& b) {
+  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a), "+v"(b));
+}
+
+template <int HG>
+__global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaParams p) {
+  using G_ = Geo<HG>;
+  constexpr int SPW = G_::kSpw;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = (int)threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // ---- which (query, KV group, head chunk, split): workgroups that gather the same rows
+  //      (the head chunks of one query and split) get ids that are equal modulo 8, i.e.
+  //      the same XCD and L2 ----
+  const int chunks = (p.heads_per_group + 32 * HG - 1) / (32 * HG);
+  const long long units = (long long)p.B * p.S * p.G * p.num_splits;
+  const long long units8 = units & ~7ll;
+  long long unit;
+  int chunk;
+  {
+    const long long id = blockIdx.x;
+    if (id < units8 * chunks) {
+      const long long slot = id >> 3;
+      unit = (slot / chunks) * 8 + (id & 7);
+      chunk = (int)(slot % chunks);
+    } else {
+      const long long r = id - units8 * chunks;
+      unit = units8 + r / chunks;
+      chunk = (int)(r % chunks);
+    }
+  }
+  const int split = (int)(unit % p.num_splits);
+  const long long qg = unit / p.num_splits;
+  const int g = (int)(qg % p.G);
+  const size_t bs = (size_t)(qg / p.G);           // b*S + s
+  const int b = (int)(bs / p.S);
+  const int head0 = g * p.heads_per_group + chunk * 32 * HG;
+  const int heads_here = min(32 * HG, p.heads_per_group - chunk * 32 * HG);
+  const size_t idx_base = (bs * p.G + g) * (size_t)p.topk;
+  const int key_begin = split * p.keys_per_split;
+  const int key_end = min(p.topk, key_begin + p.keys_per_split);
+  const int n_keys = max(0, key_end - key_begin);
+  const int n_tiles = (n_keys + kTK - 1) / kTK;
+
+  const int nblk = p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK ? kLat / p.kv_scale_block : 1;   // 1, 2 or 4
+  const bool has_scale = p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;
+
+  // roles: this wavefront produces scores for head group hgq and sub-tiles sub0.., and
+  // accumulates value channels 128*wave.. for every head group
+  const int hgq = wave % HG;
+  const int sub0 = (wave / HG) * SPW;
+
+  int* keys = reinterpret_cast<int*>(smem + G_::kKeyOff);
+  float* facbuf = reinterpret_cast<float*>(smem + G_::kFacOff);
+  int* flagbuf = reinterpret_cast<int*>(smem + G_::kFlagOff);
+  float* stats = reinterpret_cast<float*>(smem + G_::kStatOff);
+
+  // ---- cache rows of this split's keys -> LDS (-1 = skipped) ----
+  for (int i = tid; i < n_tiles * kTK + 4 * kTK; i += 256) {
+    int row = -1;
+    if (i < n_keys) {
+      const long long k = load_index(p, idx_base + key_begin + i);
+      if (k >= 0 && k < p.Skv) row = (int)k;
+    }
+    keys[i] = row;
+  }
+
+  // ---- Q^T fragments: lane (head n = lane%16, kq = lane/16), heads n and 16+n of group hgq.
+  //      latent step ks (64 channels): fragments 2ks, 2ks+1 hold channels 64ks + 16kq + {0..7}, {8..15};
+  //      rope step r: fragment 16+r holds channels 512 + 32r + 8kq + {0..7} ----
+  bf16x8 qf[2][18];
+  {
+    const int n = lane & 15, kq = lane >> 4;
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int h = 32 * hgq + hh * 16 + n;
+      const bool live = h < heads_here;
+      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (live ? h : 0)) * (size_t)kDqk;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        uint4 t0 = make_uint4(0, 0, 0, 0), t1 = t0;
+        if (live) {
+          t0 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq);
+          t1 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq + 8);
+        }
+        qf[hh][2 * ks] = __builtin_bit_cast(bf16x8, t0);
+        qf[hh][2 * ks + 1] = __builtin_bit_cast(bf16x8, t1);
+      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        uint4 t = make_uint4(0, 0, 0, 0);
+        if (live) t = *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kq);
+        qf[hh][16 + r] = __builtin_bit_cast(bf16x8, t);
+      }
+    }
+  }
+  __syncthreads();                                // keys[] is complete
+
+  // ---- HBM -> LDS: this wavefront brings rows 8*wave .. 8*wave+7 of a tile.  A skipped key
+  //      fetches cache row 0 instead (its probability is zero), so every wavefront issues
+  //      the same number of loads for every tile and the in-order load counter can be
+  //      waited on by count. ----
+  const size_t row_base = (size_t)b * p.Skv;
+  const bool scale_op = has_scale && 64 * wave < kTK * nblk;
+  auto issue_tile = [&](int tau) {
+    unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
+    const int* tk = keys + tau * kTK;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {                 // latent: rows 8w+2i (lanes 0..31), 8w+2i+1 (lanes 32..63)
+      const int rr = 8 * wave + 2 * i + (lane >> 5);
+      const int row = max(tk[rr], 0);
+      const size_t krow = (row_base + (size_t)row) * p.G + g;
+      const unsigned char* src = (const unsigned char*)p.kv + krow * kLat + (((lane & 31) ^ (rr & 7)) << 4);
+      __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(slot + (8 * wave + 2 * i) * kLat), 16, 0, 0);
+    }
+    {                                             // rope: rows 8w + lane/8, 8 chunks of 16 bytes each
+      const int rr = 8 * wave + (lane >> 3);
+      const int row = max(tk[rr], 0);
+      const size_t krow = (row_base + (size_t)row) * p.G + g;
+      const unsigned char* src = (const unsigned char*)p.rope + krow * (kRope * 2) + (((lane & 7) ^ (rr & 7)) << 4);
+      __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(slot + kLatBytes + 8 * wave * (kRope * 2)), 16, 0, 0);
+    }
+    if (scale_op) {                               // scales: element e = 64w + lane of [32 rows][nblk]
+      const int e = 64 * wave + lane;
+      if (e < kTK * nblk) {
+        const int rr = e / nblk;
+        const int row = max(tk[rr], 0);
+        const size_t krow = (row_base + (size_t)row) * p.G + g;
+        const float* src = (const float*)p.kv_scale + krow * nblk + (e - rr * nblk);
+        __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(slot + kLatBytes + kRopeBytes + 256 * wave), 4, 0, 0);
+      }
+    }
+  };
+  auto wait_tiles_but_one = [&]() {               // everything but the most recently issued tile has landed
+    if (scale_op) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  };
+
+  // ---- score side state ----
+  float m_run[2] = {-INFINITY, -INFINITY};        // base-2 running reference of heads n and 16+n
+  float l_run[2] = {0.0f, 0.0f};                  // this lane's share of the denominators
+  const float qk_scale = p.sm_scale * kLog2e;
+
+  // S^T of tile tau for this wavefront's head group and sub-tiles, softmax, P -> LDS
+  auto score_tile = [&](int tau) {
+    const unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
+    const int par = tau & 1;
+    const int m = lane & 15, kq = lane >> 4;
+    f32x4 st[SPW][2];
+#pragma unroll
+    for (int sj = 0; sj < SPW; ++sj) {
+      const int r = 16 * (sub0 + sj) + m;         // tile row of this lane's K fragment
+      const int r7 = r & 7;
+      const unsigned char* lat0 = slot + r * kLat + ((kq ^ r7) << 4);
+      const unsigned char* lat1 = slot + r * kLat + (((4 + kq) ^ r7) << 4);
+      const unsigned char* rope = slot + kLatBytes + r * (kRope * 2);
+      const float* scl = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + r * nblk;
+      // the power-of-two part of a key's scale goes into the conversion of its K fragment (this
+      // lane's row r); the mantissa part multiplies the partial sums, which this lane holds for
+      // keys 4*(lane/16) + i
+      const float* sclc = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * kq) * nblk;
+      float pw[4];
+#pragma unroll
+      for (int grp = 0; grp < 4; ++grp) pw[grp] = has_scale ? scale_pow2(scl[(grp * nblk) >> 2]) : 1.0f;
+      f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int grp = 0; grp < 4; ++grp) {         // 128 latent channels = two 64-channel steps
+        f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int ks = 2 * grp + half;
+          const uint4 raw = *reinterpret_cast<const uint4*>((half ? lat1 : lat0) + 128 * grp);
+          const bf16x8 f0 = cvt8(raw.x, raw.y, pw[grp]);
+          const bf16x8 f1 = cvt8(raw.z, raw.w, pw[grp]);
+          mfma_qk(a0, f0, qf[0][2 * ks]);
+          mfma_qk(a1, f0, qf[1][2 * ks]);
+          mfma_qk(a0, f1, qf[0][2 * ks + 1]);
+          mfma_qk(a1, f1, qf[1][2 * ks + 1]);
+        }
+        settle4(a0, a1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float mant = has_scale ? scale_mant(sclc[i * nblk + ((grp * nblk) >> 2)]) : 1.0f;
+          tot0[i] += mant * a0[i];
+          tot1[i] += mant * a1[i];
+        }
+      }
+      {
+        f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int rs = 0; rs < 2; ++rs) {
+          const bf16x8 f = *reinterpret_cast<const bf16x8*>(rope + (((4 * rs + kq) ^ r7) << 4));
+          mfma_qk(a0, f, qf[0][16 + rs]);
+          mfma_qk(a1, f, qf[1][16 + rs]);
+        }
+        settle4(a0, a1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          tot0[i] += a0[i];
+          tot1[i] += a1[i];
+        }
+      }
+      st[sj][0] = tot0;
+      st[sj][1] = tot1;
+    }
+    // lane (n = lane%16, gq = lane/16) holds keys 4gq+i of each sub-tile for heads n (st[.][0]) and 16+n
+    const int n = lane & 15, gq = lane >> 4;
+    float sv[SPW][2][4];
+    float mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+    for (int sj = 0; sj < SPW; ++sj) {
+      const int4 kk = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * (sub0 + sj) + 4 * gq);
+      const bool ok[4] = {kk.x >= 0, kk.y >= 0, kk.z >= 0, kk.w >= 0};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sv[sj][0][i] = ok[i] ? st[sj][0][i] * qk_scale : -INFINITY;
+        sv[sj][1][i] = ok[i] ? st[sj][1][i] * qk_scale : -INFINITY;
+        mx[0] = fmaxf(mx[0], sv[sj][0][i]);
+        mx[1] = fmaxf(mx[1], sv[sj][1][i]);
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      mx[hh] = fmaxf(mx[hh], xor16(mx[hh]));
+      mx[hh] = fmaxf(mx[hh], xor32(mx[hh]));
+    }
+    // lazy running reference; consumers rescale their accumulators by fac before adding this tile
+    const bool grow = (mx[0] > m_run[0] + kLazy) || (mx[1] > m_run[1] + kLazy);
+    const bool any_grow = __ballot(grow) != 0ull;
+    if (any_grow) {
+      float fac[2];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const float m_new = (mx[hh] > m_run[hh] + kLazy) ? mx[hh] : m_run[hh];
+        fac[hh] = (m_run[hh] == -INFINITY) ? 0.0f : exp2f(m_run[hh] - m_new);
+        l_run[hh] *= fac[hh];
+        m_run[hh] = m_new;
+      }
+      if (lane < 16) {
+        facbuf[(par * 4 + wave) * 32 + n] = fac[0];
+        facbuf[(par * 4 + wave) * 32 + 16 + n] = fac[1];
+      }
+    }
+    if (lane == 0) flagbuf[par * 4 + wave] = any_grow ? 1 : 0;
+
+    // P (x V's block scale) -> LDS in the B-operand layout of the 32x32x16 product:
+    // lane (head, kq8 = key/8) owns 16 bytes = keys 8kq8..8kq8+7; this lane holds keys 4gq..4gq+3
+    const int variants = has_scale ? nblk : 1;
+    unsigned char* pbase = smem + G_::kPOff + par * G_::kPBytes;
+#pragma unroll
+    for (int sj = 0; sj < SPW; ++sj) {
+      float pr[2][4];
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pr[hh][i] = (sv[sj][hh][i] == -INFINITY) ? 0.0f : exp2f(sv[sj][hh][i] - m_run[hh]);
+          l_run[hh] += pr[hh][i];
+        }
+      const int slot_id = (sub0 + sj) * HG + hgq;
+      const float* scl = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * gq) * nblk;
+      for (int v = 0; v < variants; ++v) {
+        float sc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sc[i] = has_scale ? scl[i * nblk + v] : 1.0f;
+        unsigned char* dst = pbase + ((v * G_::kSlots + slot_id) * 64 + (gq >> 1) * 32) * 16 + (gq & 1) * 8;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          const uint2 w = make_uint2(pack_bf16(pr[hh][0] * sc[0], pr[hh][1] * sc[1]),
+                                     pack_bf16(pr[hh][2] * sc[2], pr[hh][3] * sc[3]));
+          *reinterpret_cast<uint2*>(dst + (hh * 16 + n) * 16) = w;
+        }
+      }
+    }
+  };
+
+  // ---- value side state: o[4*dvb + producer] = O^T[32 channels x 32 heads] ----
+  f32x16 o[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) o[i][j] = 0.0f;
+  const int pvar = has_scale ? (wave * nblk) >> 2 : 0;         // scale block of channels 128*wave..
+  int pv_off[4];                                               // transposing-read offsets per 32-channel block
+  {
+    const int t = lane & 15, half = (lane >> 4) & 1, kq2 = lane >> 5;
+    const int r = 8 * kq2 + (t >> 1);                          // row within a 16-key step (r & 7 = t >> 1)
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+      const int c = 8 * wave + 2 * dvb + half;                 // 16-byte chunk of the row
+      pv_off[dvb] = r * kLat + ((c ^ (r & 7)) << 4) + 8 * (t & 1);
+    }
+  }
+  auto scale_acc = [&](int prod, float f) {                    // o[.][prod] *= f (per-lane factor)
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) o[4 * dvb + prod][j] *= f;
+      asm volatile("" : "+a"(o[4 * dvb + prod]));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto value_tile = [&](int tau) {
+    const unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
+    const int par = tau & 1;
+    {
+      const int4 fl = *reinterpret_cast<const int4*>(flagbuf + par * 4);
+      const int f4[4] = {fl.x, fl.y, fl.z, fl.w};
+      bool any = false;
+#pragma unroll
+      for (int prod = 0; prod < 4; ++prod) any = any || (__builtin_amdgcn_readfirstlane(f4[prod]) != 0);
+      if (any) {
+        mfma_settle_acc(o);
+#pragma unroll
+        for (int prod = 0; prod < 4; ++prod) {
+          if (__builtin_amdgcn_readfirstlane(f4[prod]) != 0) scale_acc(prod, facbuf[(par * 4 + prod) * 32 + (lane & 31)]);
+        }
+        mfma_settle_acc(o);
+      }
+    }
+    const unsigned char* pbase = smem + G_::kPOff + par * G_::kPBytes + (pvar * G_::kSlots * 64 + lane) * 16;
+#pragma unroll
+    for (int kstep = 0; kstep < 2; ++kstep) {
+      bf16x8 pb[HG];
+#pragma unroll
+      for (int hg = 0; hg < HG; ++hg) pb[hg] = *reinterpret_cast<const bf16x8*>(pbase + (kstep * HG + hg) * 1024);
+#pragma unroll
+      for (int dvb = 0; dvb < 4; ++dvb) {
+        typedef __attribute__((ext_vector_type(2))) int i32x2;
+        const i32x2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (__attribute__((address_space(3))) i32x2*)(slot + 16 * kstep * kLat + pv_off[dvb]));
+        const bf16x8 a = cvt8((unsigned)raw[0], (unsigned)raw[1], 1.0f);
+#pragma unroll
+        for (int hg = 0; hg < HG; ++hg) {
+          const int prod = HG == 4 ? hg : hg + 2 * kstep;      // the wavefront that produced this P
+          mfma_pv(o[4 * dvb + prod], a, pb[hg]);
+        }
+      }
+    }
+  };
+
+  // ---- pipeline ----
+  issue_tile(0);
+  issue_tile(1);
+  issue_tile(2);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  score_tile(0);
+  for (int t = 0; t < n_tiles; ++t) {
+    wait_tiles_but_one();                         // tile t+1 (issued two iterations ago) has landed
+    __syncthreads();                              // ... for every wavefront; P(t) is complete; PV(t-1) is done
+    issue_tile(t + 3);                            // into the slot of tile t-1
+    if (t + 1 < n_tiles) score_tile(t + 1);
+    value_tile(t);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the prefetches past the end
+  mfma_settle_acc(o);
+
+  // ---- epilogue ----
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {                // a head's denominator is spread over lanes n, n+16, n+32, n+48
+    l_run[hh] += xor16(l_run[hh]);
+    l_run[hh] += xor32(l_run[hh]);
+  }
+  if (lane < 16) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      stats[(wave * 32 + hh * 16 + lane) * 2 + 0] = m_run[hh];
+      stats[(wave * 32 + hh * 16 + lane) * 2 + 1] = l_run[hh];
+    }
+  }
+  __syncthreads();                                // statistics are visible; the ring is free
+
+  const int hd = lane & 31, gq2 = lane >> 5;
+  const bool direct = p.num_splits == 1;
+  float* xbuf = reinterpret_cast<float*>(smem) + wave * 32 * kXPitch;     // private to this wavefront
+  const size_t q_index = bs;
+#pragma unroll
+  for (int hg = 0; hg < HG; ++hg) {
+    float m_all, l_all;
+    if (HG == 4) {
+      m_all = stats[(hg * 32 + hd) * 2];
+      l_all = stats[(hg * 32 + hd) * 2 + 1];
+    } else {                                      // two producers per head group: hg and hg + 2
+      const float ma = stats[(hg * 32 + hd) * 2], la = stats[(hg * 32 + hd) * 2 + 1];
+      const float mb = stats[((hg + 2) * 32 + hd) * 2], lb = stats[((hg + 2) * 32 + hd) * 2 + 1];
+      m_all = fmaxf(ma, mb);
+      const float fa = (ma == -INFINITY) ? 0.0f : exp2f(ma - m_all);
+      const float fb = (mb == -INFINITY) ? 0.0f : exp2f(mb - m_all);
+      l_all = la * fa + lb * fb;
+#pragma unroll
+      for (int dvb = 0; dvb < 4; ++dvb) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o[4 * dvb + hg][j] = o[4 * dvb + hg][j] * fa + o[4 * dvb + hg + 2][j] * fb;
+        asm volatile("" : "+a"(o[4 * dvb + hg]));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const int h_local = 32 * hg + hd;
+    float out_scale = 1.0f, lse_val = 0.0f;
+    if (direct) {
+      float m_fin = m_all, l_fin = l_all;
+      if (p.sinks && h_local < heads_here) {
+        const float sk = p.sinks[head0 + h_local] * kLog2e;
+        const float m2 = fmaxf(m_fin, sk);
+        const float keep = (m_fin == -INFINITY) ? 0.0f : exp2f(m_fin - m2);
+        l_fin = l_fin * keep + exp2f(sk - m2);
+        out_scale = keep;
+        m_fin = m2;
+      }
+      if (l_fin > 0.0f) {
+        out_scale = out_scale / l_fin;
+        lse_val = (m_fin + log2f(l_fin)) * kLn2;
+      } else {
+        out_scale = 0.0f;
+      }
+    }
+    // transpose through LDS: lane (head hd, gq2) holds channels 32dvb + 8j + 4gq2 + (0..3) in o[.][4j..4j+3]
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x16& acc = o[4 * dvb + hg];
+        const float4 v = make_float4(acc[4 * j] * out_scale, acc[4 * j + 1] * out_scale, acc[4 * j + 2] * out_scale,
+                                     acc[4 * j + 3] * out_scale);
+        *reinterpret_cast<float4*>(xbuf + hd * kXPitch + 32 * dvb + 8 * j + 4 * gq2) = v;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // rows of 128 channels leave coalesced: 32 lanes x 4 channels, two heads per step
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+      const int row = 2 * it + gq2;
+      const int hl = 32 * hg + row;
+      if (hl >= heads_here) continue;
+      const float4 v = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + hd * 4);
+      const int ch = 128 * wave + hd * 4;
+      if (direct) {
+        const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + ch;
+        if (p.out_dtype == CPPMEGA_MI355_F32) {
+          *reinterpret_cast<float4*>((float*)p.out + off) = v;
+        } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
+          *reinterpret_cast<uint2*>((unsigned short*)p.out + off) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
+        } else {
+          unsigned short* dst = (unsigned short*)p.out + off;
+          dst[0] = f32_to_f16_bits(v.x); dst[1] = f32_to_f16_bits(v.y);
+          dst[2] = f32_to_f16_bits(v.z); dst[3] = f32_to_f16_bits(v.w);
+        }
+      } else {
+        float* part = (float*)p.workspace + ((q_index * p.H + head0 + hl) * (size_t)p.num_splits + split) * kLat + ch;
+        *reinterpret_cast<float4*>(part) = v;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (wave == 0 && lane < 32 && h_local < heads_here) {
+      if (direct) {
+        if (p.lse) p.lse[q_index * p.H + head0 + h_local] = lse_val;
+      } else {
+        float* ml = (float*)p.workspace + (size_t)p.B * p.S * p.H * p.num_splits * kLat +
+                    ((q_index * p.H + head0 + h_local) * (size_t)p.num_splits + split) * 2;
+        ml[0] = m_all;
+        ml[1] = l_all;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+bool sparse_mla_latent_supported(const MlaParams& p) {
+  if (p.q_dtype != CPPMEGA_MI355_BF16 || p.q_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
+  if (p.d_qk != kDqk || p.d_v != kLat || p.d_kv != kLat) return false;
+  if (p.kv_dtype != CPPMEGA_MI355_E4M3) return false;
+  if (p.rope_dim != kRope || p.rope_dtype != CPPMEGA_MI355_BF16) return false;
+  if (p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK) {
+    if (p.kv_scale_block != 128 && p.kv_scale_block != 256 && p.kv_scale_block != 512) return false;
+  } else if (p.kv_scale_kind != CPPMEGA_MI355_SCALE_PER_TOKEN && p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE) {
+    return false;
+  }
+  if (p.heads_per_group <= 32) return false;      // a single 32-head group gains nothing from sharing
+  if (p.topk < 1 || (size_t)p.B * p.S == 0) return false;
+  if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
+  if (p.kv_scale && ((uintptr_t)p.kv_scale & 3)) return false;
+  return true;
+}
+
+// heads per workgroup (in units of 32) and the key-split factor
+void sparse_mla_latent_plan(MlaParams& p) {
+  int hg = p.heads_per_group > 64 ? 4 : 2;
+  const long long queries = (long long)p.B * p.S * p.G;
+  // few queries: smaller head chunks need fewer key splits to fill the device, and each
+  // split writes (and the combine step re-reads) an fp32 partial per head
+  if (hg == 4 && queries * ((p.heads_per_group + 127) / 128) < 128) hg = 2;
+  if (const char* env = getenv("CPPMEGA_MI355_MLA_HEADS_PER_WG")) {
+    const int v = atoi(env);
+    if (v == 64) hg = 2;
+    if (v == 128) hg = 4;
+  }
+  p.heads_per_wg = 32 * hg;
+  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const long long base = queries * chunks;
+  int splits = 1;
+  while (base * splits < 256 && p.topk / (splits * 2) >= 4 * kTK && splits < 16) splits *= 2;
+  while ((p.topk + splits - 1) / splits > kMaxKeys) splits *= 2;
+  const int tiles = (p.topk + kTK - 1) / kTK;
+  const int tiles_per_split = (tiles + splits - 1) / splits;
+  p.num_splits = splits;
+  p.keys_per_split = tiles_per_split * kTK;
+}
+
+int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream) {
+  const int hg = p.heads_per_wg / 32;
+  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const long long wgs = (long long)p.B * p.S * p.G * p.num_splits * chunks;
+  if (wgs > 0x7fffffffll || p.keys_per_split > kMaxKeys) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse MLA: launch too large");
+  const dim3 grid((unsigned)wgs), block(256);
+  if (hg == 4) {
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     Geo<4>::kSmem));
+    hipLaunchKernelGGL(sparse_mla_latent_kernel<4>, grid, block, Geo<4>::kSmem, stream, p);
+  } else {
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     Geo<2>::kSmem));
+    hipLaunchKernelGGL(sparse_mla_latent_kernel<2>, grid, block, Geo<2>::kSmem, stream, p);
+  }
+  CM_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+}  // namespace cm

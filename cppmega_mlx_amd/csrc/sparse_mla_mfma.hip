@@ -29,6 +29,7 @@
 //           the B operand with one v_permlane16_swap, never through memory.
 
 #include "sparse_mla_common.h"
+#include "mfma_util.h"
 
 namespace cm {
 namespace {
@@ -52,12 +53,7 @@ constexpr int kXBytes = kWaves * kHeads * kXPitch * 4;    // 133120
 constexpr int kStatOff = kXBytes;                         // [4 waves][32 heads][2] floats
 constexpr int kSmemBytes = kXBytes + kWaves * kHeads * 2 * 4;
 static_assert(kWaves * kWaveBytes <= kXBytes, "the merge buffer reuses the tile area");
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kLazy = 8.0f;      // rescale when the running max grows by more than 2^8
-
-typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void glb_void;
 
 // 16-byte chunk q of row r lives at chunk (q with its low 3 bits xor f(r)):
 // 8 consecutive rows hit 8 different bank groups for the same q (16-byte
@@ -76,77 +72,6 @@ __device__ __forceinline__ bf16x4 lds_read_tr16_b64(const unsigned char* addr) {
   typedef __attribute__((ext_vector_type(4))) short s16x4;
   const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)addr);
   return __builtin_bit_cast(bf16x4, v);
-}
-
-// The two MFMA shapes as inline assembly with fixed register classes.  The
-// 32 x 512 fp32 output accumulators fill all 256 accumulation registers (AGPRs);
-// the small score accumulators therefore have to live in ordinary VGPRs, which
-// the builtin form of the instruction cannot express once a kernel uses AGPRs.
-// Dependent MFMAs on the same accumulator are interlocked by the hardware; a
-// VALU read of a result is not, hence mfma_settle().
-__device__ __forceinline__ void mfma_qk(f32x4& acc, const bf16x8& a, const bf16x8& b) {
-  asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_pv(f32x16& acc, const bf16x8& a, const bf16x8& b) {
-  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-}
-// wait states between the last MFMA writing these registers and the first non-MFMA use
-__device__ __forceinline__ void mfma_settle(f32x4& s0, f32x4& s1) {
-  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(s0), "+v"(s1));
-}
-__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[16]) {
-  asm volatile("s_nop 15\n\ts_nop 7"
-               : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]),
-                 "+a"(o[8]), "+a"(o[9]), "+a"(o[10]), "+a"(o[11]), "+a"(o[12]), "+a"(o[13]), "+a"(o[14]), "+a"(o[15]));
-}
-
-__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
-  // round-to-nearest-even; inputs are finite and non-negative probabilities or dequantised values
-  typedef __attribute__((ext_vector_type(2))) __bf16 v2;
-  v2 r;
-  r[0] = (__bf16)a;
-  r[1] = (__bf16)b;
-  return __builtin_bit_cast(unsigned, r);
-}
-
-__device__ __forceinline__ bool scale_is_pow2(float s) {
-  const unsigned u = __float_as_uint(s);
-  const unsigned e = u >> 23;                 // sign + exponent
-  return (u & 0x007fffffu) == 0u && e >= 1u && e <= 254u;
-}
-
-// 16 e4m3 bytes * scale -> 16 bf16 (two 16-byte LDS chunks).  POW2: the scale is a
-// normal power of two, which the converter applies exactly (it only looks at the
-// exponent of its scale operand); otherwise convert unscaled and multiply in fp32.
-template <bool POW2>
-__device__ __forceinline__ void dequant16(const uint4 raw, float scale, uint4& lo, uint4& hi) {
-  const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
-  unsigned o[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (POW2) {
-      o[2 * i] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[i], scale, false));
-      o[2 * i + 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[i], scale, true));
-    } else {
-      const f32x2 a = e4m3x2_lo(w[i]), b = e4m3x2_hi(w[i]);
-      o[2 * i] = pack_bf16(a[0] * scale, a[1] * scale);
-      o[2 * i + 1] = pack_bf16(b[0] * scale, b[1] * scale);
-    }
-  }
-  lo = make_uint4(o[0], o[1], o[2], o[3]);
-  hi = make_uint4(o[4], o[5], o[6], o[7]);
-}
-
-// value of lane (lane ^ 16) / (lane ^ 32), VALU only
-__device__ __forceinline__ float xor16(float v) {
-  const unsigned u = __float_as_uint(v);
-  const u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  return __uint_as_float((lane_id() & 16) ? r[0] : r[1]);
-}
-__device__ __forceinline__ float xor32(float v) {
-  const unsigned u = __float_as_uint(v);
-  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __uint_as_float((lane_id() & 32) ? r[0] : r[1]);
 }
 
 // KV_FP8: latent e4m3 + fp32 scales (+ bf16 rope tail); otherwise a bf16 row of 576 (or 512 + rope tail)
@@ -623,6 +548,7 @@ __global__ __launch_bounds__(256) void sparse_mla_combine_kernel(const MlaParams
 }  // namespace
 
 bool sparse_mla_mfma_supported(const MlaParams& p) {
+  if (sparse_mla_latent_supported(p)) return true;
   if (p.q_dtype != CPPMEGA_MI355_BF16 || p.q_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
   if (p.d_qk != kDqk || p.d_v != kLat) return false;
   if (p.rope_dim != 0 && (p.rope_dim != kRope || p.rope_dtype != CPPMEGA_MI355_BF16)) return false;
@@ -647,6 +573,11 @@ bool sparse_mla_mfma_supported(const MlaParams& p) {
 
 // Chooses the key-split factor: enough workgroups to cover the 256 CUs, at least 64 keys per wavefront.
 void sparse_mla_mfma_plan(MlaParams& p) {
+  p.heads_per_wg = 0;
+  if (sparse_mla_latent_supported(p)) {
+    sparse_mla_latent_plan(p);
+    return;
+  }
   const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
   const long long base = (long long)p.B * p.S * p.G * groups_per_kv;
   int splits = 1;
@@ -663,6 +594,16 @@ size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p) {
 }
 
 int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
+  if (p.heads_per_wg != 0) {
+    const int rc = sparse_mla_latent_launch(p, stream);
+    if (rc != 0) return rc;
+    if (p.num_splits > 1) {
+      const size_t qh = (size_t)p.B * p.S * p.H;
+      hipLaunchKernelGGL(sparse_mla_combine_kernel, dim3((unsigned)((qh + 3) / 4)), dim3(256), 0, stream, p);
+      CM_HIP_CHECK(hipGetLastError());
+    }
+    return 0;
+  }
   const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
   const dim3 grid((unsigned)((size_t)p.B * p.S * p.G * groups_per_kv), (unsigned)p.num_splits), block(kWaves * 64);
   if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
