@@ -28,6 +28,9 @@ HIPCC_FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA builtins keep their accumulators in ordinary VGPRs; kernels that want AGPR
+    # accumulators say so with inline assembly
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-result",
 ]
 

@@ -79,6 +79,9 @@ struct Geo {
   static_assert(4 * 32 * kXPitch * 4 <= kRingBytes, "the output transpose reuses the ring");
 };
 
+// 2^x by the hardware instruction alone (x <= ~8 here; tiny results may flush to zero)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ bf16x8 cvt8(unsigned w0, unsigned w1, float pow2_scale) {
   const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, pow2_scale, false));
   const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, pow2_scale, true));
@@ -95,11 +98,16 @@ __device__ __forceinline__ float scale_mant(float s) {
   return __uint_as_float((__float_as_uint(s) & 0x807fffffu) | 0x3f800000u);
 }
 
-__device__ __forceinline__ void settle4(f32x4& a, f32x4& b) {
-  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a), "+v"(b));
+// The score product uses the compiler's own MFMA (this file is built with
+// -mllvm -amdgpu-mfma-vgpr-form, so its accumulators are ordinary VGPRs): the compiler then
+// knows the instruction's latency and pads its hazards exactly.  The value product keeps the
+// inline form: its 256 accumulator registers must be AGPRs.
+__device__ __forceinline__ void mfma_s(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
 }
 
-template <int HG>
+// HG: 32-head groups per workgroup (2 or 4); NBLK: fp32 scales per key row (1, 2 or 4)
+template <int HG, int NBLK>
 __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaParams p) {
   using G_ = Geo<HG>;
   constexpr int SPW = G_::kSpw;
@@ -140,8 +148,8 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   const int n_keys = max(0, key_end - key_begin);
   const int n_tiles = (n_keys + kTK - 1) / kTK;
 
-  const int nblk = p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK ? kLat / p.kv_scale_block : 1;   // 1, 2 or 4
-  const bool has_scale = p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;
+  constexpr int nblk = NBLK;
+  const bool has_scale = p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;   // otherwise the scale area holds ones
 
   // roles: this wavefront produces scores for head group hgq and sub-tiles sub0.., and
   // accumulates value channels 128*wave.. for every head group
@@ -192,41 +200,55 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       }
     }
   }
+  if (!has_scale) {                               // no scales in memory: every slot's scale area is 1.0 for good
+    for (int i = tid; i < kRing * kTK; i += 256)
+      reinterpret_cast<float*>(smem + (i / kTK) * kSlotBytes + kLatBytes + kRopeBytes)[i % kTK] = 1.0f;
+  }
   __syncthreads();                                // keys[] is complete
 
   // ---- HBM -> LDS: this wavefront brings rows 8*wave .. 8*wave+7 of a tile.  A skipped key
   //      fetches cache row 0 instead (its probability is zero), so every wavefront issues
   //      the same number of loads for every tile and the in-order load counter can be
   //      waited on by count. ----
-  const size_t row_base = (size_t)b * p.Skv;
+  // Row numbers fit 32 bits (checked on the host).  The loads are written as inline assembly:
+  // the compiler would otherwise order every later LDS read behind them (vmcnt(0)), which
+  // serialises the pipeline this kernel is built around.
+  //   latent : instruction i of wavefront w carries rows 8i+2w (lanes 0..31) and 8i+2w+1, so a
+  //            lane's swizzle term (row & 7) is the same for all i
+  //   rope   : one instruction, rows 8w + lane/8
+  //   scales : element 64w + lane of [32 rows][nblk]
   const bool scale_op = has_scale && 64 * wave < kTK * nblk;
+  const size_t group_row0 = ((size_t)b * p.Skv) * p.G + g;     // cache row of key 0; key k is G rows further per step
+  const int lat_row = 2 * wave + (lane >> 5);                 // + 8i
+  const int rope_row = 8 * wave + (lane >> 3);
+  const int sc_elem = 64 * wave + lane;
+  const int sc_row = min(sc_elem / nblk, kTK - 1);
+  const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + (((lane & 31) ^ (lat_row & 7)) << 4);
+  const unsigned char* rope_src = (const unsigned char*)p.rope + group_row0 * (kRope * 2) + (((lane & 7) ^ (rope_row & 7)) << 4);
+  const unsigned char* sc_src = (const unsigned char*)p.kv_scale + (group_row0 * nblk + (unsigned)(sc_elem % nblk)) * 4;
+  const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = (unsigned)p.G * nblk * 4;
+  auto dma16 = [&](const unsigned char* src, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "memory", "m0");
+  };
+  auto dma4 = [&](const unsigned char* src, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "memory", "m0");
+  };
+  const unsigned smem_base = (unsigned)(size_t)(lds_void*)smem;                 // LDS byte address of the ring
   auto issue_tile = [&](int tau) {
-    unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
+    const unsigned slot = smem_base + (unsigned)(tau & (kRing - 1)) * kSlotBytes;
     const int* tk = keys + tau * kTK;
+    int rows[6];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {                 // latent: rows 8w+2i (lanes 0..31), 8w+2i+1 (lanes 32..63)
-      const int rr = 8 * wave + 2 * i + (lane >> 5);
-      const int row = max(tk[rr], 0);
-      const size_t krow = (row_base + (size_t)row) * p.G + g;
-      const unsigned char* src = (const unsigned char*)p.kv + krow * kLat + (((lane & 31) ^ (rr & 7)) << 4);
-      __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(slot + (8 * wave + 2 * i) * kLat), 16, 0, 0);
-    }
-    {                                             // rope: rows 8w + lane/8, 8 chunks of 16 bytes each
-      const int rr = 8 * wave + (lane >> 3);
-      const int row = max(tk[rr], 0);
-      const size_t krow = (row_base + (size_t)row) * p.G + g;
-      const unsigned char* src = (const unsigned char*)p.rope + krow * (kRope * 2) + (((lane & 7) ^ (rr & 7)) << 4);
-      __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(slot + kLatBytes + 8 * wave * (kRope * 2)), 16, 0, 0);
-    }
-    if (scale_op) {                               // scales: element e = 64w + lane of [32 rows][nblk]
-      const int e = 64 * wave + lane;
-      if (e < kTK * nblk) {
-        const int rr = e / nblk;
-        const int row = max(tk[rr], 0);
-        const size_t krow = (row_base + (size_t)row) * p.G + g;
-        const float* src = (const float*)p.kv_scale + krow * nblk + (e - rr * nblk);
-        __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(slot + kLatBytes + kRopeBytes + 256 * wave), 4, 0, 0);
-      }
+    for (int i = 0; i < 4; ++i) rows[i] = tk[8 * i + lat_row];
+    rows[4] = tk[rope_row];
+    rows[5] = scale_op ? tk[sc_row] : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      dma16(lat_src + (size_t)(unsigned)max(rows[i], 0) * lat_step, slot + (8 * i + 2 * wave) * kLat);
+    dma16(rope_src + (size_t)(unsigned)max(rows[4], 0) * rope_step, slot + kLatBytes + 8 * wave * (kRope * 2));
+    if (scale_op) {
+      if (sc_elem < kTK * nblk)
+        dma4(sc_src + (size_t)(unsigned)max(rows[5], 0) * sc_step, slot + kLatBytes + kRopeBytes + 256 * wave);
     }
   };
   auto wait_tiles_but_one = [&]() {               // everything but the most recently issued tile has landed
@@ -239,12 +261,10 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   float l_run[2] = {0.0f, 0.0f};                  // this lane's share of the denominators
   const float qk_scale = p.sm_scale * kLog2e;
 
-  // S^T of tile tau for this wavefront's head group and sub-tiles, softmax, P -> LDS
-  auto score_tile = [&](int tau) {
+  // S^T of tile tau for this wavefront's head group and sub-tiles
+  auto qk_tile = [&](int tau, f32x4 (&st)[SPW][2]) {
     const unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
-    const int par = tau & 1;
     const int m = lane & 15, kq = lane >> 4;
-    f32x4 st[SPW][2];
 #pragma unroll
     for (int sj = 0; sj < SPW; ++sj) {
       const int r = 16 * (sub0 + sj) + m;         // tile row of this lane's K fragment
@@ -258,29 +278,46 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       // keys 4*(lane/16) + i
       const float* sclc = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * kq) * nblk;
       float pw[4];
+      bool plain = true;                          // every scale of this row is a power of two
 #pragma unroll
-      for (int grp = 0; grp < 4; ++grp) pw[grp] = has_scale ? scale_pow2(scl[(grp * nblk) >> 2]) : 1.0f;
+      for (int grp = 0; grp < 4; ++grp) {
+        const float sc = scl[(grp * nblk) >> 2];
+        pw[grp] = scale_pow2(sc);
+        plain = plain && (pw[grp] == sc);
+      }
       f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
+      if (__ballot(!plain) == 0ull) {             // (uniform) one accumulation chain, no mantissa factors
 #pragma unroll
-      for (int grp = 0; grp < 4; ++grp) {         // 128 latent channels = two 64-channel steps
-        f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int ks = 2 * grp + half;
-          const uint4 raw = *reinterpret_cast<const uint4*>((half ? lat1 : lat0) + 128 * grp);
-          const bf16x8 f0 = cvt8(raw.x, raw.y, pw[grp]);
-          const bf16x8 f1 = cvt8(raw.z, raw.w, pw[grp]);
-          mfma_qk(a0, f0, qf[0][2 * ks]);
-          mfma_qk(a1, f0, qf[1][2 * ks]);
-          mfma_qk(a0, f1, qf[0][2 * ks + 1]);
-          mfma_qk(a1, f1, qf[1][2 * ks + 1]);
+        for (int ks = 0; ks < 8; ++ks) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(((ks & 1) ? lat1 : lat0) + 128 * (ks >> 1));
+          const bf16x8 f0 = cvt8(raw.x, raw.y, pw[ks >> 1]);
+          const bf16x8 f1 = cvt8(raw.z, raw.w, pw[ks >> 1]);
+          mfma_s(tot0, f0, qf[0][2 * ks]);
+          mfma_s(tot1, f0, qf[1][2 * ks]);
+          mfma_s(tot0, f1, qf[0][2 * ks + 1]);
+          mfma_s(tot1, f1, qf[1][2 * ks + 1]);
         }
-        settle4(a0, a1);
+      } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float mant = has_scale ? scale_mant(sclc[i * nblk + ((grp * nblk) >> 2)]) : 1.0f;
-          tot0[i] += mant * a0[i];
-          tot1[i] += mant * a1[i];
+        for (int grp = 0; grp < 4; ++grp) {       // 128 latent channels = two 64-channel steps
+          f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const int ks = 2 * grp + half;
+            const uint4 raw = *reinterpret_cast<const uint4*>((half ? lat1 : lat0) + 128 * grp);
+            const bf16x8 f0 = cvt8(raw.x, raw.y, pw[grp]);
+            const bf16x8 f1 = cvt8(raw.z, raw.w, pw[grp]);
+            mfma_s(a0, f0, qf[0][2 * ks]);
+            mfma_s(a1, f0, qf[1][2 * ks]);
+            mfma_s(a0, f1, qf[0][2 * ks + 1]);
+            mfma_s(a1, f1, qf[1][2 * ks + 1]);
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float mant = scale_mant(sclc[i * nblk + ((grp * nblk) >> 2)]);
+            tot0[i] += mant * a0[i];
+            tot1[i] += mant * a1[i];
+          }
         }
       }
       {
@@ -288,10 +325,9 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
 #pragma unroll
         for (int rs = 0; rs < 2; ++rs) {
           const bf16x8 f = *reinterpret_cast<const bf16x8*>(rope + (((4 * rs + kq) ^ r7) << 4));
-          mfma_qk(a0, f, qf[0][16 + rs]);
-          mfma_qk(a1, f, qf[1][16 + rs]);
+          mfma_s(a0, f, qf[0][16 + rs]);
+          mfma_s(a1, f, qf[1][16 + rs]);
         }
-        settle4(a0, a1);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           tot0[i] += a0[i];
@@ -301,75 +337,6 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       st[sj][0] = tot0;
       st[sj][1] = tot1;
     }
-    // lane (n = lane%16, gq = lane/16) holds keys 4gq+i of each sub-tile for heads n (st[.][0]) and 16+n
-    const int n = lane & 15, gq = lane >> 4;
-    float sv[SPW][2][4];
-    float mx[2] = {-INFINITY, -INFINITY};
-#pragma unroll
-    for (int sj = 0; sj < SPW; ++sj) {
-      const int4 kk = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * (sub0 + sj) + 4 * gq);
-      const bool ok[4] = {kk.x >= 0, kk.y >= 0, kk.z >= 0, kk.w >= 0};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sv[sj][0][i] = ok[i] ? st[sj][0][i] * qk_scale : -INFINITY;
-        sv[sj][1][i] = ok[i] ? st[sj][1][i] * qk_scale : -INFINITY;
-        mx[0] = fmaxf(mx[0], sv[sj][0][i]);
-        mx[1] = fmaxf(mx[1], sv[sj][1][i]);
-      }
-    }
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      mx[hh] = fmaxf(mx[hh], xor16(mx[hh]));
-      mx[hh] = fmaxf(mx[hh], xor32(mx[hh]));
-    }
-    // lazy running reference; consumers rescale their accumulators by fac before adding this tile
-    const bool grow = (mx[0] > m_run[0] + kLazy) || (mx[1] > m_run[1] + kLazy);
-    const bool any_grow = __ballot(grow) != 0ull;
-    if (any_grow) {
-      float fac[2];
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        const float m_new = (mx[hh] > m_run[hh] + kLazy) ? mx[hh] : m_run[hh];
-        fac[hh] = (m_run[hh] == -INFINITY) ? 0.0f : exp2f(m_run[hh] - m_new);
-        l_run[hh] *= fac[hh];
-        m_run[hh] = m_new;
-      }
-      if (lane < 16) {
-        facbuf[(par * 4 + wave) * 32 + n] = fac[0];
-        facbuf[(par * 4 + wave) * 32 + 16 + n] = fac[1];
-      }
-    }
-    if (lane == 0) flagbuf[par * 4 + wave] = any_grow ? 1 : 0;
-
-    // P (x V's block scale) -> LDS in the B-operand layout of the 32x32x16 product:
-    // lane (head, kq8 = key/8) owns 16 bytes = keys 8kq8..8kq8+7; this lane holds keys 4gq..4gq+3
-    const int variants = has_scale ? nblk : 1;
-    unsigned char* pbase = smem + G_::kPOff + par * G_::kPBytes;
-#pragma unroll
-    for (int sj = 0; sj < SPW; ++sj) {
-      float pr[2][4];
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pr[hh][i] = (sv[sj][hh][i] == -INFINITY) ? 0.0f : exp2f(sv[sj][hh][i] - m_run[hh]);
-          l_run[hh] += pr[hh][i];
-        }
-      const int slot_id = (sub0 + sj) * HG + hgq;
-      const float* scl = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * gq) * nblk;
-      for (int v = 0; v < variants; ++v) {
-        float sc[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) sc[i] = has_scale ? scl[i * nblk + v] : 1.0f;
-        unsigned char* dst = pbase + ((v * G_::kSlots + slot_id) * 64 + (gq >> 1) * 32) * 16 + (gq & 1) * 8;
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          const uint2 w = make_uint2(pack_bf16(pr[hh][0] * sc[0], pr[hh][1] * sc[1]),
-                                     pack_bf16(pr[hh][2] * sc[2], pr[hh][3] * sc[3]));
-          *reinterpret_cast<uint2*>(dst + (hh * 16 + n) * 16) = w;
-        }
-      }
-    }
   };
 
   // ---- value side state: o[4*dvb + producer] = O^T[32 channels x 32 heads] ----
@@ -378,7 +345,7 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   for (int i = 0; i < 16; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) o[i][j] = 0.0f;
-  const int pvar = has_scale ? (wave * nblk) >> 2 : 0;         // scale block of channels 128*wave..
+  const int pvar = (wave * nblk) >> 2;                         // scale block of channels 128*wave..
   int pv_off[4];                                               // transposing-read offsets per 32-channel block
   {
     const int t = lane & 15, half = (lane >> 4) & 1, kq2 = lane >> 5;
@@ -389,53 +356,182 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       pv_off[dvb] = r * kLat + ((c ^ (r & 7)) << 4) + 8 * (t & 1);
     }
   }
-  auto scale_acc = [&](int prod, float f) {                    // o[.][prod] *= f (per-lane factor)
+  // One pipeline stage: the value product of tile tv (8 steps of one V^T fragment and HG MFMAs)
+  // with the softmax of tile ts cut into pieces that run in the shadow of those MFMAs.
+  // do_s / do_v are uniform.
+  auto stage = [&](int tv, bool do_v, int ts, bool do_s) {
+    typedef __attribute__((ext_vector_type(2))) int i32x2;
+    const int n = lane & 15, gq = lane >> 4;
+    const unsigned char* vslot = smem + (tv & (kRing - 1)) * kSlotBytes;
+    const unsigned char* sslot = smem + (ts & (kRing - 1)) * kSlotBytes;
+    const int vpar = tv & 1, spar = ts & 1;
+    f32x4 st[SPW][2];
+    const unsigned char* pfrag = smem + G_::kPOff + vpar * G_::kPBytes + (pvar * G_::kSlots * 64 + lane) * 16;
+    unsigned char* pdst = smem + G_::kPOff + spar * G_::kPBytes;
+    float sv[SPW][2][4];
+    float pr[2][4];
+    float mx[2] = {-INFINITY, -INFINITY};
+    // V's block scales of this lane's keys (4gq + i of each sub-tile) and their validity: read once, up front
+    // (with two sub-tiles per wavefront there are no registers to spare: those read when needed)
+    constexpr bool kHoist = SPW == 1;
+    float vsc[SPW][4][nblk];
+    int4 kvalid[SPW];
+    auto read_scales = [&](int sj) {
+      const float* scl = reinterpret_cast<const float*>(sslot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * gq) * nblk;
 #pragma unroll
-    for (int dvb = 0; dvb < 4; ++dvb) {
-      __builtin_amdgcn_sched_barrier(0);
+      for (int i = 0; i < 4; ++i) {
+        if (nblk == 4) {
+          const float4 v4 = *reinterpret_cast<const float4*>(scl + 4 * i);
+          vsc[sj][i][0] = v4.x; vsc[sj][i][1 % nblk] = v4.y; vsc[sj][i][2 % nblk] = v4.z; vsc[sj][i][3 % nblk] = v4.w;
+        } else if (nblk == 2) {
+          const float2 v2 = *reinterpret_cast<const float2*>(scl + 2 * i);
+          vsc[sj][i][0] = v2.x; vsc[sj][i][1 % nblk] = v2.y;
+        } else {
+          vsc[sj][i][0] = scl[i];
+        }
+      }
+    };
+    if (do_s && kHoist) {
 #pragma unroll
-      for (int j = 0; j < 16; ++j) o[4 * dvb + prod][j] *= f;
-      asm volatile("" : "+a"(o[4 * dvb + prod]));
+      for (int sj = 0; sj < SPW; ++sj) {
+        kvalid[sj] = *reinterpret_cast<const int4*>(keys + ts * kTK + 16 * (sub0 + sj) + 4 * gq);
+        read_scales(sj);
+      }
     }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  auto value_tile = [&](int tau) {
-    const unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
-    const int par = tau & 1;
-    {
-      const int4 fl = *reinterpret_cast<const int4*>(flagbuf + par * 4);
-      const int f4[4] = {fl.x, fl.y, fl.z, fl.w};
-      bool any = false;
-#pragma unroll
-      for (int prod = 0; prod < 4; ++prod) any = any || (__builtin_amdgcn_readfirstlane(f4[prod]) != 0);
-      if (any) {
+    if (do_v) {                                   // producers moved their reference: rescale (rare)
+      const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
+      if (__builtin_amdgcn_readfirstlane(fl.x | fl.y | fl.z | fl.w) != 0) {
         mfma_settle_acc(o);
 #pragma unroll
-        for (int prod = 0; prod < 4; ++prod) {
-          if (__builtin_amdgcn_readfirstlane(f4[prod]) != 0) scale_acc(prod, facbuf[(par * 4 + prod) * 32 + (lane & 31)]);
+        for (int i = 0; i < 16; ++i) {
+          // one accumulator block at a time: the values pass through ordinary VGPRs
+          const float fsc = facbuf[(vpar * 4 + (i & 3)) * 32 + (lane & 31)];
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = 0; j < 16; ++j) o[i][j] *= fsc;
+          asm volatile("" : "+a"(o[i]));
         }
+        __builtin_amdgcn_sched_barrier(0);
         mfma_settle_acc(o);
       }
     }
-    const unsigned char* pbase = smem + G_::kPOff + par * G_::kPBytes + (pvar * G_::kSlots * 64 + lane) * 16;
+    bf16x8 pb[HG];
+    i32x2 vraw = {0, 0};
+    auto load_v = [&](int i) {                    // V^T fragment of step i = (k-step i/4, channel block i%4)
+      return __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) i32x2*)(vslot + 16 * (i >> 2) * kLat + pv_off[i & 3]));
+    };
+    auto load_p = [&](int kstep) {
 #pragma unroll
-    for (int kstep = 0; kstep < 2; ++kstep) {
-      bf16x8 pb[HG];
+      for (int hg = 0; hg < HG; ++hg) pb[hg] = *reinterpret_cast<const bf16x8*>(pfrag + (kstep * HG + hg) * 1024);
+    };
+    auto probs = [&](int sj) {                    // pr = exp2(score - reference), denominators
 #pragma unroll
-      for (int hg = 0; hg < HG; ++hg) pb[hg] = *reinterpret_cast<const bf16x8*>(pbase + (kstep * HG + hg) * 1024);
+      for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
-      for (int dvb = 0; dvb < 4; ++dvb) {
-        typedef __attribute__((ext_vector_type(2))) int i32x2;
-        const i32x2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-            (__attribute__((address_space(3))) i32x2*)(slot + 16 * kstep * kLat + pv_off[dvb]));
-        const bf16x8 a = cvt8((unsigned)raw[0], (unsigned)raw[1], 1.0f);
+        for (int i = 0; i < 4; ++i) {
+          pr[hh][i] = (sv[sj][hh][i] == -INFINITY) ? 0.0f : fast_exp2(sv[sj][hh][i] - m_run[hh]);
+          l_run[hh] += pr[hh][i];
+        }
+    };
+    // P (x V's block scale) -> LDS in the B-operand layout of the 32x32x16 product: lane
+    // (head, key/8) owns 16 bytes = 8 keys; this lane holds keys 4gq..4gq+3 of sub-tile sj
+    auto write_p = [&](int sj, int v0, int v1) {
+      const int slot_id = (sub0 + sj) * HG + hgq;
+#pragma unroll
+      for (int v = v0; v < v1; ++v) {
+        if (v >= nblk) break;
+        float sc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sc[i] = vsc[sj][i][v % nblk];
+        unsigned char* dst = pdst + ((v * G_::kSlots + slot_id) * 64 + (gq >> 1) * 32) * 16 + (gq & 1) * 8;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          const uint2 w = make_uint2(pack_bf16(pr[hh][0] * sc[0], pr[hh][1] * sc[1]),
+                                     pack_bf16(pr[hh][2] * sc[2], pr[hh][3] * sc[3]));
+          *reinterpret_cast<uint2*>(dst + (hh * 16 + n) * 16) = w;
+        }
+      }
+    };
+    auto softmax_piece = [&](int i) {
+      if (i == 0) {                               // mask, scale, local maxima
+#pragma unroll
+        for (int sj = 0; sj < SPW; ++sj) {
+          const int4 kk = kHoist ? kvalid[sj] : *reinterpret_cast<const int4*>(keys + ts * kTK + 16 * (sub0 + sj) + 4 * gq);
+          const bool ok[4] = {kk.x >= 0, kk.y >= 0, kk.z >= 0, kk.w >= 0};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sv[sj][0][e] = ok[e] ? st[sj][0][e] * qk_scale : -INFINITY;
+            sv[sj][1][e] = ok[e] ? st[sj][1][e] * qk_scale : -INFINITY;
+            mx[0] = fmaxf(mx[0], sv[sj][0][e]);
+            mx[1] = fmaxf(mx[1], sv[sj][1][e]);
+          }
+        }
+      } else if (i == 1) {                        // maxima across the four key quarters; lazy reference
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          mx[hh] = fmaxf(mx[hh], xor16(mx[hh]));
+          mx[hh] = fmaxf(mx[hh], xor32(mx[hh]));
+        }
+        const bool grow = (mx[0] > m_run[0] + kLazy) || (mx[1] > m_run[1] + kLazy);
+        const bool any_grow = __ballot(grow) != 0ull;
+        // accumulators of a head whose reference was -inf are still zero: nothing to rescale
+        const bool rescale = (mx[0] > m_run[0] + kLazy && m_run[0] != -INFINITY) || (mx[1] > m_run[1] + kLazy && m_run[1] != -INFINITY);
+        const bool any_rescale = __ballot(rescale) != 0ull;
+        if (any_grow) {                           // consumers rescale their accumulators by fac first
+          float fac[2];
+#pragma unroll
+          for (int hh = 0; hh < 2; ++hh) {
+            const float m_new = (mx[hh] > m_run[hh] + kLazy) ? mx[hh] : m_run[hh];
+            fac[hh] = (m_run[hh] == -INFINITY) ? 1.0f : exp2f(m_run[hh] - m_new);
+            l_run[hh] *= fac[hh];
+            m_run[hh] = m_new;
+          }
+          if (any_rescale && lane < 16) {
+            facbuf[(spar * 4 + wave) * 32 + n] = fac[0];
+            facbuf[(spar * 4 + wave) * 32 + 16 + n] = fac[1];
+          }
+        }
+        if (!any_rescale && lane < 32) facbuf[(spar * 4 + wave) * 32 + lane] = 1.0f;
+        if (lane == 0) flagbuf[spar * 4 + wave] = any_rescale ? 1 : 0;
+      } else if (i == 2) {
+        if (!kHoist) read_scales(0);
+        probs(0);
+      } else if (i == 3) {
+        write_p(0, 0, 2);
+      } else if (i == 4) {
+        write_p(0, 2, 4);
+      } else if (SPW == 2) {
+        if (i == 5) { read_scales(1); probs(1); }
+        else if (i == 6) write_p(1, 0, 2);
+        else write_p(1, 2, 4);
+      }
+    };
+    if (do_s) qk_tile(ts, st);
+    __builtin_amdgcn_sched_barrier(0);
+    if (do_v) {
+      load_p(0);
+      vraw = load_v(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_barrier(0);
+      i32x2 vnext = vraw;
+      if (do_v && i < 7) vnext = load_v(i + 1);
+      if (do_s) softmax_piece(i);
+      if (do_v) {
+        const bf16x8 a = cvt8((unsigned)vraw[0], (unsigned)vraw[1], 1.0f);
+        const int kstep = i >> 2, dvb = i & 3;
 #pragma unroll
         for (int hg = 0; hg < HG; ++hg) {
           const int prod = HG == 4 ? hg : hg + 2 * kstep;      // the wavefront that produced this P
           mfma_pv(o[4 * dvb + prod], a, pb[hg]);
         }
+        if (i == 3) load_p(1);
       }
+      vraw = vnext;
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- pipeline ----
@@ -444,13 +540,13 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   issue_tile(2);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  score_tile(0);
+  stage(0, false, 0, true);
   for (int t = 0; t < n_tiles; ++t) {
     wait_tiles_but_one();                         // tile t+1 (issued two iterations ago) has landed
     __syncthreads();                              // ... for every wavefront; P(t) is complete; PV(t-1) is done
     issue_tile(t + 3);                            // into the slot of tile t-1
-    if (t + 1 < n_tiles) score_tile(t + 1);
-    value_tile(t);
+    __builtin_amdgcn_sched_barrier(0);
+    stage(t, true, t + 1, t + 1 < n_tiles);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the prefetches past the end
   mfma_settle_acc(o);
@@ -581,6 +677,7 @@ bool sparse_mla_latent_supported(const MlaParams& p) {
   if (p.topk < 1 || (size_t)p.B * p.S == 0) return false;
   if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
   if (p.kv_scale && ((uintptr_t)p.kv_scale & 3)) return false;
+  if ((unsigned long long)p.B * p.Skv * p.G >= 0x7fffffffull) return false;   // cache rows are counted in 32 bits
   return true;
 }
 
@@ -614,15 +711,23 @@ int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream) {
   const long long wgs = (long long)p.B * p.S * p.G * p.num_splits * chunks;
   if (wgs > 0x7fffffffll || p.keys_per_split > kMaxKeys) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse MLA: launch too large");
   const dim3 grid((unsigned)wgs), block(256);
+  const int nblk = p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK ? kLat / p.kv_scale_block : 1;
+#define CM_LAUNCH_LATENT(HG_, NB_)                                                                                      \
+  do {                                                                                                                  \
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<HG_, NB_>,                                    \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, Geo<HG_>::kSmem));                      \
+    hipLaunchKernelGGL((sparse_mla_latent_kernel<HG_, NB_>), grid, block, Geo<HG_>::kSmem, stream, p);                   \
+  } while (0)
   if (hg == 4) {
-    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     Geo<4>::kSmem));
-    hipLaunchKernelGGL(sparse_mla_latent_kernel<4>, grid, block, Geo<4>::kSmem, stream, p);
+    if (nblk == 4) CM_LAUNCH_LATENT(4, 4);
+    else if (nblk == 2) CM_LAUNCH_LATENT(4, 2);
+    else CM_LAUNCH_LATENT(4, 1);
   } else {
-    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     Geo<2>::kSmem));
-    hipLaunchKernelGGL(sparse_mla_latent_kernel<2>, grid, block, Geo<2>::kSmem, stream, p);
+    if (nblk == 4) CM_LAUNCH_LATENT(2, 4);
+    else if (nblk == 2) CM_LAUNCH_LATENT(2, 2);
+    else CM_LAUNCH_LATENT(2, 1);
   }
+#undef CM_LAUNCH_LATENT
   CM_HIP_CHECK(hipGetLastError());
   return 0;
 }
