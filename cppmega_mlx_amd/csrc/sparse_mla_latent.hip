@@ -277,6 +277,10 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       // lane's row r); the mantissa part multiplies the partial sums, which this lane holds for
       // keys 4*(lane/16) + i
       const float* sclc = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * kq) * nblk;
+      auto load_k = [&](int ks) {                 // raw bytes of the 64-channel step ks
+        return *reinterpret_cast<const uint4*>(((ks & 1) ? lat1 : lat0) + 128 * (ks >> 1));
+      };
+      uint4 raw_a = load_k(0), raw_b = load_k(1);
       float pw[4];
       bool plain = true;                          // every scale of this row is a power of two
 #pragma unroll
@@ -285,54 +289,57 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
         pw[grp] = scale_pow2(sc);
         plain = plain && (pw[grp] == sc);
       }
+      const bool all_plain = __ballot(!plain) == 0ull;     // (uniform) no mantissa factors in this sub-tile
       f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
-      if (__ballot(!plain) == 0ull) {             // (uniform) one accumulation chain, no mantissa factors
+      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+      // software pipeline: step ks multiplies fragments converted during step ks-1 from bytes
+      // read during step ks-2
+      bf16x8 f0 = cvt8(raw_a.x, raw_a.y, pw[0]), f1 = cvt8(raw_a.z, raw_a.w, pw[0]);
+      bf16x8 rf0 = f0, rf1 = f0;                  // rope fragments (read during the last two steps)
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const uint4 raw = *reinterpret_cast<const uint4*>(((ks & 1) ? lat1 : lat0) + 128 * (ks >> 1));
-          const bf16x8 f0 = cvt8(raw.x, raw.y, pw[ks >> 1]);
-          const bf16x8 f1 = cvt8(raw.z, raw.w, pw[ks >> 1]);
-          mfma_s(tot0, f0, qf[0][2 * ks]);
-          mfma_s(tot1, f0, qf[1][2 * ks]);
-          mfma_s(tot0, f1, qf[0][2 * ks + 1]);
-          mfma_s(tot1, f1, qf[1][2 * ks + 1]);
+      for (int ks = 0; ks < 8; ++ks) {
+        uint4 raw_c = raw_b;
+        if (ks + 2 < 8) raw_c = load_k(ks + 2);
+        else if (ks == 6) rf0 = *reinterpret_cast<const bf16x8*>(rope + ((kq ^ r7) << 4));
+        else rf1 = *reinterpret_cast<const bf16x8*>(rope + (((4 + kq) ^ r7) << 4));
+        bf16x8 n0 = f0, n1 = f1;
+        if (ks + 1 < 8) {
+          n0 = cvt8(raw_b.x, raw_b.y, pw[(ks + 1) >> 1]);
+          n1 = cvt8(raw_b.z, raw_b.w, pw[(ks + 1) >> 1]);
         }
-      } else {
+        mfma_s(a0, f0, qf[0][2 * ks]);
+        mfma_s(a1, f0, qf[1][2 * ks]);
+        mfma_s(a0, f1, qf[0][2 * ks + 1]);
+        mfma_s(a1, f1, qf[1][2 * ks + 1]);
+        // one LDS read, then MFMA and conversion pairs alternating
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #pragma unroll
-        for (int grp = 0; grp < 4; ++grp) {       // 128 latent channels = two 64-channel steps
-          f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int ks = 2 * grp + half;
-            const uint4 raw = *reinterpret_cast<const uint4*>((half ? lat1 : lat0) + 128 * grp);
-            const bf16x8 f0 = cvt8(raw.x, raw.y, pw[grp]);
-            const bf16x8 f1 = cvt8(raw.z, raw.w, pw[grp]);
-            mfma_s(a0, f0, qf[0][2 * ks]);
-            mfma_s(a1, f0, qf[1][2 * ks]);
-            mfma_s(a0, f1, qf[0][2 * ks + 1]);
-            mfma_s(a1, f1, qf[1][2 * ks + 1]);
-          }
+        for (int q4 = 0; q4 < 4; ++q4) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        }
+        if ((ks & 1) && !all_plain) {             // end of a 128-channel block: apply its mantissa factors
+          const int grp = ks >> 1;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float mant = scale_mant(sclc[i * nblk + ((grp * nblk) >> 2)]);
             tot0[i] += mant * a0[i];
             tot1[i] += mant * a1[i];
+            a0[i] = 0.0f;
+            a1[i] = 0.0f;
           }
         }
+        f0 = n0; f1 = n1;
+        raw_b = raw_c;
       }
-      {
-        f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+      mfma_s(a0, rf0, qf[0][16]);
+      mfma_s(a1, rf0, qf[1][16]);
+      mfma_s(a0, rf1, qf[0][17]);
+      mfma_s(a1, rf1, qf[1][17]);
 #pragma unroll
-        for (int rs = 0; rs < 2; ++rs) {
-          const bf16x8 f = *reinterpret_cast<const bf16x8*>(rope + (((4 * rs + kq) ^ r7) << 4));
-          mfma_s(a0, f, qf[0][16 + rs]);
-          mfma_s(a1, f, qf[1][16 + rs]);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          tot0[i] += a0[i];
-          tot1[i] += a1[i];
-        }
+      for (int i = 0; i < 4; ++i) {
+        tot0[i] += a0[i];
+        tot1[i] += a1[i];
       }
       st[sj][0] = tot0;
       st[sj][1] = tot1;
@@ -391,13 +398,6 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
         }
       }
     };
-    if (do_s && kHoist) {
-#pragma unroll
-      for (int sj = 0; sj < SPW; ++sj) {
-        kvalid[sj] = *reinterpret_cast<const int4*>(keys + ts * kTK + 16 * (sub0 + sj) + 4 * gq);
-        read_scales(sj);
-      }
-    }
     if (do_v) {                                   // producers moved their reference: rescale (rare)
       const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
       if (__builtin_amdgcn_readfirstlane(fl.x | fl.y | fl.z | fl.w) != 0) {
@@ -509,6 +509,13 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
     };
     if (do_s) qk_tile(ts, st);
     __builtin_amdgcn_sched_barrier(0);
+    if (do_s && kHoist) {
+#pragma unroll
+      for (int sj = 0; sj < SPW; ++sj) {
+        kvalid[sj] = *reinterpret_cast<const int4*>(keys + ts * kTK + 16 * (sub0 + sj) + 4 * gq);
+        read_scales(sj);
+      }
+    }
     if (do_v) {
       load_p(0);
       vraw = load_v(0);
@@ -617,8 +624,8 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x16& acc = o[4 * dvb + hg];
-        const float4 v = make_float4(acc[4 * j] * out_scale, acc[4 * j + 1] * out_scale, acc[4 * j + 2] * out_scale,
-                                     acc[4 * j + 3] * out_scale);
+        float4 v = make_float4(acc[4 * j], acc[4 * j + 1], acc[4 * j + 2], acc[4 * j + 3]);
+        if (direct) v = make_float4(v.x * out_scale, v.y * out_scale, v.z * out_scale, v.w * out_scale);   // (uniform)
         *reinterpret_cast<float4*>(xbuf + hd * kXPitch + 32 * dvb + 8 * j + 4 * gq2) = v;
       }
     }
