@@ -12,12 +12,21 @@
 //    for all rows.  Per row a lane issues 16-byte weight loads, converts two
 //    bytes per instruction, accumulates in fp32 per 128-wide scale block, and
 //    the row sum is a wavefront reduction followed by a 4-way LDS combine.
-//  * 2 <= M <= 16 (skinny_mfma_kernel): the activation rows are the 16-wide N
-//    side of v_mfma_f32_16x16x32_bf16 (e4m3 -> bf16 is exact), the weight rows
-//    the M side; K is split across workgroups, partial sums go to a workspace
-//    and the last workgroup to finish a row tile adds them in a fixed order.
+//  * 2 <= M <= 4, bf16 activations (gemv_stream_kernel): the same streaming shape with the
+//    M activation rows held in registers and v_dot2_f32_bf16 accumulation.
+//  * 5 <= M <= 16, bf16 activations (skinny_mfma_kernel): v_mfma_f32_16x16x32_bf16 with 16
+//    weight rows as the M side and the (padded) activation rows as the N side.  A
+//    workgroup owns 16 weight rows; its 8 wavefronts own one eighth of K each and add
+//    their 16x16 partial tiles through LDS at the end, so nothing but the result is
+//    written to memory.  Weight fragments go from HBM straight into registers
+//    (16 bytes per lane and load: two MFMA k-steps, with the contraction order inside
+//    the 64-channel step permuted the same way for both operands) and are converted
+//    e4m3 -> bf16 with the 128-channel block scale applied in the conversion; the
+//    activations (L2-resident) are loaded per step.
 //  * anything else (odd K, misaligned rows): rowwise_kernel, one wavefront per
 //    output row, scalar byte loads.
+
+#include <cstdlib>
 
 #include "common.h"
 
@@ -282,6 +291,150 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
   }
 }
 
+// 5 <= M <= 16 with bf16 activations, K a multiple of 1024: see the file header.
+constexpr int kSkinnySplits = 8;         // K is cut into eighths, one per workgroup column
+constexpr int kSkinnyWaves = 7;          // 448 row tiles x 8 splits = 256 workgroups x 7 wavefronts x 2 tiles at N = 7168
+constexpr int kSkinnyDepth = 8;          // 64-channel weight steps in flight per wavefront
+constexpr int kSkinnyMaxKw = 2048;       // channels per split the LDS activation slice can hold
+constexpr int kXPitchBytes = kSkinnyMaxKw * 2 + 16;   // row pitch of the slice: 16 rows fall on distinct banks
+
+__global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const VecmatParams p) {
+  extern __shared__ __align__(16) unsigned char xs[];    // [16][kXPitchBytes]: bf16 activations of this split
+  const int lane = lane_id();
+  const int wave = (int)(threadIdx.x >> 6);
+  const int K = p.k;
+  const int kw = K / kSkinnySplits;                      // channels of this split (multiple of 128)
+  const int split = (int)blockIdx.y;
+  const int k0 = split * kw;
+  const int steps = kw / 64;
+  // activation slice -> LDS (rows >= M are zero)
+  for (int i = (int)threadIdx.x; i < 16 * (kw / 8); i += kSkinnyWaves * 64) {
+    const int m = i / (kw / 8), c = i % (kw / 8);
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (m < p.m) v = *reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k0 + 8 * c);
+    *reinterpret_cast<uint4*>(xs + m * kXPitchBytes + 16 * c) = v;
+  }
+  __syncthreads();
+
+  const int r16 = lane & 15, kq = lane >> 4;
+  const unsigned char* xrow = xs + r16 * kXPitchBytes + 32 * kq;        // B fragments: activation r16, channels 16kq.. of a step
+  const int tiles = (p.n + 15) / 16;
+  // this wavefront's tiles: first, first + 7, ...; their steps form one continuous stream so the
+  // weight prefetch never drains between tiles
+  const int first = (int)blockIdx.x * p.rows_per_wg + wave;
+  const int tile_end = min(tiles, ((int)blockIdx.x + 1) * p.rows_per_wg);
+  const int my_tiles = first < tile_end ? (tile_end - first + kSkinnyWaves - 1) / kSkinnyWaves : 0;
+  const int total = my_tiles * steps;
+  // prefetch cursor: next weight bytes / scale of this lane, advanced step by step
+  int pf_tile = first, pf_st = 0;
+  const unsigned char* pf_w = nullptr;
+  const float* pf_s = nullptr;
+  auto pf_seek = [&]() {                                 // (per tile) row of this lane in tile pf_tile
+    const int n = min(pf_tile * 16 + r16, p.n - 1);
+    pf_w = p.w + (size_t)n * K + k0 + 16 * kq;
+    pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
+  };
+  auto pf_next = [&](uint4& wdst, float& sdst, bool with_scale) {
+    wdst = *reinterpret_cast<const uint4*>(pf_w + 64 * pf_st);
+    if (with_scale) sdst = pf_s[(size_t)(pf_st >> 1) * p.scol_stride];
+    if (++pf_st == steps) {                              // (uniform)
+      pf_st = 0;
+      pf_tile += kSkinnyWaves;
+      if (pf_tile < tile_end) pf_seek();
+    }
+  };
+  uint4 wq[kSkinnyDepth];
+  float sq[kSkinnyDepth / 2];                            // one scale per 128 channels = two steps
+  if (total > 0) {
+    pf_seek();
+#pragma unroll
+    for (int d = 0; d < kSkinnyDepth; ++d) {
+      if (d < total) pf_next(wq[d], sq[d >> 1], (d & 1) == 0);
+      else { wq[d] = make_uint4(0, 0, 0, 0); if ((d & 1) == 0) sq[d >> 1] = 1.0f; }
+    }
+  }
+  float sq_next[kSkinnyDepth / 2];
+#pragma unroll
+  for (int i = 0; i < kSkinnyDepth / 2; ++i) sq_next[i] = 1.0f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  int st = 0, tile = first;                              // position of flat step f0 + d, tracked incrementally
+  for (int f0 = 0; f0 < total; f0 += kSkinnyDepth) {     // steps is a multiple of the depth? not required: see the guards
+#pragma unroll
+    for (int d = 0; d < kSkinnyDepth; ++d) {
+      const int f = f0 + d;
+      const uint4 wv = wq[d];
+      const float sc = sq[d >> 1];
+      float sc_next = sc;
+      if (f + kSkinnyDepth < total) pf_next(wq[d], sc_next, (d & 1) == 0);
+      if ((d & 1) == 0) sq_next[d >> 1] = sc_next;       // takes effect once the odd step of the pair is done
+      else sq[d >> 1] = sq_next[d >> 1];
+      if (f < total) {                                   // (uniform)
+        const uint4 x0 = *reinterpret_cast<const uint4*>(xrow + 128 * st);
+        const uint4 x1 = *reinterpret_cast<const uint4*>(xrow + 128 * st + 16);
+        bf16x8 a0, a1;
+        const bool pow2 = (__float_as_uint(sc) & 0x007fffffu) == 0u && sc > 0.0f && sc < INFINITY;
+        if (__ballot(!pow2) == 0ull) {                   // the conversion applies a power-of-two scale exactly
+          const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.x, sc, false));
+          const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.x, sc, true));
+          const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.y, sc, false));
+          const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.y, sc, true));
+          const unsigned o4 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.z, sc, false));
+          const unsigned o5 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.z, sc, true));
+          const unsigned o6 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.w, sc, false));
+          const unsigned o7 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.w, sc, true));
+          a0 = __builtin_bit_cast(bf16x8, make_uint4(o0, o1, o2, o3));
+          a1 = __builtin_bit_cast(bf16x8, make_uint4(o4, o5, o6, o7));
+        } else {                                         // general scale: fp32 multiply, round to bf16
+          const unsigned wd[4] = {wv.x, wv.y, wv.z, wv.w};
+          unsigned o[8];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const f32x2 lo = e4m3x2_lo(wd[i]), hi = e4m3x2_hi(wd[i]);
+            typedef __attribute__((ext_vector_type(2))) __bf16 v2;
+            v2 r0, r1;
+            r0[0] = (__bf16)(lo[0] * sc); r0[1] = (__bf16)(lo[1] * sc);
+            r1[0] = (__bf16)(hi[0] * sc); r1[1] = (__bf16)(hi[1] * sc);
+            o[2 * i] = __builtin_bit_cast(unsigned, r0);
+            o[2 * i + 1] = __builtin_bit_cast(unsigned, r1);
+          }
+          a0 = __builtin_bit_cast(bf16x8, make_uint4(o[0], o[1], o[2], o[3]));
+          a1 = __builtin_bit_cast(bf16x8, make_uint4(o[4], o[5], o[6], o[7]));
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, x0), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, x1), acc, 0, 0, 0);
+        if (++st == steps) {                             // (uniform) tile finished: partial[split][m][row]
+          // lane (m = lane%16, g = lane/16) holds weight rows 4g + i of activation m
+          const int row0 = tile * 16;
+          if (r16 < p.m) {
+            float* dst = p.partial + ((size_t)split * p.m + r16) * p.n + row0 + 4 * kq;
+            if (row0 + 4 * kq + 3 < p.n && (p.n & 3) == 0) {
+              *reinterpret_cast<float4*>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            } else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (row0 + 4 * kq + i < p.n) dst[i] = acc[i];
+            }
+          }
+          acc = f32x4{0.f, 0.f, 0.f, 0.f};
+          st = 0;
+          tile += kSkinnyWaves;
+        }
+      }
+    }
+  }
+}
+
+// out[m][n] = sum over the K splits of partial[split][m][n], in split order
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const VecmatParams p) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t total = (size_t)p.m * p.n;
+  if (i >= total) return;
+  float s = 0.0f;
+#pragma unroll
+  for (int z = 0; z < kSkinnySplits; ++z) s += p.partial[(size_t)z * total + i];
+  store_as(p.out, i, p.out_dtype, s);
+}
+
 // Any shape: one wavefront per output row, all M activations in turn.
 __global__ __launch_bounds__(256) void rowwise_kernel(const VecmatParams p) {
   const int lane = lane_id();
@@ -326,9 +479,25 @@ static int validate(const cppmega_mi355_vecmat_args_t& a) {
   return 0;
 }
 
+static bool vecmat_aligned(const cppmega_mi355_vecmat_args_t& a) {
+  const size_t xelt = (size_t)dtype_size(a.x_dtype);
+  return (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) && (((size_t)a.k * xelt) % 16 == 0);
+}
+static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) {
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 4096 == 0) && a.k <= 16384;
+}
+// the split-K MFMA kernel: bf16 activations, 2 <= M <= 16, K in eighths of whole scale blocks that fit the LDS slice
+static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 2 && a.m <= 16 && !stream_shape(a) &&
+         (a.k % (kSkinnySplits * 128) == 0) && a.k / kSkinnySplits <= kSkinnyMaxKw;
+}
+static bool skinny_ok(const cppmega_mi355_vecmat_args_t& a) { return vecmat_aligned(a) && skinny_shape(a); }
+
 int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes) {
   if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "vecmat: bytes is NULL");
-  *bytes = 0;
+  // pointers may be absent in a sizing call: decided from the shape alone (a misaligned call then
+  // simply does not use the workspace)
+  *bytes = skinny_shape(a) ? (size_t)kSkinnySplits * a.m * a.n * sizeof(float) : 0;
   return 0;
 }
 
@@ -343,10 +512,8 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   rc = fill_scale_layout(a, p);
   if (rc) return rc;
 
-  const size_t xelt = (size_t)dtype_size(a.x_dtype);
-  const bool aligned = (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) &&
-                       (((size_t)a.k * xelt) % 16 == 0);
-  const bool stream_ok = aligned && a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 4096 == 0) && a.k <= 16384;
+  const bool aligned = vecmat_aligned(a);
+  const bool stream_ok = aligned && stream_shape(a);
   if (stream_ok) {
     const dim3 grid((unsigned)((a.n + kStreamRows - 1) / kStreamRows)), block(kGemvWaves * 64);
     const int ch = a.k / 4096;
@@ -362,6 +529,22 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     else if (a.m == 3) CM_STREAM(3, 2);
     else CM_STREAM(4, 2);
 #undef CM_STREAM
+  } else if (skinny_ok(a)) {
+    const size_t need = (size_t)kSkinnySplits * a.m * a.n * sizeof(float);
+    if (!a.workspace || a.workspace_bytes < need)
+      return fail(CPPMEGA_MI355_ERR_WORKSPACE, "vecmat: workspace of %zu bytes needed, %zu given", need, (size_t)a.workspace_bytes);
+    p.partial = (float*)a.workspace;
+    // row tiles per workgroup: about one workgroup per CU and split, a multiple of the wavefront count
+    const int tiles = (a.n + 15) / 16;
+    int per_wave = (tiles * kSkinnySplits + 256 * kSkinnyWaves - 1) / (256 * kSkinnyWaves);
+    if (per_wave < 1) per_wave = 1;
+    p.rows_per_wg = per_wave * kSkinnyWaves;
+    const dim3 grid((unsigned)((tiles + p.rows_per_wg - 1) / p.rows_per_wg), kSkinnySplits), block(kSkinnyWaves * 64);
+    const int smem = 16 * kXPitchBytes;
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    hipLaunchKernelGGL(skinny_mfma_kernel, grid, block, smem, stream, p);
+    CM_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(skinny_reduce_kernel, dim3((unsigned)(((size_t)a.m * a.n + 255) / 256)), dim3(256), 0, stream, p);
   } else if (a.m == 1 && aligned) {
     // rows per workgroup: keep at least ~3 workgroups per CU in the grid
     int rows = 16;
