@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   const int key_begin = split * p.keys_per_split;
   const int key_end = min(p.topk, key_begin + p.keys_per_split);
   const int n_keys = max(0, key_end - key_begin);
-  const int n_tiles = (n_keys + kTK - 1) / kTK;
+  const int list_tiles = (n_keys + kTK - 1) / kTK;   // tiles the index list spans; trailing all-skipped tiles are dropped below
 
   constexpr int nblk = NBLK;
   const bool has_scale = p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;   // otherwise the scale area holds ones
@@ -162,13 +162,26 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   float* stats = reinterpret_cast<float*>(smem + G_::kStatOff);
 
   // ---- cache rows of this split's keys -> LDS (-1 = skipped) ----
-  for (int i = tid; i < n_tiles * kTK + 4 * kTK; i += 256) {
-    int row = -1;
-    if (i < n_keys) {
-      const long long k = load_index(p, idx_base + key_begin + i);
-      if (k >= 0 && k < p.Skv) row = (int)k;
+  int* last_valid = reinterpret_cast<int*>(smem);          // (ring memory, not yet in use)
+  if (tid == 0) *last_valid = -1;
+  __syncthreads();
+  {
+    int mine = -1;
+    for (int i = tid; i < list_tiles * kTK + 4 * kTK; i += 256) {
+      int row = -1;
+      if (i < n_keys) {
+        const long long k = load_index(p, idx_base + key_begin + i);
+        if (k >= 0 && k < p.Skv) { row = (int)k; mine = i; }
+      }
+      keys[i] = row;
     }
-    keys[i] = row;
+    mine = max(mine, __shfl_xor(mine, 1, 64));
+    mine = max(mine, __shfl_xor(mine, 2, 64));
+    mine = max(mine, __shfl_xor(mine, 4, 64));
+    mine = max(mine, __shfl_xor(mine, 8, 64));
+    mine = max(mine, __shfl_xor(mine, 16, 64));
+    mine = max(mine, __shfl_xor(mine, 32, 64));
+    if (lane == 0 && mine >= 0) atomicMax(last_valid, mine);
   }
 
   // ---- Q^T fragments: lane (head n = lane%16, kq = lane/16), heads n and 16+n of group hgq.
@@ -205,6 +218,9 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       reinterpret_cast<float*>(smem + (i / kTK) * kSlotBytes + kLatBytes + kRopeBytes)[i % kTK] = 1.0f;
   }
   __syncthreads();                                // keys[] is complete
+  // causal padding puts the skipped (-1) slots at the end of a list: tiles past the last valid key do nothing
+  const int n_tiles = __builtin_amdgcn_readfirstlane((*last_valid + kTK) / kTK);
+  __syncthreads();                                // everyone has read it before the ring is written
 
   // ---- HBM -> LDS: this wavefront brings rows 8*wave .. 8*wave+7 of a tile.  A skipped key
   //      fetches cache row 0 instead (its probability is zero), so every wavefront issues
