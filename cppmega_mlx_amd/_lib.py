@@ -40,6 +40,7 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_sparse_mla_workspace_bytes",
     "cppmega_mi355_sparse_mla_fwd",
     "cppmega_mi355_sparse_mla_select_kernel",
+    "cppmega_mi355_sparse_mla_scores",
     "cppmega_mi355_fp8_vecmat_workspace_bytes",
     "cppmega_mi355_fp8_vecmat",
 )
@@ -186,6 +187,8 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_sparse_mla_workspace_bytes.restype = C.c_int
         lib.cppmega_mi355_sparse_mla_select_kernel.argtypes = [C.POINTER(SparseMlaArgs), C.c_size_t]
         lib.cppmega_mi355_sparse_mla_select_kernel.restype = C.c_int
+        lib.cppmega_mi355_sparse_mla_scores.argtypes = [C.POINTER(SparseMlaArgs), C.c_size_t, C.c_void_p, C.c_void_p]
+        lib.cppmega_mi355_sparse_mla_scores.restype = C.c_int
         lib.cppmega_mi355_fp8_vecmat.argtypes = [C.POINTER(VecmatArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_fp8_vecmat.restype = C.c_int
         lib.cppmega_mi355_fp8_vecmat_workspace_bytes.argtypes = [

@@ -35,7 +35,7 @@ static bool is_float_carrier(int dt) {
 }
 
 // Validates the request and fills the kernel parameter block.
-static int build_mla_params(const cppmega_mi355_sparse_mla_args_t& a, MlaParams& p, bool need_pointers) {
+static int build_mla_params(const cppmega_mi355_sparse_mla_args_t& a, MlaParams& p, bool need_pointers, bool need_out = true) {
   if (a.batch < 0 || a.seq_q < 0 || a.heads < 1 || a.kv_groups < 1 || a.seq_kv < 0 || a.topk < 0)
     return fail(CPPMEGA_MI355_ERR_SHAPE, "sparse_mla: negative or empty dimension");
   if (a.heads % a.kv_groups != 0)
@@ -66,13 +66,13 @@ static int build_mla_params(const cppmega_mi355_sparse_mla_args_t& a, MlaParams&
     }
   }
   if (need_pointers) {
-    if (!a.q || !a.kv || !a.indices || !a.out) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla: q/kv/indices/out is NULL");
+    if (!a.q || !a.kv || !a.indices || (need_out && !a.out)) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla: q/kv/indices/out is NULL");
     if (a.q_scale_kind != CPPMEGA_MI355_SCALE_NONE && !a.q_scale) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla: q_scale is NULL");
     if (a.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE && !a.kv_scale) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla: kv_scale is NULL");
     if (a.rope_dim > 0 && !a.kv_rope) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla: kv_rope is NULL");
   }
   p.q = a.q; p.q_scale = a.q_scale; p.kv = a.kv; p.kv_scale = a.kv_scale; p.rope = a.kv_rope;
-  p.indices = a.indices; p.sinks = a.sinks; p.out = a.out; p.lse = a.lse; p.workspace = a.workspace;
+  p.indices = a.indices; p.sinks = a.sinks; p.out = a.out; p.lse = a.lse; p.workspace = a.workspace; p.scores = nullptr;
   p.q_dtype = a.q_dtype; p.q_scale_kind = a.q_scale_kind; p.q_scale_block = a.q_scale_block > 0 ? a.q_scale_block : a.d_qk;
   p.kv_dtype = a.kv_dtype; p.kv_scale_kind = a.kv_scale_kind; p.kv_scale_block = a.kv_scale_block > 0 ? a.kv_scale_block : d_kv;
   p.rope_dtype = a.rope_dtype; p.rope_dim = a.rope_dim; p.index_dtype = a.index_dtype; p.out_dtype = a.out_dtype;
@@ -195,6 +195,17 @@ int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, si
     return sparse_mla_mfma_launch(p, (hipStream_t)stream);
   }
   return sparse_mla_scalar_launch(p, (hipStream_t)stream);
+}
+
+int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size, float* scores,
+                                    void* stream) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_sparse_mla_args_t);
+  if (!scores) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla_scores: scores is NULL");
+  MlaParams p;
+  const int rc = build_mla_params(*args, p, true, false);
+  if (rc) return rc;
+  p.scores = scores;
+  return sparse_mla_scores_launch(p, (hipStream_t)stream);
 }
 
 int cppmega_mi355_fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t* args, size_t args_size,

@@ -16,6 +16,7 @@ struct MlaParams {
   void* out;
   float* lse;
   void* workspace;
+  float* scores;        // score-only entry point: [B, S, H, topk] fp32
   int q_dtype, q_scale_kind, q_scale_block;
   int kv_dtype, kv_scale_kind, kv_scale_block;
   int rope_dtype, rope_dim;
@@ -45,6 +46,7 @@ __device__ __forceinline__ float row_scale(const void* scale, int kind, size_t r
 }
 
 int sparse_mla_scalar_launch(const MlaParams& p, hipStream_t stream);
+int sparse_mla_scores_launch(const MlaParams& p, hipStream_t stream);
 int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream);
 bool sparse_mla_mfma_supported(const MlaParams& p);
 size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p);

@@ -142,6 +142,54 @@ __global__ __launch_bounds__(64) void sparse_mla_scalar_kernel(const MlaParams p
   if (p.lse && lane == 0) p.lse[bsh] = l > 0.0f ? m + logf(l) : 0.0f;
 }
 
+// Scores only: scores[b, s, h, j] = sm_scale * q . key(indices[b, s, g, j]) in fp32; a skipped slot
+// (index < 0 or >= Skv) holds the most negative finite fp32 value.  One wavefront per (b, s, h).
+template <int KVDT>
+__global__ __launch_bounds__(64) void sparse_mla_scores_kernel(const MlaParams p) {
+  extern __shared__ __align__(16) float smem[];
+  float* qf = smem;                       // [d_qk]
+  const int lane = lane_id();
+  const size_t bsh = blockIdx.x;
+  const int h = (int)(bsh % p.H);
+  const size_t bs = bsh / p.H;
+  const int b = (int)(bs / p.S);
+  const int g = h / p.heads_per_group;
+  const size_t idx_base = (bs * p.G + g) * (size_t)p.topk;
+  {
+    const int qblk = p.q_scale_kind == CPPMEGA_MI355_SCALE_NONE || p.q_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN
+                         ? p.d_qk : p.q_scale_block;
+    const int nblk = (p.d_qk + qblk - 1) / qblk;
+    for (int d = lane; d < p.d_qk; d += 64) {
+      const float sc = row_scale(p.q_scale, p.q_scale_kind, bsh, nblk, d / qblk);
+      qf[d] = load_as(p.q, bsh * p.d_qk + d, p.q_dtype) * sc;
+    }
+  }
+  __syncthreads();
+  const int kblk = (p.kv_scale_kind == CPPMEGA_MI355_SCALE_NONE || p.kv_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN)
+                       ? p.d_kv : p.kv_scale_block;
+  const int nkblk = (p.d_kv + kblk - 1) / kblk;
+  for (int jj = lane; jj < p.topk; jj += 64) {
+    const long long key = load_index(p, idx_base + jj);
+    float score = -3.4028234663852886e38f;
+    if (key >= 0 && key < p.Skv) {
+      const size_t krow = ((size_t)b * p.Skv + (size_t)key) * p.G + g;
+      float dot = 0.0f;
+      for (int kb = 0; kb < nkblk; ++kb) {
+        const int d0 = kb * kblk, d1 = min(d0 + kblk, p.d_kv);
+        const float sc = row_scale(p.kv_scale, p.kv_scale_kind, krow, nkblk, kb);
+        dot = fmaf(sc, dot_span<KVDT>(p.kv, krow * p.d_kv, qf, d0, d1), dot);
+      }
+      if (p.rope_dim > 0) {
+        const size_t roff = krow * p.rope_dim;
+        for (int d = 0; d < p.rope_dim; ++d)
+          dot = fmaf(qf[p.d_kv + d], load_as(p.rope, roff + d, p.rope_dtype), dot);
+      }
+      score = dot * p.sm_scale;
+    }
+    p.scores[bsh * p.topk + jj] = score;
+  }
+}
+
 template <int KVDT>
 int launch_dv(const MlaParams& p, hipStream_t stream) {
   const dim3 grid((unsigned)((size_t)p.B * p.S * p.H)), block(64);
@@ -175,6 +223,22 @@ int sparse_mla_scalar_launch(const MlaParams& p, hipStream_t stream) {
     default: return fail(CPPMEGA_MI355_ERR_DTYPE, "sparse_mla: kv dtype %d", p.kv_dtype);
   }
   if (rc) return rc;
+  CM_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int sparse_mla_scores_launch(const MlaParams& p, hipStream_t stream) {
+  if ((size_t)p.B * p.S * p.H == 0 || p.topk == 0) return 0;
+  if (p.d_qk > 8192) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla: d_qk %d exceeds 8192", p.d_qk);
+  const dim3 grid((unsigned)((size_t)p.B * p.S * p.H)), block(64);
+  const size_t smem = (size_t)p.d_qk * 4;
+  switch (p.kv_dtype) {
+    case CPPMEGA_MI355_F32: hipLaunchKernelGGL(sparse_mla_scores_kernel<CPPMEGA_MI355_F32>, grid, block, smem, stream, p); break;
+    case CPPMEGA_MI355_F16: hipLaunchKernelGGL(sparse_mla_scores_kernel<CPPMEGA_MI355_F16>, grid, block, smem, stream, p); break;
+    case CPPMEGA_MI355_BF16: hipLaunchKernelGGL(sparse_mla_scores_kernel<CPPMEGA_MI355_BF16>, grid, block, smem, stream, p); break;
+    case CPPMEGA_MI355_E4M3: hipLaunchKernelGGL(sparse_mla_scores_kernel<CPPMEGA_MI355_E4M3>, grid, block, smem, stream, p); break;
+    default: return fail(CPPMEGA_MI355_ERR_DTYPE, "sparse_mla: kv dtype %d", p.kv_dtype);
+  }
   CM_HIP_CHECK(hipGetLastError());
   return 0;
 }

@@ -27,7 +27,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ... import _lib
+from ... import _lib, ops
 from . import _prepared
 
 __all__ = [
@@ -37,6 +37,7 @@ __all__ = [
     "sparse_mla_blockscaled_path_c_apply",
     "sparse_mla_blockscaled_path_c_apply_direct",
     "sparse_mla_blockscaled_path_c_status",
+    "blockscaled_sparse_mla_qk_reduce_path_c",
 ]
 
 E8M0_BLOCK_SIZE = _prepared.E8M0_BLOCK_SIZE
@@ -141,3 +142,46 @@ def sparse_mla_blockscaled_path_c_apply(
             f"sparse_mla_blockscaled_path_c_apply: kernel dispatch failed: {type(exc).__name__}: {exc}"
         ) from exc
     return (out, lse) if return_lse else out
+
+
+E8M0_BLOCK_SIZE = 32
+
+
+def blockscaled_sparse_mla_qk_reduce_path_c(A_fp8, A_scale, B_fp8, B_scale, *, outputs_per_block: int = 4,
+                                            reduce_threads: int = 32, vec: int = 4):
+    """``(1, N)`` float32 scores of one E8M0 block-scaled query row ``A_fp8 u8[1,K]`` (scales
+    ``u8[K/32]``) against ``B_fp8 u8[N,K]`` (scales ``u8[K/32]`` broadcast or ``u8[N,K/32]``):
+    reference ``sparse_mla_blockscaled_path_c.py:883-932``, validation ``:820-880``.
+    Returns ``None`` when no gfx950 device is usable.  The schedule keywords are ignored."""
+    if A_fp8.ndim != 2 or A_fp8.shape[0] != 1:
+        raise ValueError(f"A_fp8 must have shape (1, K); got {tuple(A_fp8.shape)}")
+    if B_fp8.ndim != 2:
+        raise ValueError(f"B_fp8 must have shape (N, K); got {tuple(B_fp8.shape)}")
+    if A_fp8.dtype != torch.uint8 or B_fp8.dtype != torch.uint8:
+        raise ValueError(f"A_fp8/B_fp8 must be uint8 e4m3 storage; got {A_fp8.dtype}, {B_fp8.dtype}")
+    if A_scale.dtype != torch.uint8 or B_scale.dtype != torch.uint8:
+        raise TypeError(f"A_scale/B_scale must be uint8 E8M0 storage; got {A_scale.dtype}, {B_scale.dtype}")
+    n, k = int(B_fp8.shape[0]), int(A_fp8.shape[1])
+    if n <= 0 or k <= 0 or int(B_fp8.shape[1]) != k:
+        raise ValueError(f"A_fp8/B_fp8 shape mismatch: A={tuple(A_fp8.shape)}, B={tuple(B_fp8.shape)}")
+    if k % E8M0_BLOCK_SIZE != 0:
+        raise ValueError(f"E8M0 QK reducer requires K divisible by {E8M0_BLOCK_SIZE}; got K={k}")
+    blocks = k // E8M0_BLOCK_SIZE
+    if A_scale.numel() != blocks:
+        raise ValueError(f"A_scale must contain K/{E8M0_BLOCK_SIZE}={blocks} E8M0 bytes; got shape {tuple(A_scale.shape)}")
+    if B_scale.numel() not in (blocks, n * blocks):
+        raise ValueError(
+            f"B_scale must contain K/{E8M0_BLOCK_SIZE}={blocks} broadcast bytes or N*K/{E8M0_BLOCK_SIZE}={n * blocks} "
+            f"row-block bytes; got shape {tuple(B_scale.shape)}")
+    if not sparse_mla_blockscaled_path_c_status().available:
+        return None
+    # one query, one head, N keys in order: the score-only attention kernel with identity indices
+    b_rows = B_scale.reshape(1, blocks).expand(n, blocks).contiguous() if B_scale.numel() == blocks else B_scale.reshape(n, blocks)
+    q = A_fp8.reshape(1, 1, 1, k)
+    kv = B_fp8.reshape(1, n, 1, k)
+    idx = torch.arange(n, dtype=torch.int32, device=A_fp8.device).reshape(1, 1, 1, n)
+    scores = torch.empty((1, 1, 1, n), dtype=torch.float32, device=A_fp8.device)
+    ops.sparse_mla_scores(q, kv, idx, sm_scale=1.0, scores=scores,
+                          q_spec=ops.QuantSpec(_lib.SCALE_E8M0, A_scale.reshape(1, 1, 1, blocks), E8M0_BLOCK_SIZE),
+                          kv_spec=ops.QuantSpec(_lib.SCALE_E8M0, b_rows.reshape(1, n, 1, blocks), E8M0_BLOCK_SIZE))
+    return scores.reshape(1, n)

@@ -19,7 +19,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ... import _lib
+from ... import _lib, ops
 from . import _prepared
 
 __all__ = [
@@ -28,6 +28,8 @@ __all__ = [
     "sparse_mla_fp8_path_c_apply",
     "sparse_mla_fp8_path_c_apply_direct",
     "sparse_mla_fp8_path_c_status",
+    "fp8_sparse_mla_indexed_qk_reduce_path_c",
+    "fp8_sparse_mla_qk_reduce_path_c",
 ]
 
 _OP = "FP8 Sparse-MLA Path C apply"
@@ -156,3 +158,55 @@ def sparse_mla_fp8_path_c_apply(
             f"sparse_mla_fp8_path_c_apply: kernel dispatch failed: {type(exc).__name__}: {exc}"
         ) from exc
     return (out, lse) if return_lse else out
+
+
+# invalid slots of the score-only kernels hold this finite sentinel
+# (reference sparse_mla_fp8_path_c.py:80)
+_SMFP8_INVALID_SCORE_SENTINEL = -3.4028234663852886e38
+
+
+def fp8_sparse_mla_qk_reduce_path_c(A_fp8, A_scale, B_fp8, B_scale, *, outputs_per_block=None, reduce_threads=None,
+                                    vec=None):
+    """``(1, N)`` float32 scores ``(dec(B) . dec(A)) * A_scale * B_scale`` for one query row
+    ``A_fp8 u8[1,K]`` against ``B_fp8 u8[N,K]`` (reference :1548-1608; validation :1419-1462).
+    ``A_scale`` holds one float32, ``B_scale`` one or N.  Returns ``None`` when no gfx950
+    device is usable.  The schedule keywords are accepted and ignored."""
+    if A_fp8.ndim != 2 or A_fp8.shape[0] != 1:
+        raise ValueError(f"A_fp8 must have shape (1, K); got {tuple(A_fp8.shape)}")
+    if B_fp8.ndim != 2:
+        raise ValueError(f"B_fp8 must have shape (N, K); got {tuple(B_fp8.shape)}")
+    if A_fp8.dtype != torch.uint8 or B_fp8.dtype != torch.uint8:
+        raise ValueError(f"A_fp8/B_fp8 must be uint8 e4m3 storage; got {A_fp8.dtype}, {B_fp8.dtype}")
+    n, k = int(B_fp8.shape[0]), int(A_fp8.shape[1])
+    if n <= 0 or k <= 0 or int(B_fp8.shape[1]) != k:
+        raise ValueError(f"A_fp8/B_fp8 shape mismatch: A={tuple(A_fp8.shape)}, B={tuple(B_fp8.shape)}")
+    if A_scale.numel() != 1:
+        raise ValueError(f"A_scale must contain exactly one FP32 scale; got shape {tuple(A_scale.shape)}")
+    if B_scale.numel() not in (1, n):
+        raise ValueError(f"B_scale must contain one scalar scale or N={n} row scales; got shape {tuple(B_scale.shape)}")
+    if A_scale.dtype != torch.float32 or B_scale.dtype != torch.float32:
+        raise TypeError(f"A_scale/B_scale must be float32; got {A_scale.dtype}, {B_scale.dtype}")
+    if not sparse_mla_fp8_path_c_status().available:
+        return None
+    out = torch.empty((1, n), dtype=torch.float32, device=A_fp8.device)
+    kind = _lib.WSCALE_SCALAR if B_scale.numel() == 1 else _lib.WSCALE_PER_ROW
+    ops.fp8_vecmat(A_fp8, B_fp8, B_scale.reshape(-1), out=out, scale_x=A_scale.reshape(1), scale_w_kind=kind)
+    return out
+
+
+def fp8_sparse_mla_indexed_qk_reduce_path_c(q_fp8, q_scale, kv_fp8, kv_scale, indices, *, sm_scale,
+                                            outputs_per_block=None, reduce_threads=None, vec=None):
+    """``scores[B,S,H,TOPK]`` float32 of the per-token-scaled FP8 layout (reference :1611-1690;
+    validation :1465-1545): ``sm_scale * q_scale * kv_scale * (dec(q) . dec(kv[index]))``; a slot
+    whose index is negative or >= S_kv holds the finite sentinel -3.4028234663852886e38.
+    Returns ``None`` when no gfx950 device is usable."""
+    plan = _prepared.plan_prepared(q_fp8, q_scale, kv_fp8, kv_scale, indices, d_v=None, kv_rope=None,
+                                   op_name="FP8 Sparse-MLA indexed QK reducer", family="fp8")
+    if q_fp8.dtype != torch.uint8:
+        raise ValueError(f"q_fp8/kv_fp8 must be uint8 e4m3 storage; got {q_fp8.dtype}, {kv_fp8.dtype}")
+    if not sparse_mla_fp8_path_c_status().available:
+        return None
+    scores = torch.empty((plan.batch, plan.seq_len, plan.heads, int(indices.shape[-1])), dtype=torch.float32,
+                         device=q_fp8.device)
+    return ops.sparse_mla_scores(q_fp8, kv_fp8, indices, sm_scale=float(sm_scale), scores=scores,
+                                 q_spec=plan.q_spec, kv_spec=plan.kv_spec)

@@ -195,6 +195,40 @@ def sparse_mla_forward(
     return out, lse
 
 
+def sparse_mla_scores(
+    q: torch.Tensor,
+    kv: torch.Tensor,
+    indices: torch.Tensor,
+    *,
+    sm_scale: float,
+    scores: torch.Tensor,
+    q_spec: QuantSpec | None = None,
+    kv_spec: QuantSpec | None = None,
+    kv_rope: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """scores[b,s,h,j] = sm_scale * q . key(indices[b,s,g,j]) into caller-owned float32
+    ``scores`` [B,S,H,topk]; skipped slots hold the most negative finite float32."""
+    q_spec = q_spec or QuantSpec()
+    kv_spec = kv_spec or QuantSpec()
+    for name, t in (("q", q), ("kv", kv), ("indices", indices), ("scores", scores), ("kv_rope", kv_rope),
+                    ("q_scale", q_spec.scale), ("kv_scale", kv_spec.scale)):
+        if t is not None:
+            _lib.require_device_tensor(t, name, q if name != "q" else None)
+    if q.ndim != 4 or kv.ndim != 4 or indices.ndim != 4:
+        raise ValueError("sparse_mla: q, kv and indices must be rank 4")
+    B, S, H, _ = q.shape
+    want = (B, S, H, indices.shape[-1])
+    if tuple(scores.shape) != want or scores.dtype != torch.float32:
+        raise ValueError(f"scores must be float32 with shape {want}; got {scores.dtype} {tuple(scores.shape)}")
+    d_kv = kv.shape[-1]
+    a = _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_kv, None, None, None, "scalar")
+    with torch.cuda.device(q.device):
+        rc = _lib.load().cppmega_mi355_sparse_mla_scores(C.byref(a), C.sizeof(a), scores.data_ptr(),
+                                                         _lib.current_stream(q.device))
+    _lib.check(rc, "sparse_mla_scores")
+    return scores
+
+
 def sparse_mla_workspace_bytes(q, kv, indices, *, d_v, q_spec=None, kv_spec=None, kv_rope=None, kernel="auto") -> int:
     a = _fill_mla_args(q, q_spec or QuantSpec(), kv, kv_spec or QuantSpec(), kv_rope, indices, 1.0, d_v, None,
                        None, None, kernel)

@@ -196,6 +196,15 @@ int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, si
 int cppmega_mi355_sparse_mla_select_kernel(const cppmega_mi355_sparse_mla_args_t* args,
                                            size_t args_size);
 
+/* Scores only: scores[b, s, h, j] = sm_scale * q . key(indices[b, s, g, j]), float32
+ * [B, S, H, topk]; a skipped slot holds -3.4028234663852886e38 (the most negative
+ * finite float32).  Replaces the QK-only kernels the reference keeps as test seams:
+ * fp8_sparse_mla_indexed_qk_reduce_path_c
+ * (cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:1611-1690, sentinel :80).
+ * `out`, `lse`, `sinks`, `d_v` (any valid value) and `workspace` of args are ignored. */
+int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size,
+                                    float* scores, void* stream);
+
 /* ---- FP8 vecmat / skinny GEMM ----------------------------------------------
  * Replaces fp8_vecmat_reduce_direct, called as kernel(A, A_scale, B, B_scale, C)
  * (cppmega_mlx/nn/_tilelang/fp8_vecmat_path_c.py:737-821, 1039-1046) and the

@@ -150,3 +150,28 @@ def dequant_block_latent(codes: np.ndarray, scale: np.ndarray, rope: np.ndarray 
     if rope is None:
         return lat
     return np.concatenate([lat, np.asarray(rope, dtype=np.float64)], axis=-1)
+
+
+INVALID_SCORE_SENTINEL = np.float32(-3.4028234663852886e38)
+
+
+def sparse_mla_scores_oracle(q: np.ndarray, kv: np.ndarray, indices: np.ndarray, *, sm_scale: float) -> np.ndarray:
+    """scores[b,s,h,j] = sm_scale * q[b,s,h] . kv[b, indices[b,s,g,j], g] in float64 -> float32; a slot
+    whose index is negative or >= S_kv holds the finite sentinel.  Follows the score stage of the
+    reference's fused kernel and its QK-only seam
+    (cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:1862-1884, sentinel :80)."""
+    B, S, H, D = q.shape
+    _, Skv, G, _ = kv.shape
+    topk = indices.shape[-1]
+    hpg = H // G
+    out = np.empty((B, S, H, topk), dtype=np.float32)
+    for b in range(B):
+        for s in range(S):
+            for g in range(G):
+                idx = indices[b, s, g]
+                ok = (idx >= 0) & (idx < Skv)
+                rows = kv[b, np.where(ok, idx, 0), g].astype(np.float64)            # [topk, D]
+                qs = q[b, s, g * hpg:(g + 1) * hpg].astype(np.float64)               # [hpg, D]
+                sc = (qs @ rows.T) * float(sm_scale)
+                out[b, s, g * hpg:(g + 1) * hpg] = np.where(ok[None, :], sc, INVALID_SCORE_SENTINEL).astype(np.float32)
+    return out

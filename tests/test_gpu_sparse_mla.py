@@ -283,3 +283,42 @@ def test_tiny_bf16_config(device):
             assert (idx[0, 0, 0] >= 0).sum() == 1                    # first query sees one key: out == that V row
             np.testing.assert_allclose(out[0, 0].float().cpu().numpy(), np.broadcast_to(kvf[0, idx[0, 0, 0, 0], 0, :512], (16, 512)),
                                        atol=2e-2, rtol=1e-2)
+
+
+def test_score_only_entry_points(device):
+    """QK-only seams: per-token FP8 indexed scores, the (1, N) FP8 reducer and the E8M0 reducer."""
+    rng = np.random.default_rng(91)
+    B, S, H, G, Skv, topk, D = 2, 3, 8, 2, 50, 20, 64
+    qc, qs = fp8.quantize_per_token(rng.standard_normal((B, S, H, D)).astype(np.float32))
+    kc, ks = fp8.quantize_per_token(rng.standard_normal((B, Skv, G, D)).astype(np.float32))
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[..., -3:] = -1
+    idx[0, 0, 0, 0] = Skv + 5
+    want = om.sparse_mla_scores_oracle(om.dequant_per_token(qc, qs), om.dequant_per_token(kc, ks), idx, sm_scale=0.125)
+    got = f8.fp8_sparse_mla_indexed_qk_reduce_path_c(to_dev(qc, device), to_dev(qs, device), to_dev(kc, device),
+                                                     to_dev(ks, device), to_dev(idx.astype(np.int32), device), sm_scale=0.125)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    bad = want == om.INVALID_SCORE_SENTINEL
+    assert (got[bad] == om.INVALID_SCORE_SENTINEL).all()
+    np.testing.assert_allclose(got[~bad], want[~bad], rtol=1e-5, atol=1e-5)
+
+    N, K = 37, 128
+    a, a_s = fp8.quantize_per_token(rng.standard_normal((1, K)).astype(np.float32))
+    bm, b_s = fp8.quantize_per_token(rng.standard_normal((N, K)).astype(np.float32))
+    want2 = (fp8.e4m3_decode(bm).astype(np.float64) @ fp8.e4m3_decode(a[0]).astype(np.float64)) * float(a_s[0]) * b_s.astype(np.float64)
+    got2 = f8.fp8_sparse_mla_qk_reduce_path_c(to_dev(a, device), to_dev(a_s.reshape(1), device), to_dev(bm, device), to_dev(b_s, device))
+    torch.cuda.synchronize()
+    assert tuple(got2.shape) == (1, N)
+    np.testing.assert_allclose(got2.cpu().numpy()[0], want2, rtol=1e-5, atol=1e-5)
+
+    ac, ab = fp8.quantize_mxfp8(rng.standard_normal((1, K)).astype(np.float32))
+    bc, bb = fp8.quantize_mxfp8(rng.standard_normal((N, K)).astype(np.float32))
+    want3 = om.dequant_e8m0(bc, bb).astype(np.float64) @ om.dequant_e8m0(ac, ab)[0].astype(np.float64)
+    got3 = bs.blockscaled_sparse_mla_qk_reduce_path_c(to_dev(ac, device), to_dev(ab.reshape(-1), device), to_dev(bc, device), to_dev(bb, device))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(got3.cpu().numpy()[0], want3, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        f8.fp8_sparse_mla_qk_reduce_path_c(to_dev(a, device), to_dev(a_s.reshape(1), device), to_dev(bm[:, :64].copy(), device), to_dev(b_s, device))
+    with pytest.raises(TypeError):
+        bs.blockscaled_sparse_mla_qk_reduce_path_c(to_dev(ac, device), to_dev(ab.reshape(-1).astype(np.float32), device), to_dev(bc, device), to_dev(bb, device))
