@@ -43,6 +43,7 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_sparse_mla_scores",
     "cppmega_mi355_fp8_vecmat_workspace_bytes",
     "cppmega_mi355_fp8_vecmat",
+    "cppmega_mi355_fp8_quantize",
 )
 
 
@@ -145,6 +146,23 @@ class VecmatArgs(C.Structure):
     ]
 
 
+class QuantizeArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("x_dtype", C.c_int32),
+        ("x", C.c_void_p),
+        ("rows", C.c_int64),
+        ("k", C.c_int32),
+        ("mode", C.c_int32),
+        ("codes", C.c_void_p),
+        ("scale", C.c_void_p),
+        ("recovered", C.c_void_p),
+        ("scratch", C.c_void_p),
+    ]
+
+
+QUANT_PER_TOKEN, QUANT_PER_TENSOR, QUANT_MXFP8, DEQUANT_PER_TOKEN, DEQUANT_MXFP8 = range(5)
+
 _lock = threading.RLock()
 _lib: C.CDLL | None = None
 
@@ -191,6 +209,8 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_sparse_mla_scores.restype = C.c_int
         lib.cppmega_mi355_fp8_vecmat.argtypes = [C.POINTER(VecmatArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_fp8_vecmat.restype = C.c_int
+        lib.cppmega_mi355_fp8_quantize.argtypes = [C.POINTER(QuantizeArgs), C.c_size_t, C.c_void_p]
+        lib.cppmega_mi355_fp8_quantize.restype = C.c_int
         lib.cppmega_mi355_fp8_vecmat_workspace_bytes.argtypes = [
             C.POINTER(VecmatArgs), C.c_size_t, C.POINTER(C.c_size_t)]
         lib.cppmega_mi355_fp8_vecmat_workspace_bytes.restype = C.c_int

@@ -15,6 +15,8 @@ from .fp8_vecmat_path_c import (
 )
 from .fused_fp8_gemm import fused_fp8_gemm
 from .sparse_mla import sparse_mla_apply
+from .sparse_mla_blockscaled import sparse_mla_blockscaled_apply, sparse_mla_blockscaled_reference
+from .sparse_mla_fp8 import sparse_mla_fp8_apply, sparse_mla_fp8_reference
 from .sparse_mla_blockscaled_path_c import (
     sparse_mla_blockscaled_path_c_apply,
     sparse_mla_blockscaled_path_c_apply_direct,
@@ -38,6 +40,10 @@ __all__ = [
     "fp8_vecmat_path_c_status",
     "fused_fp8_gemm",
     "sparse_mla_apply",
+    "sparse_mla_blockscaled_apply",
+    "sparse_mla_blockscaled_reference",
+    "sparse_mla_fp8_apply",
+    "sparse_mla_fp8_reference",
     "sparse_mla_blockscaled_path_c_apply",
     "sparse_mla_blockscaled_path_c_apply_direct",
     "sparse_mla_fp8_path_c_apply",

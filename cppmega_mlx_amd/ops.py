@@ -293,3 +293,83 @@ def fp8_vecmat(
         rc = lib.cppmega_mi355_fp8_vecmat(C.byref(a), C.sizeof(a), stream)
     _lib.check(rc, "fp8_vecmat")
     return out
+
+
+# ---------------------------------------------------------------------------
+# FP8 producers
+# ---------------------------------------------------------------------------
+
+_QUANT_MODES = {"per_token": _lib.QUANT_PER_TOKEN, "per_tensor": _lib.QUANT_PER_TENSOR, "mxfp8": _lib.QUANT_MXFP8}
+_scratch_words: dict[int, torch.Tensor] = {}
+
+
+def _scratch_word(device: torch.device) -> torch.Tensor:
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    buf = _scratch_words.get(key)
+    if buf is None:
+        buf = torch.zeros(1, dtype=torch.int32, device=device)
+        _scratch_words[key] = buf
+    return buf
+
+
+def fp8_quantize(x: torch.Tensor, mode: str, *, codes: torch.Tensor | None = None, scale: torch.Tensor | None = None,
+                 recovered: torch.Tensor | None = None):
+    """Quantise ``x[..., K]`` to e4m3 into caller-owned buffers (any subset of them):
+    ``codes`` uint8 like x; ``scale`` float32 ``x.shape[:-1]`` (per_token / per_tensor) or uint8
+    ``[..., K/32]`` (mxfp8); ``recovered`` = dec(codes) * scale in x's dtype."""
+    if mode not in _QUANT_MODES:
+        raise ValueError(f"unknown quantiser mode {mode!r}")
+    _lib.require_device_tensor(x, "x", None)
+    if not x.is_contiguous():
+        raise ValueError("fp8_quantize: x must be contiguous")
+    k = int(x.shape[-1])
+    rows = x.numel() // k if k else 0
+    for name, t, dt, shape in (
+        ("codes", codes, torch.uint8, tuple(x.shape)),
+        ("scale", scale, torch.uint8 if mode == "mxfp8" else torch.float32,
+         tuple(x.shape[:-1]) + (k // 32,) if mode == "mxfp8" else tuple(x.shape[:-1])),
+        ("recovered", recovered, x.dtype, tuple(x.shape)),
+    ):
+        if t is None:
+            continue
+        _lib.require_device_tensor(t, name, x)
+        if t.dtype != dt or tuple(t.shape) != shape or not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous {dt} with shape {shape}; got {t.dtype} {tuple(t.shape)}")
+    a = _lib.QuantizeArgs()
+    a.struct_size = C.sizeof(a)
+    a.x_dtype = _dtype_or_raise(x, "x", (_lib.F32, _lib.F16, _lib.BF16))
+    a.x = x.data_ptr()
+    a.rows, a.k, a.mode = rows, k, _QUANT_MODES[mode]
+    a.codes, a.scale, a.recovered = _lib.ptr(codes), _lib.ptr(scale), _lib.ptr(recovered)
+    if mode == "per_tensor":
+        a.scratch = _scratch_word(x.device).data_ptr()
+    with torch.cuda.device(x.device):
+        rc = _lib.load().cppmega_mi355_fp8_quantize(C.byref(a), C.sizeof(a), _lib.current_stream(x.device))
+    _lib.check(rc, "fp8_quantize")
+    return codes, scale, recovered
+
+
+def fp8_dequantize(codes: torch.Tensor, scale: torch.Tensor, *, out: torch.Tensor) -> torch.Tensor:
+    """out = dec(codes) * scale; ``scale`` float32 ``codes.shape[:-1]`` or E8M0 uint8 ``[..., K/32]``."""
+    for name, t in (("codes", codes), ("scale", scale), ("out", out)):
+        _lib.require_device_tensor(t, name, codes if name != "codes" else None)
+    k = int(codes.shape[-1])
+    if codes.dtype != torch.uint8 or tuple(out.shape) != tuple(codes.shape) or not (codes.is_contiguous() and out.is_contiguous()):
+        raise ValueError("fp8_dequantize: codes must be contiguous uint8 and out a contiguous tensor of the same shape")
+    if scale.dtype == torch.uint8:
+        mode, want = _lib.DEQUANT_MXFP8, tuple(codes.shape[:-1]) + (k // 32,)
+    elif scale.dtype == torch.float32:
+        mode, want = _lib.DEQUANT_PER_TOKEN, tuple(codes.shape[:-1])
+    else:
+        raise TypeError(f"scale must be float32 (per row) or uint8 (E8M0 per 32); got {scale.dtype}")
+    if tuple(scale.shape) != want or not scale.is_contiguous():
+        raise ValueError(f"scale must be contiguous with shape {want}; got {tuple(scale.shape)}")
+    a = _lib.QuantizeArgs()
+    a.struct_size = C.sizeof(a)
+    a.x_dtype = _dtype_or_raise(out, "out", (_lib.F32, _lib.F16, _lib.BF16))
+    a.rows, a.k, a.mode = (codes.numel() // k if k else 0), k, mode
+    a.codes, a.scale, a.recovered = codes.data_ptr(), scale.data_ptr(), out.data_ptr()
+    with torch.cuda.device(codes.device):
+        rc = _lib.load().cppmega_mi355_fp8_quantize(C.byref(a), C.sizeof(a), _lib.current_stream(codes.device))
+    _lib.check(rc, "fp8_dequantize")
+    return out

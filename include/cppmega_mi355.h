@@ -245,6 +245,44 @@ int cppmega_mi355_fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t* 
 
 int cppmega_mi355_fp8_vecmat(const cppmega_mi355_vecmat_args_t* args, size_t args_size, void* stream);
 
+/* ---- FP8 producers ------------------------------------------------------------
+ * The quantisers that write the prepared buffers of the attention entry points, and the
+ * matching dequantiser:
+ *   PER_TOKEN   fp8_per_token_quant(x, fp8, scale)
+ *               (cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:2667-2753):
+ *               scale[row] = max(amax(row) * (1/448), 1e-12), code = rne(clamp(x / scale, +-448))
+ *   PER_TENSOR  _to_fp8_with_per_tensor_scale (sparse_mla_fp8.py:123-145): one amax over
+ *               the tensor, the scale replicated per row
+ *   MXFP8       _quantize_mxfp8 (sparse_mla_blockscaled.py:60-76): one E8M0 byte per 32
+ *               channels, byte = clamp(127 + ceil(log2(amax/448)), 1, 254)
+ *   DEQUANT_*   _from_fp8_with_scale (sparse_mla_fp8.py:148-157) / _dequantize_mxfp8
+ *               (sparse_mla_blockscaled.py:79-87): recovered = dec(codes) * scale
+ * x is [rows, k] float32/float16/bfloat16, dense.  Any of codes / scale / recovered may be
+ * NULL in a quantise call (at least one is not); `recovered` receives dec(code) * scale in
+ * x's dtype.  PER_TENSOR needs `scratch`, 4 bytes of device memory. */
+enum {
+  CPPMEGA_MI355_QUANT_PER_TOKEN = 0,
+  CPPMEGA_MI355_QUANT_PER_TENSOR = 1,
+  CPPMEGA_MI355_QUANT_MXFP8 = 2,
+  CPPMEGA_MI355_DEQUANT_PER_TOKEN = 3,   /* codes + float32 scale[rows] -> recovered */
+  CPPMEGA_MI355_DEQUANT_MXFP8 = 4        /* codes + uint8 scale[rows, k/32] -> recovered */
+};
+
+typedef struct cppmega_mi355_quantize_args {
+  uint32_t struct_size;
+  int32_t x_dtype;            /* F32/F16/BF16: dtype of x and of recovered          */
+  const void* x;              /* [rows, k]; unused by the DEQUANT modes             */
+  int64_t rows;
+  int32_t k;
+  int32_t mode;               /* CPPMEGA_MI355_QUANT_* / DEQUANT_*                   */
+  uint8_t* codes;             /* [rows, k] e4m3 bytes (output; input of DEQUANT)    */
+  void* scale;                /* float32 [rows] or uint8 [rows, k/32]               */
+  void* recovered;            /* [rows, k] in x_dtype                               */
+  void* scratch;              /* 4 bytes, PER_TENSOR only                           */
+} cppmega_mi355_quantize_args_t;
+
+int cppmega_mi355_fp8_quantize(const cppmega_mi355_quantize_args_t* args, size_t args_size, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -85,17 +85,42 @@ def e4m3_encode(values: np.ndarray) -> np.ndarray:
 
 
 def quantize_per_token(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
-    """Per-row (last axis) amax quantiser: scale = max(amax/448, 1e-12).
+    """Per-row (last axis) amax quantiser in float32 arithmetic, as the producer kernel
+    states it: scale = max(amax * float32(1/448), 1e-12); code = rne(clamp(x / scale, +-448)).
 
-    Follows the producer kernel contract of
-    cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:2683-2709.
+    Follows cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:2683-2709.
     Returns (codes uint8 [..., K], scale float32 [...]).
     """
     x = np.asarray(x, dtype=np.float32)
-    amax = np.max(np.abs(x), axis=-1)
-    scale = np.maximum(amax / np.float32(E4M3_MAX), np.float32(1e-12)).astype(np.float32)
-    codes = e4m3_encode(x.astype(np.float64) / scale[..., None].astype(np.float64))
-    return codes, scale
+    amax = np.max(np.abs(x), axis=-1).astype(np.float32)
+    scale = np.maximum(amax * np.float32(1.0 / 448.0), np.float32(1e-12)).astype(np.float32)
+    norm = np.clip((x / scale[..., None]).astype(np.float32), np.float32(-E4M3_MAX), np.float32(E4M3_MAX))
+    return e4m3_encode(norm), scale
+
+
+def quantize_per_tensor(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """One amax scale for the whole tensor, replicated per row: the float-carrier producer
+    cppmega_mlx/nn/_tilelang/sparse_mla_fp8.py:123-145 (scale = max(amax/448, 1e-12), float32
+    arithmetic).  The rounding of ``mx.to_fp8`` is not in the tree (parity unpinned); this uses
+    round-to-nearest-even with saturation like the per-token producer kernel."""
+    x = np.asarray(x, dtype=np.float32)
+    amax = np.float32(np.max(np.abs(x))) if x.size else np.float32(0)
+    scale = np.maximum(amax * np.float32(1.0 / 448.0), np.float32(1e-12)).astype(np.float32)
+    norm = np.clip((x / scale).astype(np.float32), np.float32(-E4M3_MAX), np.float32(E4M3_MAX))
+    return e4m3_encode(norm), np.full(x.shape[:-1], scale, dtype=np.float32)
+
+
+def roundtrip_per_tensor(x: np.ndarray) -> np.ndarray:
+    """dec(quantize_per_tensor(x)) * scale in float32 (sparse_mla_fp8.py:160-166)."""
+    codes, scale = quantize_per_tensor(x)
+    return (e4m3_decode(codes) * scale[..., None]).astype(np.float32)
+
+
+def roundtrip_mxfp8(x: np.ndarray) -> np.ndarray:
+    """dec(quantize_mxfp8(x)) * 2^(byte-127) in float32 (sparse_mla_blockscaled.py:90-98)."""
+    codes, byte = quantize_mxfp8(x)
+    sc = np.repeat(e8m0_decode(byte), 32, axis=-1)
+    return (e4m3_decode(codes) * sc).astype(np.float32)
 
 
 def quantize_block(x: np.ndarray, block: int = 128, pow2: bool = True) -> tuple[np.ndarray, np.ndarray]:

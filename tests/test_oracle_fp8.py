@@ -90,3 +90,34 @@ def test_bf16_round_matches_torch():
     x = (rng.standard_normal(10000) * 10).astype(np.float32)
     want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
     np.testing.assert_array_equal(fp8.bf16_round(x), want)
+
+
+def test_producer_quantisers_closed_forms():
+    """Scales and codes of the producer restatements on inputs whose answer is known in closed form."""
+    x = np.zeros((3, 64), dtype=np.float32)
+    x[0, :4] = [448.0, -224.0, 1.0, 0.0]          # amax 448 -> scale 1 -> codes are the values' own bytes
+    x[1, :2] = [2.0, -1.0]                        # amax 2 -> scale 2/448; 2 -> 448 (0x7E), -1 -> -224 (0xF6)
+    codes, scale = fp8.quantize_per_token(x)
+    assert scale[0] == np.float32(448.0) * np.float32(1.0 / 448.0)
+    assert list(codes[0, :4]) == [0x7E, 0xF6, 0x38, 0x00]
+    assert list(codes[1, :2]) == [0x7E, 0xF6]
+    assert scale[2] == np.float32(1e-12) and not codes[2].any()      # all-zero row: floor scale, zero bytes
+    tcodes, tscale = fp8.quantize_per_tensor(x)
+    assert (tscale == tscale.flat[0]).all() and tscale.shape == (3,)
+    assert list(tcodes[1, :2]) == [0x40, 0xB8]    # with the tensor amax 448: 2 -> 0x40, -1 -> 0xB8
+    # the round trip is a projection: quantising it again changes nothing
+    rng = np.random.default_rng(0)
+    y = rng.standard_normal((5, 96)).astype(np.float32)
+    r = fp8.roundtrip_per_tensor(y)
+    np.testing.assert_array_equal(fp8.roundtrip_per_tensor(r), r)
+    assert np.abs(r - y).max() <= np.abs(y).max() / 448.0 * 16.0      # half an ulp of the top binade (ulp 32 at 448)
+    # MXFP8: 448 * 2^e is the largest amax a block with exponent e holds
+    z = np.zeros((1, 96), dtype=np.float32)
+    z[0, 0] = 448.0
+    z[0, 32] = 448.0 * 2.0 ** -5
+    z[0, 64] = np.nextafter(np.float32(448.0), np.float32(1e9))
+    mcodes, mbytes = fp8.quantize_mxfp8(z)
+    assert list(mbytes[0]) == [127, 122, 128]
+    assert mcodes[0, 0] == 0x7E and mcodes[0, 32] == 0x7E and mcodes[0, 64] == 0x76   # 448.00003/2 = 224 -> 0x76
+    rm = fp8.roundtrip_mxfp8(y)
+    np.testing.assert_array_equal(fp8.roundtrip_mxfp8(rm), rm)
