@@ -161,29 +161,6 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   int* flagbuf = reinterpret_cast<int*>(smem + G_::kFlagOff);
   float* stats = reinterpret_cast<float*>(smem + G_::kStatOff);
 
-  // ---- cache rows of this split's keys -> LDS (-1 = skipped) ----
-  int* last_valid = reinterpret_cast<int*>(smem);          // (ring memory, not yet in use)
-  if (tid == 0) *last_valid = -1;
-  __syncthreads();
-  {
-    int mine = -1;
-    for (int i = tid; i < list_tiles * kTK + 4 * kTK; i += 256) {
-      int row = -1;
-      if (i < n_keys) {
-        const long long k = load_index(p, idx_base + key_begin + i);
-        if (k >= 0 && k < p.Skv) { row = (int)k; mine = i; }
-      }
-      keys[i] = row;
-    }
-    mine = max(mine, __shfl_xor(mine, 1, 64));
-    mine = max(mine, __shfl_xor(mine, 2, 64));
-    mine = max(mine, __shfl_xor(mine, 4, 64));
-    mine = max(mine, __shfl_xor(mine, 8, 64));
-    mine = max(mine, __shfl_xor(mine, 16, 64));
-    mine = max(mine, __shfl_xor(mine, 32, 64));
-    if (lane == 0 && mine >= 0) atomicMax(last_valid, mine);
-  }
-
   // ---- Q^T fragments: lane (head n = lane%16, kq = lane/16), heads n and 16+n of group hgq.
   //      latent step ks (64 channels): fragments 2ks, 2ks+1 hold channels 64ks + 16kq + {0..7}, {8..15};
   //      rope step r: fragment 16+r holds channels 512 + 32r + 8kq + {0..7} ----
@@ -213,6 +190,29 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       }
     }
   }
+  // ---- cache rows of this split's keys -> LDS (-1 = skipped) ----
+  int* last_valid = reinterpret_cast<int*>(smem);          // (ring memory, not yet in use)
+  if (tid == 0) *last_valid = -1;
+  __syncthreads();
+  {
+    int mine = -1;
+    for (int i = tid; i < list_tiles * kTK + 4 * kTK; i += 256) {
+      int row = -1;
+      if (i < n_keys) {
+        const long long k = load_index(p, idx_base + key_begin + i);
+        if (k >= 0 && k < p.Skv) { row = (int)k; mine = i; }
+      }
+      keys[i] = row;
+    }
+    mine = max(mine, __shfl_xor(mine, 1, 64));
+    mine = max(mine, __shfl_xor(mine, 2, 64));
+    mine = max(mine, __shfl_xor(mine, 4, 64));
+    mine = max(mine, __shfl_xor(mine, 8, 64));
+    mine = max(mine, __shfl_xor(mine, 16, 64));
+    mine = max(mine, __shfl_xor(mine, 32, 64));
+    if (lane == 0 && mine >= 0) atomicMax(last_valid, mine);
+  }
+
   if (!has_scale) {                               // no scales in memory: every slot's scale area is 1.0 for good
     for (int i = tid; i < kRing * kTK; i += 256)
       reinterpret_cast<float*>(smem + (i / kTK) * kSlotBytes + kLatBytes + kRopeBytes)[i % kTK] = 1.0f;
