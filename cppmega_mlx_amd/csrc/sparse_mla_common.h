@@ -55,6 +55,7 @@ void sparse_mla_mfma_plan(MlaParams& p);
 // shared-tile kernel for FP8 latent caches (sparse_mla_latent.hip); dispatched by the *_mfma_* functions
 bool sparse_mla_latent_supported(const MlaParams& p);
 void sparse_mla_latent_plan(MlaParams& p);
-int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream);
+int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream);   // includes its combine step
+size_t sparse_mla_latent_workspace_bytes(const MlaParams& p);
 
 }  // namespace cm

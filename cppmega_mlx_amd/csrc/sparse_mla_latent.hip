@@ -38,8 +38,9 @@
 //   pipeline     iteration t: barrier; issue tile t+3; QK + softmax of tile t+1;
 //                PV of tile t.
 //
-// Key splits write fp32 partials and (max, sum) per head to the workspace; the
-// combine kernel of sparse_mla_mfma.hip finishes them.
+// Key splits write their fp32 accumulators to the workspace exactly as the lanes hold them
+// (1 KiB per store), plus (max, sum) per head; sparse_mla_latent_combine_kernel merges the
+// splits and does the transposition to [head][channel] that the single-split path does in LDS.
 
 #include <cstdlib>
 
@@ -62,6 +63,7 @@ constexpr int kRingBytes = kRing * kSlotBytes;  // 83968
 constexpr int kMaxKeys = 2048;                  // keys of one split (their rows are staged in LDS)
 constexpr int kKeyInts = kMaxKeys + 4 * kTK;    // + the tiles the pipeline prefetches past the end
 constexpr int kXPitch = 132;                    // floats per head row of the output transpose (128 + 4)
+constexpr int kPartFloats = 4 * 16 * 64 * 4;         // partial floats of one 32-head group: [4 wavefronts][16 rows][64 lanes][4]
 constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
 
 template <int HG>
@@ -593,6 +595,9 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   const bool direct = p.num_splits == 1;
   float* xbuf = reinterpret_cast<float*>(smem) + wave * 32 * kXPitch;     // private to this wavefront
   const size_t q_index = bs;
+  // key-split partials: one block per (query, KV group, head chunk, split)
+  const size_t part_block = (size_t)(((long long)bs * p.G + g) * chunks + chunk) * p.num_splits + split;
+  const size_t part_blocks_total = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
 #pragma unroll
   for (int hg = 0; hg < HG; ++hg) {
     float m_all, l_all;
@@ -634,14 +639,34 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
         out_scale = 0.0f;
       }
     }
+    if (!direct) {
+      // key split: the unnormalised accumulators leave exactly as the lanes hold them (1 KiB per
+      // store instruction); the combine kernel knows the layout and does the transposition
+      float* blk = (float*)p.workspace + part_block * (size_t)(HG * kPartFloats) +
+                   ((size_t)((wave * HG + hg) * 16) * 64 + lane) * 4;
+#pragma unroll
+      for (int dvb = 0; dvb < 4; ++dvb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x16& acc = o[4 * dvb + hg];
+          *reinterpret_cast<float4*>(blk + (size_t)(dvb * 4 + j) * 256) = make_float4(acc[4 * j], acc[4 * j + 1], acc[4 * j + 2], acc[4 * j + 3]);
+        }
+      }
+      if (wave == 0 && lane < 32) {
+        float* ml = (float*)p.workspace + part_blocks_total * (size_t)(HG * kPartFloats) + (part_block * (32 * HG) + h_local) * 2;
+        ml[0] = m_all;
+        ml[1] = l_all;
+      }
+      continue;
+    }
     // transpose through LDS: lane (head hd, gq2) holds channels 32dvb + 8j + 4gq2 + (0..3) in o[.][4j..4j+3]
 #pragma unroll
     for (int dvb = 0; dvb < 4; ++dvb) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x16& acc = o[4 * dvb + hg];
-        float4 v = make_float4(acc[4 * j], acc[4 * j + 1], acc[4 * j + 2], acc[4 * j + 3]);
-        if (direct) v = make_float4(v.x * out_scale, v.y * out_scale, v.z * out_scale, v.w * out_scale);   // (uniform)
+        const float4 v = make_float4(acc[4 * j] * out_scale, acc[4 * j + 1] * out_scale, acc[4 * j + 2] * out_scale,
+                                     acc[4 * j + 3] * out_scale);
         *reinterpret_cast<float4*>(xbuf + hd * kXPitch + 32 * dvb + 8 * j + 4 * gq2) = v;
       }
     }
@@ -653,33 +678,98 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       const int hl = 32 * hg + row;
       if (hl >= heads_here) continue;
       const float4 v = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + hd * 4);
-      const int ch = 128 * wave + hd * 4;
-      if (direct) {
-        const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + ch;
-        if (p.out_dtype == CPPMEGA_MI355_F32) {
-          *reinterpret_cast<float4*>((float*)p.out + off) = v;
-        } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
-          *reinterpret_cast<uint2*>((unsigned short*)p.out + off) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
-        } else {
-          unsigned short* dst = (unsigned short*)p.out + off;
-          dst[0] = f32_to_f16_bits(v.x); dst[1] = f32_to_f16_bits(v.y);
-          dst[2] = f32_to_f16_bits(v.z); dst[3] = f32_to_f16_bits(v.w);
-        }
+      const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + 128 * wave + hd * 4;
+      if (p.out_dtype == CPPMEGA_MI355_F32) {
+        *reinterpret_cast<float4*>((float*)p.out + off) = v;
+      } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
+        *reinterpret_cast<uint2*>((unsigned short*)p.out + off) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
       } else {
-        float* part = (float*)p.workspace + ((q_index * p.H + head0 + hl) * (size_t)p.num_splits + split) * kLat + ch;
-        *reinterpret_cast<float4*>(part) = v;
+        unsigned short* dst = (unsigned short*)p.out + off;
+        dst[0] = f32_to_f16_bits(v.x); dst[1] = f32_to_f16_bits(v.y);
+        dst[2] = f32_to_f16_bits(v.z); dst[3] = f32_to_f16_bits(v.w);
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (wave == 0 && lane < 32 && h_local < heads_here) {
-      if (direct) {
-        if (p.lse) p.lse[q_index * p.H + head0 + h_local] = lse_val;
-      } else {
-        float* ml = (float*)p.workspace + (size_t)p.B * p.S * p.H * p.num_splits * kLat +
-                    ((q_index * p.H + head0 + h_local) * (size_t)p.num_splits + split) * 2;
-        ml[0] = m_all;
-        ml[1] = l_all;
-      }
+    if (wave == 0 && lane < 32 && h_local < heads_here && p.lse) p.lse[q_index * p.H + head0 + h_local] = lse_val;
+  }
+}
+
+// Merges the key splits written by sparse_mla_latent_kernel.  A partial block holds, per
+// (wavefront w = 128 value channels, head group hg), 16 rows of 64 lanes x float4 exactly as the
+// accumulator registers held them: row 4*dvb + j, lane (head hd = lane%32, half = lane/32), element e
+// is channel 128w + 32dvb + 8j + 4half + e of head 32hg + hd.  One workgroup per (query, KV group,
+// head chunk, w, hg): coalesced 1 KiB row reads, weights per head, transposition through LDS,
+// coalesced output rows.
+template <int HG>
+__global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const MlaParams p) {
+  __shared__ float x[32][kXPitch];
+  const int tid = (int)threadIdx.x, lane = tid & 63, r4 = tid >> 6;
+  const int chunks = (p.heads_per_group + 32 * HG - 1) / (32 * HG);
+  const int w = (int)blockIdx.y / HG, hg = (int)blockIdx.y % HG;
+  const size_t unit = blockIdx.x;                              // (b*S + s, g, chunk)
+  const int chunk = (int)(unit % chunks);
+  const size_t qg = unit / chunks;
+  const int g = (int)(qg % p.G);
+  const size_t bs = qg / p.G;
+  const int head0 = g * p.heads_per_group + chunk * 32 * HG;
+  const int heads_here = min(32 * HG, p.heads_per_group - chunk * 32 * HG);
+  const int hd = lane & 31, half = lane >> 5;
+  const int h_local = 32 * hg + hd;
+  const size_t blocks_total = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
+  const float* ml = (const float*)p.workspace + blocks_total * (size_t)(HG * kPartFloats);
+  const size_t block0 = unit * p.num_splits;
+  float m_all = -INFINITY;
+  for (int s = 0; s < p.num_splits; ++s) m_all = fmaxf(m_all, ml[((block0 + s) * (32 * HG) + h_local) * 2]);
+  float m_fin = m_all, l_fin = 0.0f;
+  if (p.sinks && h_local < heads_here) {
+    const float sk = p.sinks[head0 + h_local] * kLog2e;
+    m_fin = fmaxf(m_all, sk);
+    l_fin = exp2f(sk - m_fin);
+  }
+  float4 acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s = 0; s < p.num_splits; ++s) {
+    const float ms = ml[((block0 + s) * (32 * HG) + h_local) * 2];
+    if (ms == -INFINITY) continue;
+    const float f = exp2f(ms - m_fin);
+    l_fin += ml[((block0 + s) * (32 * HG) + h_local) * 2 + 1] * f;
+    const float* src = (const float*)p.workspace + (block0 + s) * (size_t)(HG * kPartFloats) +
+                       ((size_t)((w * HG + hg) * 16 + 4 * r4) * 64 + lane) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float4 v = *reinterpret_cast<const float4*>(src + (size_t)i * 256);
+      acc[i].x += v.x * f; acc[i].y += v.y * f; acc[i].z += v.z * f; acc[i].w += v.w * f;
+    }
+  }
+  const float inv = l_fin > 0.0f ? 1.0f / l_fin : 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {                                // row 4*r4 + i = (dvb = r4, j = i)
+    *reinterpret_cast<float4*>(&x[hd][32 * r4 + 8 * i + 4 * half]) =
+        make_float4(acc[i].x * inv, acc[i].y * inv, acc[i].z * inv, acc[i].w * inv);
+  }
+  if (p.lse && w == 0 && r4 == 0 && half == 0 && h_local < heads_here)
+    p.lse[bs * p.H + head0 + h_local] = l_fin > 0.0f ? (m_fin + log2f(l_fin)) * kLn2 : 0.0f;
+  __syncthreads();
+  // thread -> head tid/8, 16 channels (tid%8)*16
+  const int row = tid >> 3, c0 = (tid & 7) * 16;
+  if (32 * hg + row < heads_here) {
+    const size_t off = (bs * p.H + head0 + 32 * hg + row) * (size_t)kLat + 128 * w + c0;
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float4 t = *reinterpret_cast<const float4*>(&x[row][c0 + 4 * i]);
+      v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+    }
+    if (p.out_dtype == CPPMEGA_MI355_BF16) {
+      uint4 a, b;
+      a = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+      b = make_uint4(pack_bf16(v[8], v[9]), pack_bf16(v[10], v[11]), pack_bf16(v[12], v[13]), pack_bf16(v[14], v[15]));
+      *reinterpret_cast<uint4*>((unsigned short*)p.out + off) = a;
+      *reinterpret_cast<uint4*>((unsigned short*)p.out + off + 8) = b;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) store_as(p.out, off + i, p.out_dtype, v[i]);
     }
   }
 }
@@ -752,7 +842,21 @@ int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream) {
   }
 #undef CM_LAUNCH_LATENT
   CM_HIP_CHECK(hipGetLastError());
+  if (p.num_splits > 1) {
+    const dim3 cgrid((unsigned)((size_t)p.B * p.S * p.G * chunks), (unsigned)(4 * hg));
+    if (hg == 4) hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
+  }
+  CM_HIP_CHECK(hipGetLastError());
   return 0;
+}
+
+size_t sparse_mla_latent_workspace_bytes(const MlaParams& p) {
+  if (p.num_splits <= 1) return 0;
+  const int hg = p.heads_per_wg / 32;
+  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const size_t blocks = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
+  return blocks * ((size_t)hg * kPartFloats + 32 * hg * 2) * sizeof(float);
 }
 
 }  // namespace cm

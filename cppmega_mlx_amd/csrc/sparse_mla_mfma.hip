@@ -589,21 +589,13 @@ void sparse_mla_mfma_plan(MlaParams& p) {
 }
 
 size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p) {
+  if (p.heads_per_wg != 0) return sparse_mla_latent_workspace_bytes(p);
   if (p.num_splits <= 1) return 0;
   return (size_t)p.B * p.S * p.H * p.num_splits * (kLat + 2) * sizeof(float);
 }
 
 int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
-  if (p.heads_per_wg != 0) {
-    const int rc = sparse_mla_latent_launch(p, stream);
-    if (rc != 0) return rc;
-    if (p.num_splits > 1) {
-      const size_t qh = (size_t)p.B * p.S * p.H;
-      hipLaunchKernelGGL(sparse_mla_combine_kernel, dim3((unsigned)((qh + 3) / 4)), dim3(256), 0, stream, p);
-      CM_HIP_CHECK(hipGetLastError());
-    }
-    return 0;
-  }
+  if (p.heads_per_wg != 0) return sparse_mla_latent_launch(p, stream);
   const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
   const dim3 grid((unsigned)((size_t)p.B * p.S * p.G * groups_per_kv), (unsigned)p.num_splits), block(kWaves * 64);
   if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
