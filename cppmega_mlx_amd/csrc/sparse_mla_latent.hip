@@ -38,8 +38,8 @@
 //   pipeline     iteration t: barrier; issue tile t+3; QK + softmax of tile t+1;
 //                PV of tile t.
 //
-// Key splits write their fp32 accumulators to the workspace exactly as the lanes hold them
-// (1 KiB per store), plus (max, sum) per head; sparse_mla_latent_combine_kernel merges the
+// Key splits write their accumulators (rounded to bf16) to the workspace exactly as the lanes
+// hold them (512 B per store), plus (max, sum) per head; sparse_mla_latent_combine_kernel merges the
 // splits and does the transposition to [head][channel] that the single-split path does in LDS.
 
 #include <cstdlib>
@@ -63,7 +63,7 @@ constexpr int kRingBytes = kRing * kSlotBytes;  // 83968
 constexpr int kMaxKeys = 2048;                  // keys of one split (their rows are staged in LDS)
 constexpr int kKeyInts = kMaxKeys + 4 * kTK;    // + the tiles the pipeline prefetches past the end
 constexpr int kXPitch = 132;                    // floats per head row of the output transpose (128 + 4)
-constexpr int kPartFloats = 4 * 16 * 64 * 4;         // partial floats of one 32-head group: [4 wavefronts][16 rows][64 lanes][4]
+constexpr int kPartFloats = 4 * 16 * 64 * 4;         // partial values (bf16) of one 32-head group: [4 wavefronts][16 rows][64 lanes][4]
 constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
 
 template <int HG>
@@ -642,18 +642,21 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
     if (!direct) {
       // key split: the unnormalised accumulators leave exactly as the lanes hold them (1 KiB per
       // store instruction); the combine kernel knows the layout and does the transposition
-      float* blk = (float*)p.workspace + part_block * (size_t)(HG * kPartFloats) +
-                   ((size_t)((wave * HG + hg) * 16) * 64 + lane) * 4;
+      // (bf16: the values are relative to the split's own maximum, so their range is that of
+      // the output times the split's probability mass; the rounding is 2^-9 relative)
+      unsigned short* blk = (unsigned short*)p.workspace + part_block * (size_t)(HG * kPartFloats) +
+                            ((size_t)((wave * HG + hg) * 16) * 64 + lane) * 4;
 #pragma unroll
       for (int dvb = 0; dvb < 4; ++dvb) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const f32x16& acc = o[4 * dvb + hg];
-          *reinterpret_cast<float4*>(blk + (size_t)(dvb * 4 + j) * 256) = make_float4(acc[4 * j], acc[4 * j + 1], acc[4 * j + 2], acc[4 * j + 3]);
+          *reinterpret_cast<uint2*>(blk + (size_t)(dvb * 4 + j) * 256) =
+              make_uint2(pack_bf16(acc[4 * j], acc[4 * j + 1]), pack_bf16(acc[4 * j + 2], acc[4 * j + 3]));
         }
       }
       if (wave == 0 && lane < 32) {
-        float* ml = (float*)p.workspace + part_blocks_total * (size_t)(HG * kPartFloats) + (part_block * (32 * HG) + h_local) * 2;
+        float* ml = (float*)((unsigned short*)p.workspace + part_blocks_total * (size_t)(HG * kPartFloats)) + (part_block * (32 * HG) + h_local) * 2;
         ml[0] = m_all;
         ml[1] = l_all;
       }
@@ -716,10 +719,23 @@ __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const Ml
   const int hd = lane & 31, half = lane >> 5;
   const int h_local = 32 * hg + hd;
   const size_t blocks_total = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
-  const float* ml = (const float*)p.workspace + blocks_total * (size_t)(HG * kPartFloats);
+  const float* ml = (const float*)((const unsigned short*)p.workspace + blocks_total * (size_t)(HG * kPartFloats));
   const size_t block0 = unit * p.num_splits;
+  // all (max, sum) pairs first, then the partial rows four splits at a time, so that the loads
+  // of a group are in flight together (the split count is at most 16)
+  float ms[16], ls[16];
   float m_all = -INFINITY;
-  for (int s = 0; s < p.num_splits; ++s) m_all = fmaxf(m_all, ml[((block0 + s) * (32 * HG) + h_local) * 2]);
+#pragma unroll
+  for (int s = 0; s < 16; ++s) {
+    ms[s] = -INFINITY;
+    ls[s] = 0.0f;
+    if (s < p.num_splits) {
+      const float2 t = *reinterpret_cast<const float2*>(ml + ((block0 + s) * (32 * HG) + h_local) * 2);
+      ms[s] = t.x;
+      ls[s] = t.y;
+    }
+    m_all = fmaxf(m_all, ms[s]);
+  }
   float m_fin = m_all, l_fin = 0.0f;
   if (p.sinks && h_local < heads_here) {
     const float sk = p.sinks[head0 + h_local] * kLog2e;
@@ -729,17 +745,34 @@ __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const Ml
   float4 acc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int s = 0; s < p.num_splits; ++s) {
-    const float ms = ml[((block0 + s) * (32 * HG) + h_local) * 2];
-    if (ms == -INFINITY) continue;
-    const float f = exp2f(ms - m_fin);
-    l_fin += ml[((block0 + s) * (32 * HG) + h_local) * 2 + 1] * f;
-    const float* src = (const float*)p.workspace + (block0 + s) * (size_t)(HG * kPartFloats) +
-                       ((size_t)((w * HG + hg) * 16 + 4 * r4) * 64 + lane) * 4;
+  const unsigned short* src0 = (const unsigned short*)p.workspace + block0 * (size_t)(HG * kPartFloats) +
+                               ((size_t)((w * HG + hg) * 16 + 4 * r4) * 64 + lane) * 4;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float4 v = *reinterpret_cast<const float4*>(src + (size_t)i * 256);
-      acc[i].x += v.x * f; acc[i].y += v.y * f; acc[i].z += v.z * f; acc[i].w += v.w * f;
+  for (int s0 = 0; s0 < 16; s0 += 4) {
+    if (s0 >= p.num_splits) break;                            // (uniform)
+    uint2 raw[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int s = min(s0 + u, p.num_splits - 1);             // a repeated last split gets weight 0
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        raw[u][i] = *reinterpret_cast<const uint2*>(src0 + (size_t)s * (HG * kPartFloats) + (size_t)i * 256);
+    }
+    float4 v[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        v[u][i] = make_float4(__uint_as_float(raw[u][i].x << 16), __uint_as_float(raw[u][i].x & 0xffff0000u),
+                              __uint_as_float(raw[u][i].y << 16), __uint_as_float(raw[u][i].y & 0xffff0000u));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float f = (s0 + u < p.num_splits && ms[s0 + u] != -INFINITY) ? exp2f(ms[s0 + u] - m_fin) : 0.0f;
+      l_fin += ls[s0 + u] * f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[i].x += v[u][i].x * f; acc[i].y += v[u][i].y * f; acc[i].z += v[u][i].z * f; acc[i].w += v[u][i].w * f;
+      }
     }
   }
   const float inv = l_fin > 0.0f ? 1.0f / l_fin : 0.0f;
@@ -795,23 +828,34 @@ bool sparse_mla_latent_supported(const MlaParams& p) {
 }
 
 // heads per workgroup (in units of 32) and the key-split factor
+static int latent_splits(const MlaParams& p, int hg, long long* wgs) {
+  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const long long base = (long long)p.B * p.S * p.G * chunks;
+  int splits = 1;
+  while (base * splits < 256 && p.topk / (splits * 2) >= 4 * kTK && splits < 16) splits *= 2;
+  while ((p.topk + splits - 1) / splits > kMaxKeys) splits *= 2;
+  *wgs = base * splits;
+  return splits;
+}
+
 void sparse_mla_latent_plan(MlaParams& p) {
+  // 128 heads per workgroup reuse every gathered row the most; 64 only when that is what it takes
+  // to cover the device (few queries, short key lists)
   int hg = p.heads_per_group > 64 ? 4 : 2;
-  const long long queries = (long long)p.B * p.S * p.G;
-  // few queries: smaller head chunks need fewer key splits to fill the device, and each
-  // split writes (and the combine step re-reads) an fp32 partial per head
-  if (hg == 4 && queries * ((p.heads_per_group + 127) / 128) < 128) hg = 2;
+  long long wgs4 = 0, wgs2 = 0;
+  if (hg == 4) {
+    latent_splits(p, 4, &wgs4);
+    latent_splits(p, 2, &wgs2);
+    if (wgs4 < 256 && wgs2 > wgs4) hg = 2;
+  }
   if (const char* env = getenv("CPPMEGA_MI355_MLA_HEADS_PER_WG")) {
     const int v = atoi(env);
     if (v == 64) hg = 2;
     if (v == 128) hg = 4;
   }
   p.heads_per_wg = 32 * hg;
-  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
-  const long long base = queries * chunks;
-  int splits = 1;
-  while (base * splits < 256 && p.topk / (splits * 2) >= 4 * kTK && splits < 16) splits *= 2;
-  while ((p.topk + splits - 1) / splits > kMaxKeys) splits *= 2;
+  long long wgs = 0;
+  const int splits = latent_splits(p, hg, &wgs);
   const int tiles = (p.topk + kTK - 1) / kTK;
   const int tiles_per_split = (tiles + splits - 1) / splits;
   p.num_splits = splits;
@@ -856,7 +900,7 @@ size_t sparse_mla_latent_workspace_bytes(const MlaParams& p) {
   const int hg = p.heads_per_wg / 32;
   const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
   const size_t blocks = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
-  return blocks * ((size_t)hg * kPartFloats + 32 * hg * 2) * sizeof(float);
+  return blocks * ((size_t)hg * kPartFloats * sizeof(unsigned short) + 32 * hg * 2 * sizeof(float));
 }
 
 }  // namespace cm
