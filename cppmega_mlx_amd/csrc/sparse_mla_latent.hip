@@ -117,28 +117,31 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   const int tid = (int)threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  // ---- which (query, KV group, head chunk, split): workgroups that gather the same rows
-  //      (the head chunks of one query and split) get ids that are equal modulo 8, i.e.
-  //      the same XCD and L2 ----
+  // ---- which (query, KV group, head chunk, split).  Workgroup ids that are equal modulo 8 run on
+  //      the same XCD and share its L2: every workgroup of one (query, KV group) gets such ids, so
+  //      its query rows are fetched from HBM once (all key splits read them) and the head chunks
+  //      of a split find the gathered key rows of their sibling in cache ----
   const int chunks = (p.heads_per_group + 32 * HG - 1) / (32 * HG);
-  const long long units = (long long)p.B * p.S * p.G * p.num_splits;
-  const long long units8 = units & ~7ll;
-  long long unit;
-  int chunk;
+  const long long per_q = (long long)p.num_splits * chunks;    // workgroups of one (query, KV group)
+  const long long nq = (long long)p.B * p.S * p.G;
+  const long long nq8 = nq & ~7ll;
+  long long qg;
+  int chunk, split;
   {
     const long long id = blockIdx.x;
-    if (id < units8 * chunks) {
+    long long r;
+    if (id < nq8 * per_q) {
       const long long slot = id >> 3;
-      unit = (slot / chunks) * 8 + (id & 7);
-      chunk = (int)(slot % chunks);
+      qg = (slot / per_q) * 8 + (id & 7);
+      r = slot % per_q;
     } else {
-      const long long r = id - units8 * chunks;
-      unit = units8 + r / chunks;
-      chunk = (int)(r % chunks);
+      const long long rest = id - nq8 * per_q;
+      qg = nq8 + rest / per_q;
+      r = rest % per_q;
     }
+    split = (int)(r / chunks);
+    chunk = (int)(r % chunks);
   }
-  const int split = (int)(unit % p.num_splits);
-  const long long qg = unit / p.num_splits;
   const int g = (int)(qg % p.G);
   const size_t bs = (size_t)(qg / p.G);           // b*S + s
   const int b = (int)(bs / p.S);
@@ -163,6 +166,23 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   int* flagbuf = reinterpret_cast<int*>(smem + G_::kFlagOff);
   float* stats = reinterpret_cast<float*>(smem + G_::kStatOff);
 
+  // The first index entries are requested before the (much larger) query fragments: loads return
+  // in order, and the key rows can only be fetched once the indices are known.  Every load of
+  // this prologue is unconditional (positions and heads are clamped instead): only then can
+  // the compiler wait for the index words by count and leave the query loads in flight.
+  int early_lo[2], early_hi[2];
+  {
+    const bool wide = p.index_dtype == CPPMEGA_MI355_I64;
+    const int* words = (const int*)p.indices;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const size_t at = idx_base + (size_t)min(key_begin + tid + 256 * e, p.topk - 1);
+      const size_t w0 = wide ? 2 * at : at;
+      early_lo[e] = words[w0];
+      early_hi[e] = words[w0 + (wide ? 1 : 0)];
+    }
+  }
+
   // ---- Q^T fragments: lane (head n = lane%16, kq = lane/16), heads n and 16+n of group hgq.
   //      latent step ks (64 channels): fragments 2ks, 2ks+1 hold channels 64ks + 16kq + {0..7}, {8..15};
   //      rope step r: fragment 16+r holds channels 512 + 32r + 8kq + {0..7} ----
@@ -172,22 +192,18 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
       const int h = 32 * hgq + hh * 16 + n;
-      const bool live = h < heads_here;
-      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (live ? h : 0)) * (size_t)kDqk;
+      // heads past the end of the group repeat head 0: their columns stay finite and are never stored
+      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (h < heads_here ? h : 0)) * (size_t)kDqk;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        uint4 t0 = make_uint4(0, 0, 0, 0), t1 = t0;
-        if (live) {
-          t0 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq);
-          t1 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq + 8);
-        }
+        const uint4 t0 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq);
+        const uint4 t1 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq + 8);
         qf[hh][2 * ks] = __builtin_bit_cast(bf16x8, t0);
         qf[hh][2 * ks + 1] = __builtin_bit_cast(bf16x8, t1);
       }
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
-        uint4 t = make_uint4(0, 0, 0, 0);
-        if (live) t = *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kq);
+        const uint4 t = *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kq);
         qf[hh][16 + r] = __builtin_bit_cast(bf16x8, t);
       }
     }
@@ -198,7 +214,19 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   __syncthreads();
   {
     int mine = -1;
-    for (int i = tid; i < list_tiles * kTK + 4 * kTK; i += 256) {
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int i = tid + 256 * e;
+      if (i < list_tiles * kTK + 4 * kTK) {
+        const long long k = p.index_dtype == CPPMEGA_MI355_I64
+                                ? (long long)(((unsigned long long)(unsigned)early_hi[e] << 32) | (unsigned)early_lo[e])
+                                : (long long)early_lo[e];
+        const bool ok = i < n_keys && k >= 0 && k < p.Skv;
+        keys[i] = ok ? (int)k : -1;
+        if (ok) mine = i;
+      }
+    }
+    for (int i = tid + 512; i < list_tiles * kTK + 4 * kTK; i += 256) {
       int row = -1;
       if (i < n_keys) {
         const long long k = load_index(p, idx_base + key_begin + i);
