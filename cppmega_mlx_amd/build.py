@@ -34,6 +34,14 @@ HIPCC_FLAGS = [
     "-Wno-unused-result",
 ]
 
+# Per-file additions (none at present).
+FILE_FLAGS: dict[str, list[str]] = {}
+# Kernels (mangled-name fragments) that must not use scratch memory: they wait for their
+# asynchronous loads by count, and spill traffic would be counted with them.
+NO_SCRATCH = {
+    "sparse_mla_latent.hip": ("sparse_mla_latent_kernel",),
+}
+
 
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", shutil.which("hipcc")):
@@ -48,16 +56,34 @@ def sources() -> list[Path]:
 
 def _compile_one(hipcc: str, src: Path, verbose: bool) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
-    cmd = [hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc, *HIPCC_FLAGS, *FILE_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
+    if src.name in NO_SCRATCH:
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{proc.stdout}\n{proc.stderr}")
-    errs = [ln for ln in proc.stderr.splitlines() if "packed-fp32-ops" not in ln and ln.strip()]
+    if src.name in NO_SCRATCH:
+        _check_no_scratch(src.name, proc.stderr)
+    errs = [ln for ln in proc.stderr.splitlines()
+            if "packed-fp32-ops" not in ln and "kernel-resource-usage" not in ln and ln.strip()]
     if verbose and errs:
         print("\n".join(errs), flush=True)
     return obj
+
+
+def _check_no_scratch(name: str, remarks: str) -> None:
+    """Parse the compiler's resource remarks: fail the build if a listed kernel spills."""
+    current = None
+    for ln in remarks.splitlines():
+        if "Function Name:" in ln:
+            current = ln.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in ln and current:
+            size = int(ln.split("ScratchSize [bytes/lane]:")[1].split("[")[0].strip())
+            if size and any(frag in current for frag in NO_SCRATCH[name]):
+                raise RuntimeError(f"{name}: kernel {current} uses {size} bytes/lane of scratch memory; "
+                                   "it must fit its registers (see NO_SCRATCH in build.py)")
 
 
 def build(verbose: bool = True, jobs: int | None = None) -> Path:
