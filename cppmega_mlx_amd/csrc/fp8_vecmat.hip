@@ -86,6 +86,14 @@ __device__ __forceinline__ void load_x16(const VecmatParams& p, size_t off, floa
   }
 }
 
+// 16 weight bytes that are read exactly once: loaded with the non-temporal hint, so they do not
+// displace the activations and scales (which every workgroup re-reads) from the caches
+__device__ __forceinline__ uint4 load_w16(const unsigned char* src) {
+  typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
+  return make_uint4(t[0], t[1], t[2], t[3]);
+}
+
 __device__ __forceinline__ float dot16(const uint4 wv, const float (&x)[16]) {
   const unsigned wds[4] = {wv.x, wv.y, wv.z, wv.w};
   float s = 0.0f;
@@ -146,7 +154,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const VecmatParam
 #pragma unroll
           for (int c = 0; c < CH; ++c) {
             if (koff[c] < K) {
-              wv[u][c] = *reinterpret_cast<const uint4*>(wrow + koff[c]);
+              wv[u][c] = load_w16(wrow + koff[c]);
               sc[u][c] = wscale(p, n, koff[c] >> 7);
             } else {
               wv[u][c] = make_uint4(0, 0, 0, 0);
@@ -184,7 +192,6 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const VecmatParam
 //   * rows are processed in groups of U with the loads of the next group issued
 //     before the arithmetic of the current one (two register buffers);
 //   * per row: DPP wavefront reduction, then a fixed-order 4-way LDS combine.
-constexpr int kStreamRows = 16;
 
 __device__ __forceinline__ float wave_total_dpp(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, false));
@@ -202,10 +209,12 @@ struct StreamBuf {
   float sc[U][CH];
 };
 
-template <int M, int CH, int U>
+// R rows per workgroup (a multiple of U): the host picks the R that spreads the rows most evenly
+// over the compute units
+template <int M, int CH, int U, int R>
 __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const VecmatParams p) {
-  constexpr int R = kStreamRows, G = R / U;
-  static_assert(G % 2 == 0, "row groups come in pairs");
+  constexpr int G = R / U;
+  static_assert(R % U == 0, "whole row groups");
   __shared__ float red[kGemvWaves][R][M];
   const int lane = lane_id();
   const int wave = (int)(threadIdx.x >> 6);
@@ -235,7 +244,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
       const unsigned char* wrow = p.w + (size_t)n * K;
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
-        buf.w[u][c] = *reinterpret_cast<const uint4*>(wrow + koff[c]);
+        buf.w[u][c] = load_w16(wrow + koff[c]);
         buf.sc[u][c] = wscale(p, n, koff[c] >> 7);
       }
     }
@@ -274,12 +283,13 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
   StreamBuf<M, CH, U> a, b;
   load(a, 0);
 #pragma unroll
-  for (int g = 0; g < G; g += 2) {
+  for (int g = 0; g + 1 < G; g += 2) {
     load(b, g + 1);
     compute(a, g);
     if (g + 2 < G) load(a, g + 2);
     compute(b, g + 1);
   }
+  if (G % 2) compute(a, G - 1);
   __syncthreads();
   const int t = (int)threadIdx.x;
   if (t < R * M) {
@@ -335,7 +345,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
     pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
   };
   auto pf_next = [&](uint4& wdst, float& sdst, bool with_scale) {
-    wdst = *reinterpret_cast<const uint4*>(pf_w + 64 * pf_st);
+    wdst = *reinterpret_cast<const uint4*>(pf_w + 64 * pf_st);   // (plain load: the other half of the cache line follows next step)
     if (with_scale) sdst = pf_s[(size_t)(pf_st >> 1) * p.scol_stride];
     if (++pf_st == steps) {                              // (uniform)
       pf_st = 0;
@@ -501,6 +511,33 @@ int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* byt
   return 0;
 }
 
+// Rows per workgroup of the streaming kernel: the candidate whose grid leaves the smallest idle
+// share in its last round over the device's compute units (ties: more workgroups).
+static int stream_rows(int n, int m) {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+    else cus = 256;
+  }
+  if (const char* e = getenv("CPPMEGA_MI355_VECMAT_ROWS")) {
+    const int v = atoi(e);
+    if (m > 1 && (v == 16 || v == 28 || v == 14)) return v;
+  }
+  if (m == 1) return 16;
+  const int cand[3] = {16, 28, 14};
+  int best = 16;
+  double best_eff = -1.0;
+  for (int r : cand) {
+    const long long wgs = (n + r - 1) / r;
+    const long long rounds = (wgs + cus - 1) / cus;
+    const double eff = (double)wgs / (double)(rounds * cus);
+    if (eff > best_eff + 1e-9) { best_eff = eff; best = r; }
+  }
+  return best;
+}
+
 int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) {
   int rc = validate(a);
   if (rc) return rc;
@@ -515,19 +552,29 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   const bool aligned = vecmat_aligned(a);
   const bool stream_ok = aligned && stream_shape(a);
   if (stream_ok) {
-    const dim3 grid((unsigned)((a.n + kStreamRows - 1) / kStreamRows)), block(kGemvWaves * 64);
+    // rows per workgroup: 16, or 28 / 14 when that fills the last round of workgroups better
+    // (7168 rows are 448 x 16 = 1.75 rounds on 256 compute units, but exactly 256 x 28)
+    const int rows = stream_rows(a.n, a.m);
+    const dim3 grid((unsigned)((a.n + rows - 1) / rows)), block(kGemvWaves * 64);
     const int ch = a.k / 4096;
-#define CM_STREAM(M, U)                                                                             \
-  do {                                                                                              \
-    if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, U>), grid, block, 0, stream, p);      \
-    else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, U>), grid, block, 0, stream, p); \
-    else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, U>), grid, block, 0, stream, p); \
-    else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, U>), grid, block, 0, stream, p);              \
+#define CM_STREAM_R(M, U, R)                                                                           \
+  do {                                                                                                 \
+    if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, U, R>), grid, block, 0, stream, p);      \
+    else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, U, R>), grid, block, 0, stream, p); \
+    else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, U, R>), grid, block, 0, stream, p); \
+    else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, U, R>), grid, block, 0, stream, p);              \
   } while (0)
-    if (a.m == 1) CM_STREAM(1, 4);
+#define CM_STREAM(M, U)                          \
+  do {                                           \
+    if (rows == 28) CM_STREAM_R(M, U, 28);       \
+    else if (rows == 14) CM_STREAM_R(M, U, 14);  \
+    else CM_STREAM_R(M, U, 16);                  \
+  } while (0)
+    if (a.m == 1) CM_STREAM_R(1, 4, 16);          // (measured: one activation row streams best in the smaller units)
     else if (a.m == 2) CM_STREAM(2, 2);
     else if (a.m == 3) CM_STREAM(3, 2);
     else CM_STREAM(4, 2);
+#undef CM_STREAM_R
 #undef CM_STREAM
   } else if (skinny_ok(a)) {
     const size_t need = (size_t)kSkinnySplits * a.m * a.n * sizeof(float);
