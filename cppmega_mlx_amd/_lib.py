@@ -44,6 +44,9 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_fp8_vecmat_workspace_bytes",
     "cppmega_mi355_fp8_vecmat",
     "cppmega_mi355_fp8_quantize",
+    "cppmega_mi355_kv_cache_append",
+    "cppmega_mi355_causal_sparse_indices",
+    "cppmega_mi355_mask_sparse_indices",
 )
 
 
@@ -163,6 +166,66 @@ class QuantizeArgs(C.Structure):
 
 QUANT_PER_TOKEN, QUANT_PER_TENSOR, QUANT_MXFP8, DEQUANT_PER_TOKEN, DEQUANT_MXFP8 = range(5)
 
+
+class CacheAppendArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("src_dtype", C.c_int32),
+        ("src", C.c_void_p),
+        ("src_scale", C.c_void_p),
+        ("rope", C.c_void_p),
+        ("rope_dtype", C.c_int32),
+        ("scale_block", C.c_int32),
+        ("kv_cache", C.c_void_p),
+        ("scale_cache", C.c_void_p),
+        ("rope_cache", C.c_void_p),
+        ("positions", C.c_void_p),
+        ("position", C.c_int32),
+        ("batch", C.c_int32),
+        ("new_tokens", C.c_int32),
+        ("groups", C.c_int32),
+        ("dim", C.c_int32),
+        ("rope_dim", C.c_int32),
+        ("capacity", C.c_int32),
+        ("pow2_scales", C.c_int32),
+        ("reserved", C.c_int32),
+    ]
+
+
+class CausalIndicesArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("index_dtype", C.c_int32),
+        ("indices", C.c_void_p),
+        ("batch", C.c_int32),
+        ("seq", C.c_int32),
+        ("groups", C.c_int32),
+        ("topk", C.c_int32),
+        ("query_offset", C.c_int64),
+        ("key_length", C.c_int64),
+    ]
+
+
+MASK_BOOL, MASK_F32, MASK_F16, MASK_BF16 = range(4)
+
+
+class MaskIndicesArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("mask_dtype", C.c_int32),
+        ("mask", C.c_void_p),
+        ("stride_b", C.c_int64),
+        ("stride_g", C.c_int64),
+        ("stride_s", C.c_int64),
+        ("batch", C.c_int32),
+        ("seq", C.c_int32),
+        ("groups", C.c_int32),
+        ("topk", C.c_int32),
+        ("key_length", C.c_int32),
+        ("reserved", C.c_int32),
+        ("indices", C.c_void_p),
+    ]
+
 _lock = threading.RLock()
 _lib: C.CDLL | None = None
 
@@ -211,6 +274,11 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_fp8_vecmat.restype = C.c_int
         lib.cppmega_mi355_fp8_quantize.argtypes = [C.POINTER(QuantizeArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_fp8_quantize.restype = C.c_int
+        for fn, struct in ((lib.cppmega_mi355_kv_cache_append, CacheAppendArgs),
+                           (lib.cppmega_mi355_causal_sparse_indices, CausalIndicesArgs),
+                           (lib.cppmega_mi355_mask_sparse_indices, MaskIndicesArgs)):
+            fn.argtypes = [C.POINTER(struct), C.c_size_t, C.c_void_p]
+            fn.restype = C.c_int
         lib.cppmega_mi355_fp8_vecmat_workspace_bytes.argtypes = [
             C.POINTER(VecmatArgs), C.c_size_t, C.POINTER(C.c_size_t)]
         lib.cppmega_mi355_fp8_vecmat_workspace_bytes.restype = C.c_int

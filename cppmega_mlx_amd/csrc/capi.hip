@@ -30,6 +30,9 @@ int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream);
 int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream);
 int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes);
 int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stream);
+int kv_cache_append_launch(const cppmega_mi355_cache_append_args_t& a, hipStream_t stream);
+int causal_indices_launch(const cppmega_mi355_causal_indices_args_t& a, hipStream_t stream);
+int mask_indices_launch(const cppmega_mi355_mask_indices_args_t& a, hipStream_t stream);
 
 static bool is_float_carrier(int dt) {
   return dt == CPPMEGA_MI355_F32 || dt == CPPMEGA_MI355_F16 || dt == CPPMEGA_MI355_BF16;
@@ -212,6 +215,21 @@ int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args,
 int cppmega_mi355_fp8_quantize(const cppmega_mi355_quantize_args_t* args, size_t args_size, void* stream) {
   CM_CHECK_ARGS(args, args_size, cppmega_mi355_quantize_args_t);
   return fp8_quantize_launch(*args, (hipStream_t)stream);
+}
+
+int cppmega_mi355_kv_cache_append(const cppmega_mi355_cache_append_args_t* args, size_t args_size, void* stream) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_cache_append_args_t);
+  return kv_cache_append_launch(*args, (hipStream_t)stream);
+}
+
+int cppmega_mi355_causal_sparse_indices(const cppmega_mi355_causal_indices_args_t* args, size_t args_size, void* stream) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_causal_indices_args_t);
+  return causal_indices_launch(*args, (hipStream_t)stream);
+}
+
+int cppmega_mi355_mask_sparse_indices(const cppmega_mi355_mask_indices_args_t* args, size_t args_size, void* stream) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_mask_indices_args_t);
+  return mask_indices_launch(*args, (hipStream_t)stream);
 }
 
 int cppmega_mi355_fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t* args, size_t args_size,

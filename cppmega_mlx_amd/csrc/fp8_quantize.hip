@@ -130,6 +130,103 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(const QuantParams 
   }
 }
 
+
+// ---- cache append -------------------------------------------------------------------------
+struct AppendParams {
+  const void* src;
+  const float* src_scale;
+  const void* rope;
+  unsigned char* kv_cache;
+  float* scale_cache;
+  unsigned short* rope_cache;
+  const int* positions;
+  int position;
+  int B, S, G, D, R, cap;
+  int src_dtype, rope_dtype, scale_block, pow2;
+};
+
+// One wavefront per new (batch, token, group) row.  A lane owns 8 consecutive channels of every
+// 512-channel piece, so a 128-channel block is 16 lanes and its amax four butterfly steps.
+template <bool PREPARED>
+__global__ __launch_bounds__(256) void cache_append_kernel(const AppendParams p) {
+  const int lane = lane_id();
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);       // (b * S + s) * G + g
+  const long long rows = (long long)p.B * p.S * p.G;
+  if (row >= rows) return;
+  const int g = (int)(row % p.G);
+  const long long bs = row / p.G;
+  const int s = (int)(bs % p.S), b = (int)(bs / p.S);
+  const int pos = (p.positions ? p.positions[b] : p.position) + s;
+  if (pos < 0 || pos >= p.cap) return;                                         // (checked on the host when positions is NULL)
+  const size_t crow = ((size_t)b * p.cap + pos) * p.G + g;                     // cache row
+  const int nsc = p.scale_block ? p.D / p.scale_block : 1;
+  const size_t sbase = (size_t)row * p.D;
+  if (PREPARED) {
+    for (int c = lane * 16; c < p.D; c += 64 * 16)
+      *reinterpret_cast<uint4*>(p.kv_cache + crow * p.D + c) = *reinterpret_cast<const uint4*>((const unsigned char*)p.src + sbase + c);
+    if (lane < nsc) p.scale_cache[crow * nsc + lane] = p.src_scale[(size_t)row * nsc + lane];
+  } else {
+    constexpr int kMaxPieces = 4;                                              // D <= 2048
+    float v[kMaxPieces][8];
+    float am[kMaxPieces];
+    const int pieces = (p.D + 511) / 512;
+#pragma unroll
+    for (int pc = 0; pc < kMaxPieces; ++pc) {
+      am[pc] = 0.0f;
+      const int c0 = pc * 512 + lane * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        v[pc][i] = (pc < pieces && c0 + i < p.D) ? load_as(p.src, sbase + c0 + i, p.src_dtype) : 0.0f;
+        am[pc] = fmaxf(am[pc], fabsf(v[pc][i]));
+      }
+#pragma unroll
+      for (int off = 1; off <= 8; off <<= 1) am[pc] = fmaxf(am[pc], __shfl_xor(am[pc], off, 64));   // the lane's 128-channel block
+    }
+    float row_am = 0.0f;
+    if (!p.scale_block) {
+#pragma unroll
+      for (int pc = 0; pc < kMaxPieces; ++pc) row_am = fmaxf(row_am, am[pc]);
+      row_am = wave_max_f(row_am);
+    }
+#pragma unroll
+    for (int pc = 0; pc < kMaxPieces; ++pc) {
+      if (pc >= pieces) break;
+      const int c0 = pc * 512 + lane * 8;
+      if (c0 >= p.D) continue;
+      const float a = p.scale_block ? am[pc] : row_am;
+      float sc;
+      if (p.pow2) {
+        // smallest power of two s with 448 * s >= amax:  amax = fr * 2^ex, fr in [0.5, 1)
+        sc = 1.0f;
+        if (a > 0.0f) {
+          int ex;
+          const float fr = frexpf(a, &ex);
+          sc = ldexpf(1.0f, (ex - 1) - 8 + (fr > 0.875f ? 1 : 0));
+        }
+      } else {
+        sc = fmaxf(a * (1.0f / 448.0f), 1.0e-12f);
+      }
+      unsigned w0 = 0, w1 = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float nv = fminf(fmaxf(__fdiv_rn(v[pc][i], sc), -448.0f), 448.0f);
+        const unsigned code = e4m3_encode(nv);
+        if (i < 4) w0 |= code << (8 * i); else w1 |= code << (8 * (i - 4));
+      }
+      *reinterpret_cast<uint2*>(p.kv_cache + crow * p.D + c0) = make_uint2(w0, w1);
+      if (p.scale_block) {
+        if ((lane & 15) == 0) p.scale_cache[crow * nsc + (c0 >> 7)] = sc;
+      } else if (lane == 0 && pc == 0) {
+        p.scale_cache[crow] = sc;
+      }
+    }
+  }
+  if (p.rope_cache) {
+    for (int c = lane; c < p.R; c += 64)
+      store_as(p.rope_cache, crow * p.R + c, CPPMEGA_MI355_BF16, load_as(p.rope, (size_t)row * p.R + c, p.rope_dtype));
+  }
+}
+
 }  // namespace
 
 int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stream) {
@@ -170,6 +267,43 @@ int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stre
     hipLaunchKernelGGL(tensor_amax_kernel, dim3(blocks), dim3(256), 0, stream, p, word);
     hipLaunchKernelGGL(quantize_rows_kernel<1>, grid, block, 0, stream, p, (const unsigned*)word);
   }
+  CM_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int kv_cache_append_launch(const cppmega_mi355_cache_append_args_t& a, hipStream_t stream) {
+  if (a.batch < 1 || a.new_tokens < 0 || a.groups < 1 || a.dim < 1 || a.capacity < 1 || a.rope_dim < 0)
+    return fail(CPPMEGA_MI355_ERR_SHAPE, "kv_cache_append: B=%d S_new=%d G=%d D=%d R=%d capacity=%d", a.batch, a.new_tokens, a.groups, a.dim, a.rope_dim, a.capacity);
+  if (a.dim % 128 != 0 || a.dim > 2048 || a.rope_dim > 256)
+    return fail(CPPMEGA_MI355_ERR_SHAPE, "kv_cache_append: D must be a multiple of 128 up to 2048 and R <= 256, got D=%d R=%d", a.dim, a.rope_dim);
+  if (a.scale_block != 0 && a.scale_block != 128)
+    return fail(CPPMEGA_MI355_ERR_SHAPE, "kv_cache_append: scale_block must be 0 (per row) or 128, got %d", a.scale_block);
+  const bool prepared = a.src_dtype == CPPMEGA_MI355_E4M3;
+  if (!prepared && a.src_dtype != CPPMEGA_MI355_F32 && a.src_dtype != CPPMEGA_MI355_F16 && a.src_dtype != CPPMEGA_MI355_BF16)
+    return fail(CPPMEGA_MI355_ERR_DTYPE, "kv_cache_append: source dtype %d", a.src_dtype);
+  if (a.new_tokens == 0) return 0;
+  if (!a.src || !a.kv_cache || !a.scale_cache || (prepared && !a.src_scale))
+    return fail(CPPMEGA_MI355_ERR_NULL, "kv_cache_append: src / src_scale / kv_cache / scale_cache is NULL");
+  const bool with_rope = a.rope_dim > 0 && a.rope_cache != nullptr;
+  if (with_rope) {
+    if (!a.rope) return fail(CPPMEGA_MI355_ERR_NULL, "kv_cache_append: rope cache given but no rope rows");
+    if (a.rope_dtype != CPPMEGA_MI355_F32 && a.rope_dtype != CPPMEGA_MI355_F16 && a.rope_dtype != CPPMEGA_MI355_BF16)
+      return fail(CPPMEGA_MI355_ERR_DTYPE, "kv_cache_append: rope dtype %d", a.rope_dtype);
+  }
+  if (!a.positions && (a.position < 0 || (long long)a.position + a.new_tokens > a.capacity))
+    return fail(CPPMEGA_MI355_ERR_SHAPE, "kv_cache_append: positions %d..%lld exceed the capacity %d", a.position, (long long)a.position + a.new_tokens, a.capacity);
+  if (((size_t)a.src | (size_t)a.kv_cache) & 15)
+    return fail(CPPMEGA_MI355_ERR_ALIGNMENT, "kv_cache_append: src and kv_cache must be 16-byte aligned");
+  AppendParams p;
+  p.src = a.src; p.src_scale = a.src_scale; p.rope = a.rope; p.kv_cache = a.kv_cache; p.scale_cache = a.scale_cache;
+  p.rope_cache = with_rope ? (unsigned short*)a.rope_cache : nullptr;
+  p.positions = a.positions; p.position = a.position;
+  p.B = a.batch; p.S = a.new_tokens; p.G = a.groups; p.D = a.dim; p.R = a.rope_dim; p.cap = a.capacity;
+  p.src_dtype = a.src_dtype; p.rope_dtype = a.rope_dtype; p.scale_block = a.scale_block; p.pow2 = a.pow2_scales;
+  const long long rows = (long long)a.batch * a.new_tokens * a.groups;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  if (prepared) hipLaunchKernelGGL(cache_append_kernel<true>, grid, block, 0, stream, p);
+  else hipLaunchKernelGGL(cache_append_kernel<false>, grid, block, 0, stream, p);
   CM_HIP_CHECK(hipGetLastError());
   return 0;
 }

@@ -373,3 +373,107 @@ def fp8_dequantize(codes: torch.Tensor, scale: torch.Tensor, *, out: torch.Tenso
         rc = _lib.load().cppmega_mi355_fp8_quantize(C.byref(a), C.sizeof(a), _lib.current_stream(codes.device))
     _lib.check(rc, "fp8_dequantize")
     return out
+
+
+def kv_cache_append(src: torch.Tensor, *, kv_cache: torch.Tensor, scale_cache: torch.Tensor, position,
+                    src_scale: torch.Tensor | None = None, rope: torch.Tensor | None = None,
+                    rope_cache: torch.Tensor | None = None, scale_block: int = 0, pow2_scales: bool = False) -> None:
+    """Write ``src[B, S_new, G, D]`` into the preallocated cache at ``position`` (an int, or an
+    int32 device tensor ``[B]``).  uint8 ``src`` + float32 ``src_scale`` are copied as prepared
+    bytes; a float ``src`` is quantised to e4m3 on the way (one scale per row, or per 128
+    channels with ``scale_block=128``).  ``rope[B, S_new, G, R]`` lands in ``rope_cache`` as bf16."""
+    _lib.require_device_tensor(src, "src", None)
+    for name, t in (("kv_cache", kv_cache), ("scale_cache", scale_cache), ("src_scale", src_scale), ("rope", rope), ("rope_cache", rope_cache)):
+        if t is not None:
+            _lib.require_device_tensor(t, name, src)
+            if not t.is_contiguous():
+                raise ValueError(f"{name} must be contiguous")
+    if src.ndim != 4 or not src.is_contiguous():
+        raise ValueError("src must be contiguous with shape (batch, sequence, kv_heads, head_dim)")
+    B, S, G, D = (int(d) for d in src.shape)
+    if kv_cache.dtype != torch.uint8 or kv_cache.ndim != 4 or kv_cache.shape[0] != B or kv_cache.shape[2] != G or kv_cache.shape[3] != D:
+        raise ValueError(f"kv_cache must be uint8 [B, capacity, G, D] matching src; got {kv_cache.dtype} {tuple(kv_cache.shape)}")
+    cap = int(kv_cache.shape[1])
+    nsc = D // scale_block if scale_block else 1
+    want_scale = (B, cap, G) if not scale_block else (B, cap, G, nsc)
+    if scale_cache.dtype != torch.float32 or tuple(scale_cache.shape) != want_scale:
+        raise ValueError(f"scale_cache must be float32 {want_scale}; got {scale_cache.dtype} {tuple(scale_cache.shape)}")
+    prepared = src.dtype == torch.uint8
+    if prepared:
+        want = (B, S, G) if not scale_block else (B, S, G, nsc)
+        if src_scale is None or src_scale.dtype != torch.float32 or tuple(src_scale.shape) != want:
+            raise ValueError(f"prepared bytes need float32 src_scale {want}")
+    a = _lib.CacheAppendArgs()
+    a.struct_size = C.sizeof(a)
+    a.src_dtype = _lib.E4M3 if prepared else _dtype_or_raise(src, "src", (_lib.F32, _lib.F16, _lib.BF16))
+    a.src, a.src_scale = src.data_ptr(), _lib.ptr(src_scale)
+    a.kv_cache, a.scale_cache = kv_cache.data_ptr(), scale_cache.data_ptr()
+    a.scale_block, a.pow2_scales = int(scale_block), int(bool(pow2_scales))
+    if rope is not None or rope_cache is not None:
+        if rope is None or rope_cache is None:
+            raise ValueError("rope and rope_cache go together")
+        R = int(rope.shape[-1])
+        if tuple(rope.shape) != (B, S, G, R) or rope_cache.dtype != torch.bfloat16 or tuple(rope_cache.shape) != (B, cap, G, R):
+            raise ValueError("rope must be [B, S_new, G, R] and rope_cache bfloat16 [B, capacity, G, R]")
+        a.rope, a.rope_cache, a.rope_dim = rope.data_ptr(), rope_cache.data_ptr(), R
+        a.rope_dtype = _dtype_or_raise(rope, "rope", (_lib.F32, _lib.F16, _lib.BF16))
+    if isinstance(position, torch.Tensor):
+        _lib.require_device_tensor(position, "position", src)
+        if position.dtype != torch.int32 or tuple(position.shape) != (B,) or not position.is_contiguous():
+            raise ValueError("position tensor must be contiguous int32 [B]")
+        a.positions = position.data_ptr()
+    else:
+        a.position = int(position)
+    a.batch, a.new_tokens, a.groups, a.dim, a.capacity = B, S, G, D, cap
+    with torch.cuda.device(src.device):
+        rc = _lib.load().cppmega_mi355_kv_cache_append(C.byref(a), C.sizeof(a), _lib.current_stream(src.device))
+    _lib.check(rc, "kv_cache_append")
+
+
+def causal_sparse_indices(out: torch.Tensor, *, query_offset: int = 0, key_length: int) -> torch.Tensor:
+    """Fill ``out[B, S, G, topk]`` (int32 / int64) with the causal window ``q_pos - j`` (or -1)."""
+    _lib.require_device_tensor(out, "indices", None)
+    if out.ndim != 4 or not out.is_contiguous() or out.dtype not in (torch.int32, torch.int64):
+        raise ValueError("indices must be a contiguous int32/int64 tensor [B, S, G, topk]")
+    a = _lib.CausalIndicesArgs()
+    a.struct_size = C.sizeof(a)
+    a.index_dtype = _lib.I32 if out.dtype == torch.int32 else _lib.I64
+    a.indices = out.data_ptr()
+    a.batch, a.seq, a.groups, a.topk = (int(d) for d in out.shape)
+    a.query_offset, a.key_length = int(query_offset), int(key_length)
+    with torch.cuda.device(out.device):
+        rc = _lib.load().cppmega_mi355_causal_sparse_indices(C.byref(a), C.sizeof(a), _lib.current_stream(out.device))
+    _lib.check(rc, "causal_sparse_indices")
+    return out
+
+
+_MASK_DTYPES = {torch.bool: _lib.MASK_BOOL, torch.uint8: _lib.MASK_BOOL, torch.float32: _lib.MASK_F32,
+                torch.float16: _lib.MASK_F16, torch.bfloat16: _lib.MASK_BF16}
+
+
+def mask_sparse_indices(mask: torch.Tensor, out: torch.Tensor, *, topk: int) -> torch.Tensor:
+    """``mask`` is a 4-D view ``[B or 1, G or 1, S, K]`` with a unit stride along K (broadcast
+    dimensions may have stride 0); ``out`` int32 ``[B, S, G, min(topk, K)]``."""
+    _lib.require_device_tensor(mask, "mask", None)
+    _lib.require_device_tensor(out, "indices", mask)
+    if mask.dtype not in _MASK_DTYPES:
+        raise TypeError(f"mask dtype {mask.dtype} is not bool/uint8/float32/float16/bfloat16")
+    if mask.ndim != 4 or (mask.shape[-1] > 1 and mask.stride(-1) != 1):
+        raise ValueError("mask must be 4-D with a unit stride along the key axis")
+    B, S, G, n = (int(d) for d in out.shape)
+    K = int(mask.shape[-1])
+    if out.dtype != torch.int32 or not out.is_contiguous() or n != min(int(topk), K):
+        raise ValueError("indices must be contiguous int32 [B, S, G, min(topk, key_length)]")
+    a = _lib.MaskIndicesArgs()
+    a.struct_size = C.sizeof(a)
+    a.mask_dtype = _MASK_DTYPES[mask.dtype]
+    a.mask = mask.data_ptr()
+    a.stride_b = int(mask.stride(0)) if mask.shape[0] > 1 else 0
+    a.stride_g = int(mask.stride(1)) if mask.shape[1] > 1 else 0
+    a.stride_s = int(mask.stride(2))
+    a.batch, a.seq, a.groups, a.topk, a.key_length = B, S, G, int(topk), K
+    a.indices = out.data_ptr()
+    with torch.cuda.device(out.device):
+        rc = _lib.load().cppmega_mi355_mask_sparse_indices(C.byref(a), C.sizeof(a), _lib.current_stream(out.device))
+    _lib.check(rc, "mask_sparse_indices")
+    return out

@@ -283,6 +283,78 @@ typedef struct cppmega_mi355_quantize_args {
 
 int cppmega_mi355_fp8_quantize(const cppmega_mi355_quantize_args_t* args, size_t args_size, void* stream);
 
+/* ---- KV-cache append: FP8 producer fused with the write into the cache ------------------
+ * Replaces the append path in front of the sparse-attention kernels:
+ *   ContiguousKVCache.update_and_fetch_sparse_fp8 (cppmega_mlx/inference/engine.py:76-98,
+ *   validation :436-466) -- prepared e4m3 bytes + one float32 scale per row are appended
+ *   along the sequence axis -- and, in front of it, the producer fp8_per_token_quant
+ *   (cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:2667-2753).
+ * The cache is preallocated, [B, capacity, G, ...]; `new_tokens` rows per (batch, group) are
+ * written at positions `position` .. (or positions[b] ..).  Two source forms:
+ *   src_dtype E4M3      src is e4m3 bytes [B, S_new, G, D], src_scale their float32 scales
+ *                       [B, S_new, G, D/scale_block or 1]: bytes and scales are copied
+ *                       (the reference's semantics);
+ *   src_dtype F32/F16/BF16   src is quantised on the way: scale_block 0 = one scale per
+ *                       row, max(amax * (1/448), 1e-12) (the reference's producer);
+ *                       scale_block 128 = one float32 scale per 128 channels by the same
+ *                       formula, or with pow2_scales != 0 the smallest power of two s with
+ *                       448 * s >= amax (1.0 for an all-zero block): the latent cache format
+ *                       the decode kernel gathers.
+ * rope (optional, [B, S_new, G, R] float32/float16/bfloat16) is stored as bfloat16.
+ * D % 128 == 0, D <= 2048, R <= 256. */
+typedef struct cppmega_mi355_cache_append_args {
+  uint32_t struct_size;
+  int32_t src_dtype;          /* E4M3 (prepared) or F32/F16/BF16 (quantise)          */
+  const void* src;            /* [B, S_new, G, D]                                    */
+  const float* src_scale;     /* prepared form only                                  */
+  const void* rope;           /* [B, S_new, G, R] or NULL                            */
+  int32_t rope_dtype;
+  int32_t scale_block;        /* 0: one scale per row; 128: one per 128 channels     */
+  uint8_t* kv_cache;          /* [B, capacity, G, D] e4m3 bytes                      */
+  float* scale_cache;         /* [B, capacity, G, 1 or D/128]                        */
+  void* rope_cache;           /* [B, capacity, G, R] bfloat16, or NULL               */
+  const int32_t* positions;   /* [B] first position per batch entry, or NULL         */
+  int32_t position;           /* first position for every batch entry (positions NULL) */
+  int32_t batch, new_tokens, groups, dim, rope_dim, capacity;
+  int32_t pow2_scales;
+  int32_t reserved;
+} cppmega_mi355_cache_append_args_t;
+
+int cppmega_mi355_kv_cache_append(const cppmega_mi355_cache_append_args_t* args, size_t args_size, void* stream);
+
+/* ---- sparse index producers -------------------------------------------------------------
+ * causal_sparse_indices (cppmega_mlx/nn/attention.py:251-284):
+ *   indices[b, s, g, j] = query_offset + s - j if that lies in [0, key_length), else -1.
+ * sparse_indices_from_attention_mask (attention.py:287-360): per (b, s, g) the newest
+ *   n = min(topk, key_length) valid keys of the mask row in ascending order, right-aligned,
+ *   -1 in front when fewer are valid.  A key is valid where a boolean mask is non-zero or a
+ *   float mask is finite.  The mask is addressed as mask[b*stride_b + g*stride_g +
+ *   s*stride_s + k] (strides in elements; 0 broadcasts). */
+typedef struct cppmega_mi355_causal_indices_args {
+  uint32_t struct_size;
+  int32_t index_dtype;        /* I32 or I64                                          */
+  void* indices;              /* [B, S, G, topk]                                     */
+  int32_t batch, seq, groups, topk;
+  int64_t query_offset;
+  int64_t key_length;
+} cppmega_mi355_causal_indices_args_t;
+
+int cppmega_mi355_causal_sparse_indices(const cppmega_mi355_causal_indices_args_t* args, size_t args_size, void* stream);
+
+enum { CPPMEGA_MI355_MASK_BOOL = 0 /* one byte per key */, CPPMEGA_MI355_MASK_F32 = 1, CPPMEGA_MI355_MASK_F16 = 2, CPPMEGA_MI355_MASK_BF16 = 3 };
+
+typedef struct cppmega_mi355_mask_indices_args {
+  uint32_t struct_size;
+  int32_t mask_dtype;         /* CPPMEGA_MI355_MASK_*                                */
+  const void* mask;
+  int64_t stride_b, stride_g, stride_s;
+  int32_t batch, seq, groups, topk, key_length;
+  int32_t reserved;
+  int32_t* indices;           /* [B, S, G, min(topk, key_length)] int32              */
+} cppmega_mi355_mask_indices_args_t;
+
+int cppmega_mi355_mask_sparse_indices(const cppmega_mi355_mask_indices_args_t* args, size_t args_size, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
