@@ -313,6 +313,42 @@ def bench_copy(args, device):
             "gbs": 2.0 * n / per / 1e9}
 
 
+def bench_next_rows(args, device):
+    """The rows either side of the attention call: the fused producer + cache append for a
+    prefill chunk (8192 latent rows of 512 + 64 rope channels) and for one decode step (32 rows),
+    and the two index producers at prefill size.  HBM-bound; bytes are algorithmic."""
+    from cppmega_mlx_amd import ops
+    gen = torch.Generator(device=device).manual_seed(99)
+    res = {}
+    steps = max(args.steps, 30)
+
+    def hbm(name, fn, nbytes, workload):
+        secs, _ = timed_graph([fn], steps, args.warmup)
+        per = secs / steps
+        res[name] = {"workload": workload, "us_per_launch": per * 1e6, "algorithmic_bytes": nbytes,
+                     "roofline": {"bound": "hbm", "achieved": nbytes / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": nbytes / per / 1e9 / HBM_PEAK_GBS, "traffic": None}}
+
+    for tag, B, S, cap in (("append_prefill", 1, 8192, 8192), ("append_decode", 32, 1, 4096)):
+        lat = torch.randn((B, S, 1, 512), generator=gen, device=device).to(torch.bfloat16)
+        rope = torch.randn((B, S, 1, 64), generator=gen, device=device).to(torch.bfloat16)
+        kv = torch.zeros((B, cap, 1, 512), dtype=torch.uint8, device=device)
+        sc = torch.zeros((B, cap, 1, 4), dtype=torch.float32, device=device)
+        rp = torch.zeros((B, cap, 1, 64), dtype=torch.bfloat16, device=device)
+        hbm(tag, lambda lat=lat, rope=rope, kv=kv, sc=sc, rp=rp: ops.kv_cache_append(
+                lat, kv_cache=kv, scale_cache=sc, position=0, rope=rope, rope_cache=rp, scale_block=128, pow2_scales=True),
+            B * S * (512 * 2 + 64 * 2 + 656),
+            f"bf16 latent[{B},{S},1,512] + rope[..,64] -> e4m3 + fp32/128 scales + bf16 rope at the cache position")
+    S = K = 8192
+    out = torch.empty((1, S, 1, 2048), dtype=torch.int32, device=device)
+    hbm("causal_indices", lambda: ops.causal_sparse_indices(out, query_offset=0, key_length=K), out.numel() * 4,
+        "causal_sparse_indices(1, 8192, 1, 2048) int32")
+    mask = (torch.arange(K, device=device)[None, :] <= torch.arange(S, device=device)[:, None]).contiguous()
+    hbm("mask_indices", lambda: ops.mask_sparse_indices(mask[None, None], out, topk=2048), mask.numel() + out.numel() * 4,
+        "sparse_indices_from_attention_mask: bool mask [8192, 8192] -> int32 [1,8192,1,2048]")
+    return res
+
+
 def measured_traffic(name):
     """HBM bytes per launch from the committed rocprofv3 counter runs, or None."""
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
@@ -328,7 +364,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="decode,vecmat,topk")
+    ap.add_argument("--only", type=str, default="decode,vecmat,topk,next")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -395,6 +431,8 @@ def main() -> int:
         line["prefill"] = bench_prefill(args, device)
     if "copy" in parts:
         line["copy"] = bench_copy(args, device)
+    if "next" in parts:
+        line["next_rows"] = bench_next_rows(args, device)
     print(json.dumps(line))
     return 0
 

@@ -174,11 +174,23 @@ __global__ __launch_bounds__(256) void cache_append_kernel(const AppendParams p)
     for (int pc = 0; pc < kMaxPieces; ++pc) {
       am[pc] = 0.0f;
       const int c0 = pc * 512 + lane * 8;
+      const bool live = pc < pieces && c0 < p.D;           // (D % 128 == 0: a lane's 8 channels are all in or all out)
+      if (live && p.src_dtype != CPPMEGA_MI355_F32) {      // 16-bit sources: one 16-byte load
+        const uint4 t = *reinterpret_cast<const uint4*>((const unsigned short*)p.src + sbase + c0);
+        const unsigned w[4] = {t.x, t.y, t.z, t.w};
+        const bool bf = p.src_dtype == CPPMEGA_MI355_BF16;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        v[pc][i] = (pc < pieces && c0 + i < p.D) ? load_as(p.src, sbase + c0 + i, p.src_dtype) : 0.0f;
-        am[pc] = fmaxf(am[pc], fabsf(v[pc][i]));
+        for (int i = 0; i < 4; ++i) {
+          const unsigned short lo = (unsigned short)(w[i] & 0xffffu), hi = (unsigned short)(w[i] >> 16);
+          v[pc][2 * i] = bf ? bf16_bits_to_f32(lo) : f16_bits_to_f32(lo);
+          v[pc][2 * i + 1] = bf ? bf16_bits_to_f32(hi) : f16_bits_to_f32(hi);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[pc][i] = live ? load_as(p.src, sbase + c0 + i, p.src_dtype) : 0.0f;
       }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) am[pc] = fmaxf(am[pc], fabsf(v[pc][i]));
 #pragma unroll
       for (int off = 1; off <= 8; off <<= 1) am[pc] = fmaxf(am[pc], __shfl_xor(am[pc], off, 64));   // the lane's 128-channel block
     }

@@ -4,11 +4,12 @@
 //   causal   indices[b, s, g, j] = query_offset + s - j if in [0, key_length), else -1.
 //            One thread per output element; pure index arithmetic, write-bound.
 //   mask     per (b, s, g): the newest n = min(topk, key_length) valid keys of the mask row,
-//            ascending, right-aligned, -1 in front.  One wavefront per row, two passes over
-//            the row: count the valid keys, then place key number r (ascending among the
-//            valid ones, V in all) at slot n - V + r if that is >= 0.  A lane reads 16 mask
-//            bytes (boolean masks) or one float per step; ranks come from popcounts and a
-//            wavefront prefix sum.
+//            ascending, right-aligned, -1 in front.  One wavefront per row: count the valid
+//            keys (the validity bits of up to 16384 keys stay in registers, longer rows are
+//            read a second time), then place key number r (ascending among the valid ones, V
+//            in all) at slot n - V + r if that is >= 0.  A lane reads 16 mask bytes (boolean
+//            masks) or 16 floats per step; ranks come from popcounts and a wavefront prefix
+//            sum; the kept keys of a step pass through LDS so that they leave coalesced.
 
 #include "common.h"
 
@@ -30,6 +31,24 @@ __global__ __launch_bounds__(256) void causal_indices_kernel(const CausalParams 
     const long long v = (pos >= 0 && pos < p.klen) ? pos : -1;
     if (p.wide) ((long long*)p.out)[i] = v;
     else ((int*)p.out)[i] = (int)v;
+  }
+}
+
+// int32 output, topk a multiple of 4: a thread writes four consecutive window slots (16 bytes);
+// total / 4 fits 32 bits (checked on the host), so the index arithmetic is 32-bit
+__global__ __launch_bounds__(256) void causal_indices_vec4_kernel(const CausalParams p) {
+  const unsigned quads = (unsigned)(p.total >> 2), per_row = (unsigned)p.topk >> 2;
+  for (unsigned q = blockIdx.x * 256u + threadIdx.x; q < quads; q += gridDim.x * 256u) {
+    const unsigned row = q / per_row;                      // (b * S + s) * G + g
+    const int j0 = (int)(q - row * per_row) * 4;
+    const int s = (int)((row / (unsigned)p.G) % (unsigned)p.S);
+    const long long pos0 = p.qoff + s - j0;
+    int4 v;
+    v.x = (pos0 >= 0 && pos0 < p.klen) ? (int)pos0 : -1;
+    v.y = (pos0 - 1 >= 0 && pos0 - 1 < p.klen) ? (int)(pos0 - 1) : -1;
+    v.z = (pos0 - 2 >= 0 && pos0 - 2 < p.klen) ? (int)(pos0 - 2) : -1;
+    v.w = (pos0 - 3 >= 0 && pos0 - 3 < p.klen) ? (int)(pos0 - 3) : -1;
+    reinterpret_cast<int4*>(p.out)[q] = v;
   }
 }
 
@@ -63,7 +82,13 @@ __device__ __forceinline__ unsigned valid16(const MaskParams& p, const unsigned 
       const uint4 t = *reinterpret_cast<const uint4*>(row + k0);
       const unsigned w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
-      for (int i = 0; i < 16; ++i) bits |= (((w[i >> 2] >> (8 * (i & 3))) & 0xffu) ? 1u : 0u) << i;
+      for (int d = 0; d < 4; ++d) {
+        // non-zero byte -> 0x01 per byte (x | x>>1 | .. folded into bit 0), then the four bit 0s gathered by a multiply (byte i -> bit 24 + i)
+        unsigned x = w[d];
+        x |= x >> 4; x |= x >> 2; x |= x >> 1;
+        x &= 0x01010101u;
+        bits |= (((x * 0x01020408u) >> 24) & 0xfu) << (4 * d);
+      }
     } else {
       for (int i = 0; i < 16 && k0 + i < p.K; ++i) bits |= (row[k0 + i] ? 1u : 0u) << i;
     }
@@ -91,30 +116,52 @@ __global__ __launch_bounds__(256) void mask_indices_kernel(const MaskParams p) {
   const unsigned char* row = (const unsigned char*)p.mask + ((long long)b * p.sb + (long long)g * p.sg + (long long)s * p.ss) * ES;
   const bool vec_ok = (((size_t)row) & 15) == 0;
   int* out = p.out + r * p.n;
-  // pass 1: number of valid keys
+  __shared__ int strips[4][1024];
+  int* strip = strips[threadIdx.x >> 6];
+  // pass 1: validity bits (kept in registers for rows of up to 16384 keys) and their number
+  constexpr int kKeep = 16;
+  unsigned kept[kKeep];
   int mine = 0;
-  for (long long k0 = (long long)lane * 16; k0 < p.K; k0 += 64 * 16) mine += __popc(valid16<DT>(p, row, k0, vec_ok));
+  {
+    int st = 0;
+    for (long long k0 = (long long)lane * 16; k0 < p.K; k0 += 64 * 16, ++st) {
+      const unsigned bits = valid16<DT>(p, row, k0, vec_ok);
+      if (st < kKeep) kept[st] = bits;
+      mine += __popc(bits);
+    }
+  }
   int V;
   (void)wave_exclusive(mine, lane, V);
   // leading -1 slots
   const int lead = max(p.n - V, 0);
   for (int i = lane; i < lead; i += 64) out[i] = -1;
-  // pass 2: place the newest n
+  // pass 2: place the newest n; key number r (ascending among the valid ones) goes to slot n - V + r
+  const int first = V - p.n;                                                    // ranks below this are dropped
   int before = 0;                                                               // valid keys in earlier steps
-  for (long long base = 0; base < p.K; base += 64 * 16) {
+  int st = 0;
+  for (long long base = 0; base < p.K; base += 64 * 16, ++st) {
     const long long k0 = base + (long long)lane * 16;
-    const unsigned bits = k0 < p.K ? valid16<DT>(p, row, k0, vec_ok) : 0u;
+    unsigned bits = 0u;
+    if (k0 < p.K) bits = st < kKeep ? kept[st] : valid16<DT>(p, row, k0, vec_ok);
+    const int cnt = __popc(bits);
     int step_total;
-    int rank = before + wave_exclusive(__popc(bits), lane, step_total);
+    int rank = before + wave_exclusive(cnt, lane, step_total);
+    before += step_total;
+    if (before <= first) continue;                                              // (uniform) nothing of this step is kept
+    // the step's kept keys go through this wavefront's LDS strip in rank order and leave as
+    // whole 256-byte stores (a lane's keys are consecutive ranks: direct stores would scatter)
+    const int step_rank0 = before - step_total;                                 // rank of the step's first valid key
     unsigned rest = bits;
+    int rloc = rank - step_rank0;                                               // 0 .. 1023
     while (rest) {
       const int i = __builtin_ctz(rest);
       rest &= rest - 1;
-      const int slot = p.n - V + rank;
-      if (slot >= 0) out[slot] = (int)(k0 + i);
-      ++rank;
+      strip[rloc++] = (int)(k0 + i);
     }
-    before += step_total;
+    __builtin_amdgcn_wave_barrier();
+    const int lo = max(first - step_rank0, 0);                                  // first kept entry of the strip
+    for (int e = lo + lane; e < step_total; e += 64) out[step_rank0 + e - first] = strip[e];
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -134,8 +181,13 @@ int causal_indices_launch(const cppmega_mi355_causal_indices_args_t& a, hipStrea
   p.out = a.indices; p.S = a.seq; p.G = a.groups; p.topk = a.topk; p.wide = a.index_dtype == CPPMEGA_MI355_I64;
   p.qoff = a.query_offset; p.klen = a.key_length;
   p.total = (long long)a.batch * a.seq * a.groups * a.topk;
-  const unsigned blocks = (unsigned)min((p.total + 255) / 256, (long long)256 * 32);
-  hipLaunchKernelGGL(causal_indices_kernel, dim3(blocks), dim3(256), 0, stream, p);
+  if (!p.wide && a.topk % 4 == 0 && (((size_t)a.indices) & 15) == 0 && (p.total >> 2) < 0xffffffffll) {
+    const unsigned blocks = (unsigned)min(((p.total >> 2) + 255) / 256, (long long)256 * 32);
+    hipLaunchKernelGGL(causal_indices_vec4_kernel, dim3(blocks), dim3(256), 0, stream, p);
+  } else {
+    const unsigned blocks = (unsigned)min((p.total + 255) / 256, (long long)256 * 32);
+    hipLaunchKernelGGL(causal_indices_kernel, dim3(blocks), dim3(256), 0, stream, p);
+  }
   CM_HIP_CHECK(hipGetLastError());
   return 0;
 }
