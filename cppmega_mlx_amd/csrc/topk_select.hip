@@ -33,6 +33,8 @@
 // real number can reach (0x7f9..0x7ff, 0xff9..0xfff); those bins are cleared
 // before the scan instead of testing every element.
 
+#include <cstdlib>
+
 #include "common.h"
 
 namespace cm {
@@ -207,9 +209,8 @@ constexpr int kTileThreads = 256;
 constexpr int kTileScratch = kHistBins + 64;            // words: histogram + scan scratch
 __host__ __device__ constexpr int tile_pad(int E) { return E == 4 ? 0 : 4; }
 
-template <typename ScoreT, int E, int VEC>
-__global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParams p) {
-  constexpr int THREADS = kTileThreads;
+template <typename ScoreT, int E, int VEC, int THREADS = kTileThreads>
+__global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) {
   constexpr int ITEMS = E / VEC;                        // loads per thread
   constexpr int CHUNK = THREADS * VEC;                  // columns covered by one load per thread
   constexpr int PITCH = E + tile_pad(E);                // words between the runs of consecutive threads
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParam
   }
   __syncthreads();
   // two cleared histograms: pass 1 uses the first, pass 2 the second (no clear + barrier in between)
-  constexpr int kHist2 = (kTileThreads * PITCH >= 2 * kHistBins + 64) ? kHistBins + 64 : 0;
+  constexpr int kHist2 = (THREADS * PITCH >= 2 * kHistBins + 64) ? kHistBins + 64 : 0;
   zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
   __syncthreads();
 
@@ -317,7 +318,8 @@ __global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParam
         lo_bits = (p2 << 8) | (neg ? 0xffu : 0u);
       } else {
         // ---- pass 3: bits[7:0] (256 of 1024 cleared slots are used) ------------------
-        zero_hist<THREADS>(hist, 1024);
+        constexpr int NB3 = 4 * THREADS > 1024 ? 4 * THREADS : 1024;   // the scan wants one quad per thread at least
+        zero_hist<THREADS>(hist, NB3);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < E; ++i) {
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(kTileThreads) void topk_tile_kernel(const TopkParam
           if ((u >> 8) == p2) atomicAdd(&hist[u & 0xffu], 1u);
         }
         __syncthreads();
-        const BinHit h3 = find_bin<1024, THREADS>(smem, rem, neg ? kAscending : kDescending);
+        const BinHit h3 = find_bin<NB3, THREADS>(smem, rem, neg ? kAscending : kDescending);
         rem -= h3.above;
         lo_bits = (p2 << 8) | h3.bin;
         tie = rem != h3.cnt;
@@ -612,29 +614,40 @@ int launch_kernel(K kernel, const TopkParams& p, int threads, size_t smem, hipSt
   return 0;
 }
 
+static int wide_threads() {
+  if (const char* e = getenv("CPPMEGA_MI355_TOPK_THREADS")) {
+    const int v = atoi(e);
+    if (v == 256 || v == 512) return v;
+  }
+  return 512;
+}
+
 template <typename ScoreT>
 int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* smem_out) {
   const int T = p.width;
   const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
   const size_t out_words = sorted ? (size_t)p.sort_len * 2 : (size_t)p.k;
   if (T <= 8192) {
-    auto tile_smem = [&](int E) {
-      const size_t tile_words = (size_t)kTileThreads * (E + tile_pad(E));
+    auto tile_smem = [&](int E, int threads) {
+      const size_t tile_words = (size_t)threads * (E + tile_pad(E));
       const size_t need = (size_t)kTileScratch + out_words;
       return (need > tile_words ? need : tile_words) * 4;
     };
-#define CM_TOPK_TILE(E)                                                                   \
+#define CM_TOPK_TILE(E, THR)                                                              \
   do {                                                                                    \
-    const size_t smem = tile_smem(E);                                                     \
+    const size_t smem = tile_smem(E, THR);                                                \
     *smem_out = smem;                                                                     \
     if (smem > 160 * 1024) return -3;                                                     \
-    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4>, p, kTileThreads, smem, stream) \
-                : launch_kernel(topk_tile_kernel<ScoreT, E, 1>, p, kTileThreads, smem, stream); \
+    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4, THR>, p, THR, smem, stream) \
+                : launch_kernel(topk_tile_kernel<ScoreT, E, 1, THR>, p, THR, smem, stream); \
   } while (0)
-    if (T <= 1024) CM_TOPK_TILE(4);
-    if (T <= 2048) CM_TOPK_TILE(8);
-    if (T <= 4096) CM_TOPK_TILE(16);
-    CM_TOPK_TILE(32);
+    if (T <= 1024) CM_TOPK_TILE(4, kTileThreads);
+    if (T <= 2048) CM_TOPK_TILE(8, kTileThreads);
+    if (T <= 4096) CM_TOPK_TILE(16, kTileThreads);
+    // the widest rows: 512 threads x 16 columns (twice the wavefronts per row shorten every phase
+    // of the row's pipeline, and the narrower runs need fewer registers)
+    if (wide_threads() == 512) CM_TOPK_TILE(16, 512);
+    CM_TOPK_TILE(32, kTileThreads);
 #undef CM_TOPK_TILE
   }
   const size_t smem = ((size_t)kWideScratch + out_words) * 4;
