@@ -306,3 +306,51 @@ def test_path_c_float_carrier_owner_output_validation(monkeypatch):
         pc.sparse_mla_fwd_path_c(q, kv, idx, sm_scale_buf=torch.ones(1), out=out[..., :4], lse=lse)
     with pytest.raises(TypeError, match="indices must be int32 or int64"):
         pc.sparse_mla_fwd_path_c(q, kv, idx.short(), sm_scale_buf=torch.ones(1), out=out, lse=lse)
+
+
+# ---- index producers and the sparse FP8 cache: argument contracts (no GPU needed) -----------
+
+def test_causal_sparse_indices_argument_contract():
+    from cppmega_mlx_amd.nn.attention import causal_sparse_indices
+    for bad in (dict(batch_size=0), dict(seq_length=0), dict(kv_group=0), dict(topk=0), dict(query_offset=-1), dict(key_length=0)):
+        args = dict(batch_size=1, seq_length=2, kv_group=1, topk=2, query_offset=0, key_length=2)
+        args.update(bad)
+        with pytest.raises(ValueError):
+            causal_sparse_indices(**args, device="cpu")
+
+
+def test_mask_sparse_indices_argument_contract():
+    import torch
+    from cppmega_mlx_amd.nn.attention import sparse_indices_from_attention_mask
+    kw = dict(batch_size=1, seq_length=3, kv_group=1, topk=2, key_length=4)
+    m = torch.ones((3, 4), dtype=torch.bool)
+    with pytest.raises(TypeError):
+        sparse_indices_from_attention_mask([[True]], **kw)
+    with pytest.raises(ValueError):
+        sparse_indices_from_attention_mask(m[None, None, None], **kw)
+    with pytest.raises(ValueError):
+        sparse_indices_from_attention_mask(m, **{**kw, "key_length": 5})
+    with pytest.raises(ValueError):
+        sparse_indices_from_attention_mask(m.expand(3, 3, 4), **kw)
+    with pytest.raises(ValueError):
+        sparse_indices_from_attention_mask(m.expand(1, 3, 3, 4), **kw)
+    for bad in ("batch_size", "seq_length", "kv_group", "topk", "key_length"):
+        with pytest.raises(ValueError):
+            sparse_indices_from_attention_mask(m, **{**kw, bad: 0})
+
+
+def test_sparse_fp8_cache_config_contract():
+    from cppmega_mlx_amd.inference import SparseFP8KVCacheConfig
+    ok = dict(num_layers=1, batch_size=1, num_kv_heads=1, head_dim=512, max_seq_len=16)
+    SparseFP8KVCacheConfig(**ok)
+    for bad in ("num_layers", "batch_size", "num_kv_heads", "head_dim", "max_seq_len"):
+        with pytest.raises(ValueError):
+            SparseFP8KVCacheConfig(**{**ok, bad: 0})
+        with pytest.raises(TypeError):
+            SparseFP8KVCacheConfig(**{**ok, bad: 1.5})
+    with pytest.raises(ValueError):
+        SparseFP8KVCacheConfig(**{**ok, "head_dim": 100})
+    with pytest.raises(ValueError):
+        SparseFP8KVCacheConfig(**{**ok, "scale_block": 64})
+    with pytest.raises(ValueError):
+        SparseFP8KVCacheConfig(**{**ok, "rope_dim": -1})
