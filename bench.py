@@ -413,7 +413,7 @@ def main() -> int:
         torch.cuda.empty_cache()
     if "vecmat" in parts:
         line["vecmat"] = {}
-        for M in (1, 4, 16):
+        for M in (1, 4, 16, 32):
             res, sample = bench_vecmat(args, device, M)
             if not args.no_cpu_baseline and M == 1:
                 res["cpu_baseline"], res["max_rel_err_vs_oracle_on_sample"] = cpu_baseline_vecmat(sample)

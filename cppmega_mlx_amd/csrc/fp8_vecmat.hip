@@ -14,8 +14,9 @@
 //    the row sum is a wavefront reduction followed by a 4-way LDS combine.
 //  * 2 <= M <= 4, bf16 activations (gemv_stream_kernel): the same streaming shape with the
 //    M activation rows held in registers and v_dot2_f32_bf16 accumulation.
-//  * 5 <= M <= 16, bf16 activations (skinny_mfma_kernel): v_mfma_f32_16x16x32_bf16 with 16
-//    weight rows as the M side and the (padded) activation rows as the N side.  A
+//  * 5 <= M <= 32, bf16 activations (skinny_mfma_kernel): v_mfma_f32_16x16x32_bf16 with 16
+//    weight rows as the M side and the (padded) activation rows, in one or two groups of 16,
+//    as the N side.  A
 //    workgroup owns 16 weight rows; its 8 wavefronts own one eighth of K each and add
 //    their 16x16 partial tiles through LDS at the end, so nothing but the result is
 //    written to memory.  Weight fragments go from HBM straight into registers
@@ -301,15 +302,16 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
   }
 }
 
-// 5 <= M <= 16 with bf16 activations, K a multiple of 1024: see the file header.
+// 5 <= M <= 32 with bf16 activations, K a multiple of 1024: see the file header.  MT: groups of 16 activation rows.
 constexpr int kSkinnySplits = 8;         // K is cut into eighths, one per workgroup column
 constexpr int kSkinnyWaves = 7;          // 448 row tiles x 8 splits = 256 workgroups x 7 wavefronts x 2 tiles at N = 7168
 constexpr int kSkinnyDepth = 8;          // 64-channel weight steps in flight per wavefront
 constexpr int kSkinnyMaxKw = 2048;       // channels per split the LDS activation slice can hold
 constexpr int kXPitchBytes = kSkinnyMaxKw * 2 + 16;   // row pitch of the slice: 16 rows fall on distinct banks
 
+template <int MT>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const VecmatParams p) {
-  extern __shared__ __align__(16) unsigned char xs[];    // [16][kXPitchBytes]: bf16 activations of this split
+  extern __shared__ __align__(16) unsigned char xs[];    // [16 MT][kXPitchBytes]: bf16 activations of this split
   const int lane = lane_id();
   const int wave = (int)(threadIdx.x >> 6);
   const int K = p.k;
@@ -318,7 +320,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   const int k0 = split * kw;
   const int steps = kw / 64;
   // activation slice -> LDS (rows >= M are zero)
-  for (int i = (int)threadIdx.x; i < 16 * (kw / 8); i += kSkinnyWaves * 64) {
+  for (int i = (int)threadIdx.x; i < 16 * MT * (kw / 8); i += kSkinnyWaves * 64) {
     const int m = i / (kw / 8), c = i % (kw / 8);
     uint4 v = make_uint4(0, 0, 0, 0);
     if (m < p.m) v = *reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k0 + 8 * c);
@@ -366,7 +368,9 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   float sq_next[kSkinnyDepth / 2];
 #pragma unroll
   for (int i = 0; i < kSkinnyDepth / 2; ++i) sq_next[i] = 1.0f;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   int st = 0, tile = first;                              // position of flat step f0 + d, tracked incrementally
   for (int f0 = 0; f0 < total; f0 += kSkinnyDepth) {     // steps is a multiple of the depth? not required: see the guards
 #pragma unroll
@@ -379,8 +383,12 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
       if ((d & 1) == 0) sq_next[d >> 1] = sc_next;       // takes effect once the odd step of the pair is done
       else sq[d >> 1] = sq_next[d >> 1];
       if (f < total) {                                   // (uniform)
-        const uint4 x0 = *reinterpret_cast<const uint4*>(xrow + 128 * st);
-        const uint4 x1 = *reinterpret_cast<const uint4*>(xrow + 128 * st + 16);
+        uint4 x0[MT], x1[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          x0[mt] = *reinterpret_cast<const uint4*>(xrow + mt * 16 * kXPitchBytes + 128 * st);
+          x1[mt] = *reinterpret_cast<const uint4*>(xrow + mt * 16 * kXPitchBytes + 128 * st + 16);
+        }
         bf16x8 a0, a1;
         const bool pow2 = (__float_as_uint(sc) & 0x007fffffu) == 0u && sc > 0.0f && sc < INFINITY;
         if (__ballot(!pow2) == 0ull) {                   // the conversion applies a power-of-two scale exactly
@@ -410,22 +418,29 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
           a0 = __builtin_bit_cast(bf16x8, make_uint4(o[0], o[1], o[2], o[3]));
           a1 = __builtin_bit_cast(bf16x8, make_uint4(o[4], o[5], o[6], o[7]));
         }
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, x0), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, x1), acc, 0, 0, 0);
-        if (++st == steps) {                             // (uniform) tile finished: partial[split][m][row]
-          // lane (m = lane%16, g = lane/16) holds weight rows 4g + i of activation m
-          const int row0 = tile * 16;
-          if (r16 < p.m) {
-            float* dst = p.partial + ((size_t)split * p.m + r16) * p.n + row0 + 4 * kq;
-            if (row0 + 4 * kq + 3 < p.n && (p.n & 3) == 0) {
-              *reinterpret_cast<float4*>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-            } else {
 #pragma unroll
-              for (int i = 0; i < 4; ++i)
-                if (row0 + 4 * kq + i < p.n) dst[i] = acc[i];
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, x0[mt]), acc[mt], 0, 0, 0);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, x1[mt]), acc[mt], 0, 0, 0);
+        }
+        if (++st == steps) {                             // (uniform) tile finished: partial[split][m][row]
+          // lane (m = lane%16, g = lane/16) holds weight rows 4g + i of activation 16 mt + m
+          const int row0 = tile * 16;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const int m = 16 * mt + r16;
+            if (m < p.m) {
+              float* dst = p.partial + ((size_t)split * p.m + m) * p.n + row0 + 4 * kq;
+              if (row0 + 4 * kq + 3 < p.n && (p.n & 3) == 0) {
+                *reinterpret_cast<float4*>(dst) = make_float4(acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]);
+              } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  if (row0 + 4 * kq + i < p.n) dst[i] = acc[mt][i];
+              }
             }
+            acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
           }
-          acc = f32x4{0.f, 0.f, 0.f, 0.f};
           st = 0;
           tile += kSkinnyWaves;
         }
@@ -496,9 +511,9 @@ static bool vecmat_aligned(const cppmega_mi355_vecmat_args_t& a) {
 static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) {
   return a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 4096 == 0) && a.k <= 16384;
 }
-// the split-K MFMA kernel: bf16 activations, 2 <= M <= 16, K in eighths of whole scale blocks that fit the LDS slice
+// the split-K MFMA kernel: bf16 activations, 2 <= M <= 32, K in eighths of whole scale blocks that fit the LDS slice
 static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
-  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 2 && a.m <= 16 && !stream_shape(a) &&
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 2 && a.m <= 32 && !stream_shape(a) &&
          (a.k % (kSkinnySplits * 128) == 0) && a.k / kSkinnySplits <= kSkinnyMaxKw;
 }
 static bool skinny_ok(const cppmega_mi355_vecmat_args_t& a) { return vecmat_aligned(a) && skinny_shape(a); }
@@ -587,9 +602,15 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     if (per_wave < 1) per_wave = 1;
     p.rows_per_wg = per_wave * kSkinnyWaves;
     const dim3 grid((unsigned)((tiles + p.rows_per_wg - 1) / p.rows_per_wg), kSkinnySplits), block(kSkinnyWaves * 64);
-    const int smem = 16 * kXPitchBytes;
-    CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    hipLaunchKernelGGL(skinny_mfma_kernel, grid, block, smem, stream, p);
+    if (a.m <= 16) {
+      const int smem = 16 * kXPitchBytes;
+      CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+      hipLaunchKernelGGL(skinny_mfma_kernel<1>, grid, block, smem, stream, p);
+    } else {
+      const int smem = 32 * kXPitchBytes;
+      CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+      hipLaunchKernelGGL(skinny_mfma_kernel<2>, grid, block, smem, stream, p);
+    }
     CM_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(skinny_reduce_kernel, dim3((unsigned)(((size_t)a.m * a.n + 255) / 256)), dim3(256), 0, stream, p);
   } else if (a.m == 1 && aligned) {

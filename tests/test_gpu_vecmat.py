@@ -37,7 +37,8 @@ def _oracle_blocked(codes, scale, x):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (1, 100, 4096), (1, 33, 2560), (1, 16, 32768), (1, 7, 100),
-                                   (2, 64, 1024), (4, 257, 4096), (16, 130, 2048), (5, 48, 1000)])
+                                   (2, 64, 1024), (4, 257, 4096), (16, 130, 2048), (5, 48, 1000),
+                                   (17, 130, 2048), (32, 200, 4096), (24, 64, 16384), (33, 40, 2048)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_block_scaled_bf16_activation(device, M, N, K, out_dtype):
     rng = np.random.default_rng(M * 1000003 + N * 101 + K)
@@ -94,7 +95,7 @@ def test_fused_fp8_gemm_grid_scales_and_leading_dims(device):
     assert err <= F32_TOL * ref
 
 
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 4, 16, 32])
 def test_headline_config_full_size(device, M):
     """W e4m3 [7168, 16384], fp32 scale per 1x128 (power of two), x bf16 [M, 16384] -> bf16 [M, 7168]."""
     rng = np.random.default_rng(7168 + M)
