@@ -207,7 +207,7 @@ def bench_vecmat(args, device, M: int):
         "algorithmic_bytes": bytes_alg,
         "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS,
-                     "traffic": measured_traffic({1: "fp8_vecmat", 4: "fp8_vecmat_m4", 16: "fp8_vecmat_m16"}.get(M, ""))},
+                     "traffic": measured_traffic({1: "fp8_vecmat", 4: "fp8_vecmat_m4", 16: "fp8_vecmat_m16", 32: "fp8_vecmat_m32"}.get(M, ""))},
     }
     return res, (xs[0], ws[0], ss[0], outs[0])
 
