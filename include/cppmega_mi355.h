@@ -301,7 +301,10 @@ int cppmega_mi355_fp8_quantize(const cppmega_mi355_quantize_args_t* args, size_t
  *                       448 * s >= amax (1.0 for an all-zero block): the latent cache format
  *                       the decode kernel gathers.
  * rope (optional, [B, S_new, G, R] float32/float16/bfloat16) is stored as bfloat16.
- * D % 128 == 0, D <= 2048, R <= 256. */
+ * D % 128 == 0, D <= 2048, R <= 256.  With `positions` NULL the range position ..
+ * position + S_new - 1 is checked against the capacity on the host (ERR_SHAPE); per-batch
+ * positions live on the device, so rows that would fall outside [0, capacity) are skipped
+ * by the kernel instead. */
 typedef struct cppmega_mi355_cache_append_args {
   uint32_t struct_size;
   int32_t src_dtype;          /* E4M3 (prepared) or F32/F16/BF16 (quantise)          */
