@@ -267,6 +267,47 @@ def test_decode_full_config_sampled_batches(device):
     assert np.abs(lse_m - got_lse).max() <= 1e-4
 
 
+def test_prefill_full_config_sampled_queries(device):
+    """B=1, S=8192, H=128, topk=2048 with causal top-k indices over an 8192-token FP8 cache: the
+    whole chunk runs on the GPU (indices from the GPU selector), sampled queries -- heavily
+    padded early ones, the 2047/2048 boundary, the last -- are checked against the oracle, and
+    every query with no visible key beyond itself must reproduce its own value row."""
+    from cppmega_mlx_amd import _lib
+    from cppmega_mlx_amd.nn._tilelang import topk_selector as tk
+    S, H, topk = 8192, 128, 2048
+    gen = torch.Generator(device=device).manual_seed(17)
+    lat = torch.randn((S, 1, 4, 128), generator=gen, device=device)
+    sc = torch.exp2(torch.ceil(torch.log2(lat.abs().amax(dim=-1) / 448.0)))
+    codes = (lat / sc[..., None]).to(torch.float8_e4m3fn).view(torch.uint8).reshape(1, S, 1, 512)
+    scale = sc.reshape(1, S, 1, 4).contiguous()
+    rope = torch.randn((1, S, 1, 64), generator=gen, device=device).to(torch.bfloat16)
+    q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.bfloat16)
+    ends = torch.arange(1, S + 1, device=device, dtype=torch.int32)
+    idx = torch.empty((S, topk), dtype=torch.int32, device=device)
+    tk.topk_selector_tilelang_direct(torch.randn((S, S), generator=gen, device=device), topk, out=idx, ends=ends, order="index")
+    idx = idx.view(1, S, 1, topk)
+    spec = ops.QuantSpec(_lib.SCALE_F32_BLOCK, scale, 128)
+    out = torch.zeros((1, S, H, 512), dtype=torch.bfloat16, device=device)
+    lse = torch.zeros((1, S, H), dtype=torch.float32, device=device)
+    ops.sparse_mla_forward(q, codes, idx, sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse, kv_spec=spec, kv_rope=rope)
+    torch.cuda.synchronize()
+    assert ops.sparse_mla_selected_kernel(q, codes, idx, d_v=512, kv_spec=spec, kv_rope=rope) == "mfma"
+    idx_np = idx.cpu().numpy().astype(np.int64)
+    assert ((idx_np[0, :, 0, :] >= 0).sum(axis=-1) == np.minimum(np.arange(1, S + 1), topk)).all()
+    rows_all = om.dequant_block_latent(codes.cpu().numpy(), scale.cpu().numpy(), rope.float().cpu().numpy(), 128)
+    for s in (0, 1, 31, 33, 700, 2046, 2047, 2048, 5000, S - 1):
+        want_out, want_lse = om.sparse_mla_oracle(q[:, s:s + 1].float().cpu().numpy(), rows_all, idx_np[:, s:s + 1],
+                                                  sm_scale=576 ** -0.5, d_v=512)
+        err, ref = error_report(out[:, s:s + 1].float().cpu().numpy(), want_out)
+        assert err <= REL_TOL * ref, f"query {s}: max-abs {err:.3e} vs output scale {ref:.3e}"
+        assert np.abs(lse[:, s:s + 1].cpu().numpy() - want_lse).max() <= LSE_TOL_MFMA, f"query {s}"
+    # query 0 sees only key 0: softmax over one key is 1, the output is that key's value row for every head
+    v0 = rows_all[0, 0, 0, :512]
+    got0 = out[0, 0].float().cpu().numpy()
+    assert np.abs(got0 - v0[None, :]).max() <= 2.0 ** -8 * np.abs(v0).max() + 1e-6     # bf16 rounding of the output
+    assert not torch.isnan(out.float()).any()
+
+
 def test_tiny_bf16_config(device):
     """B=1, S_q=64, H=16, d_qk=576, d_v=512, Skv=256, topk=64, causal sampling, both windows."""
     for off in (0, 192):
