@@ -27,6 +27,7 @@
 //  * anything else (odd K, misaligned rows): rowwise_kernel, one wavefront per
 //    output row, scalar byte loads.
 
+#include <type_traits>
 #include <cstdlib>
 
 #include "common.h"
@@ -186,13 +187,16 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const VecmatParam
   }
 }
 
-// M <= 4 bf16 activations, K a multiple of 4096 up to 16384: the streaming kernel.
+// M <= 4 bf16 activations, K a multiple of 16 up to 32768: the streaming kernel.
+//   * W wavefronts share a row; a wavefront covers CH chunks of 1 KiB of it (16 bytes per lane).
+//     Lanes whose chunk lies past K take zero activations and re-read the row's first bytes, so
+//     the row loop itself carries no bounds test;
 //   * activations stay in registers as packed bf16 pairs;
 //   * weights go e4m3 -> bf16 pairs two bytes per instruction (exact) and meet
 //     the activations in v_dot2_f32_bf16, fp32 accumulation;
 //   * rows are processed in groups of U with the loads of the next group issued
 //     before the arithmetic of the current one (two register buffers);
-//   * per row: DPP wavefront reduction, then a fixed-order 4-way LDS combine.
+//   * per row group: one joint DPP reduction of its U x M sums, then a fixed-order LDS combine.
 
 __device__ __forceinline__ float wave_total_dpp(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, false));
@@ -204,22 +208,25 @@ __device__ __forceinline__ float wave_total_dpp(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
-template <int M, int CH, int U>
+constexpr int kStreamU = 2;              // rows per group (measured: 2 streams at least as fast as 4, in fewer registers)
+constexpr int kStreamMaxRows = 32;       // rows per workgroup, a multiple of kStreamU chosen by the host
+constexpr int kStreamMaxK = 8 * 4 * kChunk;
+
+template <int CH>
 struct StreamBuf {
-  uint4 w[U][CH];
-  float sc[U][CH];
+  uint4 w[kStreamU][CH];
+  float sc[kStreamU][CH];
 };
 
-// R rows per workgroup (a multiple of U): the host picks the R that spreads the rows most evenly
-// over the compute units
-template <int M, int CH, int U, int R>
-__global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const VecmatParams p) {
-  constexpr int G = R / U;
-  static_assert(R % U == 0, "whole row groups");
-  __shared__ float red[kGemvWaves][R][M];
+template <int M, int CH, int W>
+__global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams p) {
+  constexpr int U = kStreamU;
+  __shared__ float red[W][4][kStreamMaxRows][M];
   const int lane = lane_id();
   const int wave = (int)(threadIdx.x >> 6);
   const int K = p.k;
+  const int R = p.rows_per_wg;
+  const int G = R / U;
   const int row0 = (int)blockIdx.x * R;
   const int last_row = p.n - 1;
 
@@ -227,18 +234,23 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
   bf16x2 xp[M][CH][8];
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
-    koff[c] = (c * kGemvWaves + wave) * kChunk + lane * 16;
+    const int k = (c * W + wave) * kChunk + lane * 16;
+    const bool live = k < K;                       // (K is a multiple of 16: a lane's 16 channels are all in or all out)
+    koff[c] = live ? k : 0;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + koff[c]);
-      const uint4 a = src[0], b = src[1];
+      uint4 a = make_uint4(0, 0, 0, 0), b = a;
+      if (live) {
+        const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k);
+        a = src[0]; b = src[1];
+      }
       const unsigned wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
       for (int i = 0; i < 8; ++i) xp[m][c][i] = __builtin_bit_cast(bf16x2, wds[i]);
     }
   }
 
-  auto load = [&](StreamBuf<M, CH, U>& buf, int g) {
+  auto load = [&](StreamBuf<CH>& buf, int g) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int n = min(row0 + g * U + u, last_row);
@@ -250,12 +262,24 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
       }
     }
   };
-  auto compute = [&](const StreamBuf<M, CH, U>& buf, int g) {
+  // Per row group: U x M per-lane sums.  They are reduced together: select steps at lane distances
+  // 1 and 2 halve the number of live values (a lane keeps the value its low lane bits name and adds
+  // its partner's copy of it), then row shifts by (2,) 4 and 8 finish the 16-lane rows.  The last
+  // MP lanes of each 16-lane row then hold that row's sums; the four rows are added in the final
+  // combine.
+  constexpr int MP = M == 3 ? 4 : M;               // values per weight row in the reduction (a power of two)
+  const bool bit0 = (lane & 1) != 0, bit1 = (lane & 2) != 0;
+  const bool writer = (lane & 15) >= 16 - MP && (lane & (MP - 1)) < M;
+  const int lrow = lane >> 4, wm = lane & (MP - 1);
+  auto dpp_add = [](float v, float moved_src, auto ctrl) {
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, moved_src), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  auto compute = [&](const StreamBuf<CH>& buf, int g) {
+    float acc[U][MP];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      float acc[M];
 #pragma unroll
-      for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+      for (int m = 0; m < MP; ++m) acc[u][m] = 0.0f;
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         const unsigned wds[4] = {buf.w[u][c].x, buf.w[u][c].y, buf.w[u][c].z, buf.w[u][c].w};
@@ -270,33 +294,59 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_stream_kernel(const Vecm
           float part = 0.0f;
 #pragma unroll
           for (int i = 0; i < 8; ++i) part = __builtin_amdgcn_fdot2_f32_bf16(wp[i], xp[m][c][i], part, false);
-          acc[m] = fmaf(buf.sc[u][c], part, acc[m]);
+          acc[u][m] = fmaf(buf.sc[u][c], part, acc[u][m]);
         }
       }
+    }
 #pragma unroll
-      for (int m = 0; m < M; ++m) {
-        const float s = wave_total_dpp(acc[m]);
-        if (lane == 0) red[wave][g * U + u][m] = s;
+    for (int u = 0; u < U; ++u) {
+      float v;
+      if constexpr (MP == 4) {
+        const float k0 = bit0 ? acc[u][1] : acc[u][0], s0 = bit0 ? acc[u][0] : acc[u][1];
+        const float k1 = bit0 ? acc[u][3] : acc[u][2], s1 = bit0 ? acc[u][2] : acc[u][3];
+        const float b0 = dpp_add(k0, s0, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+        const float b1 = dpp_add(k1, s1, std::integral_constant<int, 0xB1>{});
+        const float k = bit1 ? b1 : b0, sd = bit1 ? b0 : b1;
+        v = dpp_add(k, sd, std::integral_constant<int, 0x4E>{});                 // quad_perm [2,3,0,1]
+      } else if constexpr (MP == 2) {
+        const float k = bit0 ? acc[u][1] : acc[u][0], sd = bit0 ? acc[u][0] : acc[u][1];
+        v = dpp_add(k, sd, std::integral_constant<int, 0xB1>{});
+        v = dpp_add(v, v, std::integral_constant<int, 0x112>{});                 // row_shr:2
+      } else {
+        v = dpp_add(acc[u][0], acc[u][0], std::integral_constant<int, 0x111>{}); // row_shr:1
+        v = dpp_add(v, v, std::integral_constant<int, 0x112>{});
       }
+      v = dpp_add(v, v, std::integral_constant<int, 0x114>{});                   // row_shr:4
+      v = dpp_add(v, v, std::integral_constant<int, 0x118>{});                   // row_shr:8
+      if (writer) red[wave][lrow][g * U + u][wm] = v;
     }
   };
 
-  StreamBuf<M, CH, U> a, b;
+  StreamBuf<CH> a, b;
   load(a, 0);
-#pragma unroll
-  for (int g = 0; g + 1 < G; g += 2) {
+  // (the loads inside the loop are unconditional, so every wait in it counts loads exactly: a load
+  // under a branch would make the compiler wait for everything in flight after the join)
+  int g = 0;
+  for (; g + 2 < G; g += 2) {                      // (uniform trip count)
     load(b, g + 1);
     compute(a, g);
-    if (g + 2 < G) load(a, g + 2);
+    load(a, g + 2);
     compute(b, g + 1);
   }
-  if (G % 2) compute(a, G - 1);
+  if (g + 1 < G) {
+    load(b, g + 1);
+    compute(a, g);
+    compute(b, g + 1);
+  } else {
+    compute(a, g);
+  }
   __syncthreads();
-  const int t = (int)threadIdx.x;
-  if (t < R * M) {
+  for (int t = (int)threadIdx.x; t < R * M; t += W * 64) {
     const int r = t / M, m = t % M;
     if (row0 + r <= last_row) {
-      const float s = ((red[0][r][m] + red[1][r][m]) + red[2][r][m]) + red[3][r][m];
+      float s = 0.0f;
+#pragma unroll
+      for (int w = 0; w < W; ++w) s += (red[w][0][r][m] + red[w][1][r][m]) + (red[w][2][r][m] + red[w][3][r][m]);
       store_as(p.out, (size_t)m * p.n + row0 + r, p.out_dtype, s);
     }
   }
@@ -509,7 +559,7 @@ static bool vecmat_aligned(const cppmega_mi355_vecmat_args_t& a) {
   return (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) && (((size_t)a.k * xelt) % 16 == 0);
 }
 static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) {
-  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 4096 == 0) && a.k <= 16384;
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 16 == 0) && a.k <= kStreamMaxK;
 }
 // the split-K MFMA kernel: bf16 activations, 2 <= M <= 32, K in eighths of whole scale blocks that fit the LDS slice
 static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
@@ -526,9 +576,7 @@ int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* byt
   return 0;
 }
 
-// Rows per workgroup of the streaming kernel: the candidate whose grid leaves the smallest idle
-// share in its last round over the device's compute units (ties: more workgroups).
-static int stream_rows(int n, int m) {
+static int device_cus() {
   static int cus = 0;
   if (cus == 0) {
     int dev = 0, v = 0;
@@ -536,9 +584,21 @@ static int stream_rows(int n, int m) {
         hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
     else cus = 256;
   }
+  return cus;
+}
+
+// Rows per workgroup of the streaming kernel.  Few rows: about one workgroup per compute unit.
+// Many rows: of 16, 28 and 14 the one whose grid leaves the smallest idle share in its last
+// round over the compute units (ties: the earlier candidate).
+static int stream_rows(int n, int m) {
+  const int cus = device_cus();
   if (const char* e = getenv("CPPMEGA_MI355_VECMAT_ROWS")) {
     const int v = atoi(e);
-    if (m > 1 && (v == 16 || v == 28 || v == 14)) return v;
+    if (v >= kStreamU && v <= kStreamMaxRows && v % kStreamU == 0) return v;
+  }
+  if (n < 16 * cus) {
+    const int r = (n / cus) & ~(kStreamU - 1);
+    return r < kStreamU ? kStreamU : r;
   }
   if (m == 1) return 16;
   const int cand[3] = {16, 28, 14};
@@ -551,6 +611,49 @@ static int stream_rows(int n, int m) {
     if (eff > best_eff + 1e-9) { best_eff = eff; best = r; }
   }
   return best;
+}
+
+// Wavefronts per row (W) and 1 KiB chunks per wavefront (CH) of the streaming kernel: the pair
+// with the fewest idle chunk slots, W * CH >= ceil(K / 1024); among equals the one named first
+// in the preference order below.
+static void stream_split(int k, int* w_out, int* ch_out) {
+  const int chunks = (k + kChunk - 1) / kChunk;
+  if (const char* e = getenv("CPPMEGA_MI355_VECMAT_WAVES")) {
+    const int w = atoi(e);
+    if (w >= 1 && w <= 8 && (chunks + w - 1) / w <= 4) { *w_out = w; *ch_out = (chunks + w - 1) / w; return; }
+  }
+  if (chunks < 4) { *w_out = chunks; *ch_out = 1; return; }
+  const int pref[5] = {4, 8, 7, 6, 5};
+  int best_w = 8, best_ch = 4, best_waste = 1 << 30;
+  for (int w : pref) {
+    const int ch = (chunks + w - 1) / w;
+    if (ch > 4) continue;
+    const int waste = w * ch - chunks;
+    if (waste < best_waste) { best_waste = waste; best_w = w; best_ch = ch; }
+  }
+  *w_out = best_w; *ch_out = best_ch;
+}
+
+template <int M, int W>
+static void stream_launch_ch(int ch, dim3 grid, hipStream_t stream, const VecmatParams& p) {
+  const dim3 block(W * 64);
+  if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, W>), grid, block, 0, stream, p);
+  else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, W>), grid, block, 0, stream, p);
+  else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, W>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, W>), grid, block, 0, stream, p);
+}
+template <int M>
+static void stream_launch(int w, int ch, dim3 grid, hipStream_t stream, const VecmatParams& p) {
+  switch (w) {
+    case 1: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 1>), grid, dim3(64), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 2>), grid, dim3(128), 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 3>), grid, dim3(192), 0, stream, p); break;
+    case 4: stream_launch_ch<M, 4>(ch, grid, stream, p); break;
+    case 5: stream_launch_ch<M, 5>(ch, grid, stream, p); break;
+    case 6: stream_launch_ch<M, 6>(ch, grid, stream, p); break;
+    case 7: stream_launch_ch<M, 7>(ch, grid, stream, p); break;
+    default: stream_launch_ch<M, 8>(ch, grid, stream, p); break;
+  }
 }
 
 int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) {
@@ -567,30 +670,15 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   const bool aligned = vecmat_aligned(a);
   const bool stream_ok = aligned && stream_shape(a);
   if (stream_ok) {
-    // rows per workgroup: 16, or 28 / 14 when that fills the last round of workgroups better
-    // (7168 rows are 448 x 16 = 1.75 rounds on 256 compute units, but exactly 256 x 28)
-    const int rows = stream_rows(a.n, a.m);
-    const dim3 grid((unsigned)((a.n + rows - 1) / rows)), block(kGemvWaves * 64);
-    const int ch = a.k / 4096;
-#define CM_STREAM_R(M, U, R)                                                                           \
-  do {                                                                                                 \
-    if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, U, R>), grid, block, 0, stream, p);      \
-    else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, U, R>), grid, block, 0, stream, p); \
-    else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, U, R>), grid, block, 0, stream, p); \
-    else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, U, R>), grid, block, 0, stream, p);              \
-  } while (0)
-#define CM_STREAM(M, U)                          \
-  do {                                           \
-    if (rows == 28) CM_STREAM_R(M, U, 28);       \
-    else if (rows == 14) CM_STREAM_R(M, U, 14);  \
-    else CM_STREAM_R(M, U, 16);                  \
-  } while (0)
-    if (a.m == 1) CM_STREAM_R(1, 4, 16);          // (measured: one activation row streams best in the smaller units)
-    else if (a.m == 2) CM_STREAM(2, 2);
-    else if (a.m == 3) CM_STREAM(3, 2);
-    else CM_STREAM(4, 2);
-#undef CM_STREAM_R
-#undef CM_STREAM
+    int w = 4, ch = 4;
+    stream_split(a.k, &w, &ch);
+    if (w < 4 && ch != 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "vecmat: no streaming split for k=%d", a.k);
+    p.rows_per_wg = stream_rows(a.n, a.m);
+    const dim3 grid((unsigned)((a.n + p.rows_per_wg - 1) / p.rows_per_wg));
+    if (a.m == 1) stream_launch<1>(w, ch, grid, stream, p);
+    else if (a.m == 2) stream_launch<2>(w, ch, grid, stream, p);
+    else if (a.m == 3) stream_launch<3>(w, ch, grid, stream, p);
+    else stream_launch<4>(w, ch, grid, stream, p);
   } else if (skinny_ok(a)) {
     const size_t need = (size_t)kSkinnySplits * a.m * a.n * sizeof(float);
     if (!a.workspace || a.workspace_bytes < need)

@@ -38,7 +38,11 @@ def _oracle_blocked(codes, scale, x):
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (1, 100, 4096), (1, 33, 2560), (1, 16, 32768), (1, 7, 100),
                                    (2, 64, 1024), (4, 257, 4096), (16, 130, 2048), (5, 48, 1000),
-                                   (17, 130, 2048), (32, 200, 4096), (24, 64, 16384), (33, 40, 2048)])
+                                   (17, 130, 2048), (32, 200, 4096), (24, 64, 16384), (33, 40, 2048),
+                                   # the streaming kernel's splits of K over wavefronts and chunks, whole and ragged
+                                   (1, 576, 7168), (1, 300, 1536), (3, 129, 7168), (4, 100, 18432), (2, 77, 11264),
+                                   (1, 40, 16), (4, 64, 1040), (1, 64, 29696), (2, 50, 5120), (3, 50, 6144),
+                                   (4, 31, 3072), (1, 31, 2048), (1, 5000, 1024), (4, 7000, 2048), (2, 4700, 512)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_block_scaled_bf16_activation(device, M, N, K, out_dtype):
     rng = np.random.default_rng(M * 1000003 + N * 101 + K)
