@@ -14,16 +14,10 @@
 //    the row sum is a wavefront reduction followed by a 4-way LDS combine.
 //  * 2 <= M <= 4, bf16 activations (gemv_stream_kernel): the same streaming shape with the
 //    M activation rows held in registers and v_dot2_f32_bf16 accumulation.
-//  * 5 <= M <= 32, bf16 activations (skinny_mfma_kernel): v_mfma_f32_16x16x32_bf16 with 16
-//    weight rows as the M side and the (padded) activation rows, in one or two groups of 16,
-//    as the N side.  A
-//    workgroup owns 16 weight rows; its 8 wavefronts own one eighth of K each and add
-//    their 16x16 partial tiles through LDS at the end, so nothing but the result is
-//    written to memory.  Weight fragments go from HBM straight into registers
-//    (16 bytes per lane and load: two MFMA k-steps, with the contraction order inside
-//    the 64-channel step permuted the same way for both operands) and are converted
-//    e4m3 -> bf16 with the 128-channel block scale applied in the conversion; the
-//    activations (L2-resident) are loaded per step.
+//  * 5 <= M <= 32, bf16 activations (skinny_mfma_kernel): split-K over 8 workgroup columns with
+//    v_mfma_scale_f32_16x16x128_f8f6f4.  The weights feed the matrix cores as the e4m3 bytes
+//    they are; the activations are split once per workgroup into two e4m3 planes in LDS.  The
+//    per-split partial sums go to a workspace and a second kernel adds them in split order.
 //  * anything else (odd K, misaligned rows): rowwise_kernel, one wavefront per
 //    output row, scalar byte loads.
 
@@ -42,7 +36,6 @@ struct VecmatParams {
   const float* scale_w;
   void* out;
   float* partial;          // [splits][M][N] fp32 (skinny kernel)
-  unsigned* counters;      // [row tiles]       (skinny kernel)
   int m, n, k;
   int x_dtype, out_dtype;
   int srow_shift;          // scale row index = n >> srow_shift
@@ -198,16 +191,6 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const VecmatParam
 //     before the arithmetic of the current one (two register buffers);
 //   * per row group: one joint DPP reduction of its U x M sums, then a fixed-order LDS combine.
 
-__device__ __forceinline__ float wave_total_dpp(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false));
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
-}
-
 constexpr int kStreamU = 2;              // rows per group (measured: 2 streams at least as fast as 4, in fewer registers)
 constexpr int kStreamMaxRows = 32;       // rows per workgroup, a multiple of kStreamU chosen by the host
 constexpr int kStreamMaxK = 8 * 4 * kChunk;
@@ -352,146 +335,191 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
   }
 }
 
-// 5 <= M <= 32 with bf16 activations, K a multiple of 1024: see the file header.  MT: groups of 16 activation rows.
+// 5 <= M <= 32 with bf16 activations, K a multiple of 1024: the split-K matrix-core kernel.
+//
+// The weights never leave e4m3: they are the B operand of v_mfma_scale_f32_16x16x128_f8f6f4
+// as they come from memory (32 contiguous bytes per lane, a whole 128-byte line per weight row
+// and 128-channel block).  The activations are the A operand.  A workgroup first writes its K
+// slice of them to LDS as two e4m3 planes hi + lo with x = hi 2^(e-127) + lo 2^(e-131), e one
+// exponent per activation row and 128-channel block, which the instruction applies as the
+// operand scales: hi carries the upper four significant bits of a bf16 value and lo the lower
+// four, so the pair is exact for every element within 2^-14 of the largest of its 128 and off
+// by less than 2^-22 of that largest one otherwise.  One block is two MFMAs (hi, lo) into a
+// zeroed tile whose lanes all belong to one weight row, so the block's fp32 weight scale (any
+// value, not only powers of two) is applied exactly as acc += scale * tile.
 constexpr int kSkinnySplits = 8;         // K is cut into eighths, one per workgroup column
-constexpr int kSkinnyWaves = 7;          // 448 row tiles x 8 splits = 256 workgroups x 7 wavefronts x 2 tiles at N = 7168
-constexpr int kSkinnyDepth = 8;          // 64-channel weight steps in flight per wavefront
+constexpr int kSkinnyWaves = 14;         // 448 row tiles x 8 splits = 256 workgroups x 14 wavefronts at N = 7168
+constexpr int kSkinnyDepth = 4;          // 128-channel weight blocks in flight per wavefront
 constexpr int kSkinnyMaxKw = 2048;       // channels per split the LDS activation slice can hold
-constexpr int kXPitchBytes = kSkinnyMaxKw * 2 + 16;   // row pitch of the slice: 16 rows fall on distinct banks
+constexpr int kXPitch = kSkinnyMaxKw + 16;            // bytes per row of an e4m3 plane: 16 rows fall on distinct banks
+constexpr int kXBlocks = kSkinnyMaxKw / 128;
 
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int skinny_lds_bytes(int mt) { return 2 * 16 * mt * kXPitch + 16 * mt * kXBlocks * 4; }
+
+// 32 bf16 channels of one lane (four 16-byte pieces) -> 32 e4m3 hi + 32 e4m3 lo bytes in channel
+// order.  The exponent is shared by the four lanes of a quad (one activation row's 128 channels).
+__device__ __forceinline__ int split_bf16_quad(const uint4 (&x)[4], i32x8& hi, i32x8& lo) {
+  u16x2 top = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned w[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2, w[d] & 0x7fff7fffu));
+  }
+  int amax_bits = max((int)top[0], (int)top[1]);             // bf16 bits of the largest magnitude
+  amax_bits = max(amax_bits, __builtin_amdgcn_update_dpp(0, amax_bits, 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+  amax_bits = max(amax_bits, __builtin_amdgcn_update_dpp(0, amax_bits, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+  const int e = max((amax_bits >> 7) - 7, 5);                 // |x| / 2^(e-127) < 256
+  const float unit = __uint_as_float((unsigned)e << 23);
+  const float unit_lo = __uint_as_float((unsigned)(e - 4) << 23);   // the remainder is below 2^-4 of the element
+  const i16x2 zero = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned w[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      const unsigned w0 = w[2 * d], w1 = w[2 * d + 1];
+      i16x2 h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(zero, __builtin_bit_cast(bf16x2, w0), unit, false);
+      h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(h, __builtin_bit_cast(bf16x2, w1), unit, true);
+      const unsigned hw = __builtin_bit_cast(unsigned, h);
+      const f32x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(hw, unit, false);
+      const f32x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(hw, unit, true);
+      i16x2 l = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(zero, __uint_as_float(w0 << 16) - d0[0],
+                                                         __uint_as_float(w0 & 0xffff0000u) - d0[1], unit_lo, false);
+      l = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(l, __uint_as_float(w1 << 16) - d1[0],
+                                                   __uint_as_float(w1 & 0xffff0000u) - d1[1], unit_lo, true);
+      hi[2 * j + d] = (int)hw;
+      lo[2 * j + d] = __builtin_bit_cast(int, l);
+    }
+  }
+  return e;
+}
+
+// MT: groups of 16 activation rows
 template <int MT>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const VecmatParams p) {
-  extern __shared__ __align__(16) unsigned char xs[];    // [16 MT][kXPitchBytes]: bf16 activations of this split
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* xh = smem;                                            // [16 MT][kXPitch] e4m3 hi
+  unsigned char* xl = smem + 16 * MT * kXPitch;                        // [16 MT][kXPitch] e4m3 lo
+  int* xe = reinterpret_cast<int*>(smem + 2 * 16 * MT * kXPitch);      // [16 MT][kXBlocks] exponents of the two planes
   const int lane = lane_id();
   const int wave = (int)(threadIdx.x >> 6);
   const int K = p.k;
   const int kw = K / kSkinnySplits;                      // channels of this split (multiple of 128)
   const int split = (int)blockIdx.y;
   const int k0 = split * kw;
-  const int steps = kw / 64;
-  // activation slice -> LDS (rows >= M are zero)
-  for (int i = (int)threadIdx.x; i < 16 * MT * (kw / 8); i += kSkinnyWaves * 64) {
-    const int m = i / (kw / 8), c = i % (kw / 8);
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (m < p.m) v = *reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k0 + 8 * c);
-    *reinterpret_cast<uint4*>(xs + m * kXPitchBytes + 16 * c) = v;
+  const int blocks = kw / 128;
+  // activation slice -> LDS: a quad of lanes per (row, block), 32 channels per lane (rows >= M are zero)
+  for (int t = (int)threadIdx.x; t < 16 * MT * blocks * 4; t += kSkinnyWaves * 64) {
+    const int q = t & 3, item = t >> 2;
+    const int m = item / blocks, b = item % blocks;
+    uint4 x[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) x[j] = make_uint4(0, 0, 0, 0);
+    if (m < p.m) {
+      const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k0 + 128 * b + 32 * q);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = src[j];
+    }
+    i32x8 hi, lo;
+    const int e = split_bf16_quad(x, hi, lo);
+    uint4* dh = reinterpret_cast<uint4*>(xh + m * kXPitch + 128 * b + 32 * q);
+    uint4* dl = reinterpret_cast<uint4*>(xl + m * kXPitch + 128 * b + 32 * q);
+    dh[0] = make_uint4((unsigned)hi[0], (unsigned)hi[1], (unsigned)hi[2], (unsigned)hi[3]);
+    dh[1] = make_uint4((unsigned)hi[4], (unsigned)hi[5], (unsigned)hi[6], (unsigned)hi[7]);
+    dl[0] = make_uint4((unsigned)lo[0], (unsigned)lo[1], (unsigned)lo[2], (unsigned)lo[3]);
+    dl[1] = make_uint4((unsigned)lo[4], (unsigned)lo[5], (unsigned)lo[6], (unsigned)lo[7]);
+    if (q == 0) xe[m * kXBlocks + b] = e | ((e - 4) << 8);          // byte 0: hi plane, byte 1: lo plane
   }
   __syncthreads();
 
-  const int r16 = lane & 15, kq = lane >> 4;
-  const unsigned char* xrow = xs + r16 * kXPitchBytes + 32 * kq;        // B fragments: activation r16, channels 16kq.. of a step
+  // lane (r16, g): B operand = weight row r16 of the tile, channels 32 g .. 32 g + 31 of a block;
+  // A operand = activation row r16 (+ 16 mt), the same channels.  The result tile has weight row
+  // r16 in every register of the lane: register i is activation row 4 g + i.
+  const int r16 = lane & 15, g = lane >> 4;
+  const unsigned char* ah = xh + r16 * kXPitch + 32 * g;
+  const unsigned char* al = xl + r16 * kXPitch + 32 * g;
+  const int* ae = xe + r16 * kXBlocks;
   const int tiles = (p.n + 15) / 16;
-  // this wavefront's tiles: first, first + 7, ...; their steps form one continuous stream so the
-  // weight prefetch never drains between tiles
+  // this wavefront's tiles: first, first + kSkinnyWaves, ...; their blocks form one continuous
+  // stream so the weight prefetch never drains between tiles
   const int first = (int)blockIdx.x * p.rows_per_wg + wave;
   const int tile_end = min(tiles, ((int)blockIdx.x + 1) * p.rows_per_wg);
   const int my_tiles = first < tile_end ? (tile_end - first + kSkinnyWaves - 1) / kSkinnyWaves : 0;
-  const int total = my_tiles * steps;
-  // prefetch cursor: next weight bytes / scale of this lane, advanced step by step
-  int pf_tile = first, pf_st = 0;
+  const int total = my_tiles * blocks;
+  // prefetch cursor: next weight bytes / scale of this lane, advanced block by block
+  int pf_tile = first, pf_b = 0;
   const unsigned char* pf_w = nullptr;
   const float* pf_s = nullptr;
   auto pf_seek = [&]() {                                 // (per tile) row of this lane in tile pf_tile
     const int n = min(pf_tile * 16 + r16, p.n - 1);
-    pf_w = p.w + (size_t)n * K + k0 + 16 * kq;
+    pf_w = p.w + (size_t)n * K + k0 + 32 * g;
     pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
   };
-  auto pf_next = [&](uint4& wdst, float& sdst, bool with_scale) {
-    wdst = *reinterpret_cast<const uint4*>(pf_w + 64 * pf_st);   // (plain load: the other half of the cache line follows next step)
-    if (with_scale) sdst = pf_s[(size_t)(pf_st >> 1) * p.scol_stride];
-    if (++pf_st == steps) {                              // (uniform)
-      pf_st = 0;
+  auto pf_next = [&](uint4& w0, uint4& w1, float& sc) {
+    w0 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b);
+    w1 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b + 16);
+    sc = pf_s[(size_t)pf_b * p.scol_stride];
+    if (++pf_b == blocks) {                              // (uniform)
+      pf_b = 0;
       pf_tile += kSkinnyWaves;
       if (pf_tile < tile_end) pf_seek();
     }
   };
-  uint4 wq[kSkinnyDepth];
-  float sq[kSkinnyDepth / 2];                            // one scale per 128 channels = two steps
+  uint4 wq0[kSkinnyDepth], wq1[kSkinnyDepth];
+  float sq[kSkinnyDepth];
   if (total > 0) {
     pf_seek();
 #pragma unroll
     for (int d = 0; d < kSkinnyDepth; ++d) {
-      if (d < total) pf_next(wq[d], sq[d >> 1], (d & 1) == 0);
-      else { wq[d] = make_uint4(0, 0, 0, 0); if ((d & 1) == 0) sq[d >> 1] = 1.0f; }
+      if (d < total) pf_next(wq0[d], wq1[d], sq[d]);
+      else { wq0[d] = make_uint4(0, 0, 0, 0); wq1[d] = wq0[d]; sq[d] = 0.0f; }
     }
   }
-  float sq_next[kSkinnyDepth / 2];
-#pragma unroll
-  for (int i = 0; i < kSkinnyDepth / 2; ++i) sq_next[i] = 1.0f;
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  int st = 0, tile = first;                              // position of flat step f0 + d, tracked incrementally
-  for (int f0 = 0; f0 < total; f0 += kSkinnyDepth) {     // steps is a multiple of the depth? not required: see the guards
+  int b = 0, tile = first;                               // position of flat block f0 + d, tracked incrementally
+  for (int f0 = 0; f0 < total; f0 += kSkinnyDepth) {
 #pragma unroll
     for (int d = 0; d < kSkinnyDepth; ++d) {
       const int f = f0 + d;
-      const uint4 wv = wq[d];
-      const float sc = sq[d >> 1];
-      float sc_next = sc;
-      if (f + kSkinnyDepth < total) pf_next(wq[d], sc_next, (d & 1) == 0);
-      if ((d & 1) == 0) sq_next[d >> 1] = sc_next;       // takes effect once the odd step of the pair is done
-      else sq[d >> 1] = sq_next[d >> 1];
+      const uint4 w0 = wq0[d], w1 = wq1[d];
+      const float sc = sq[d];
+      if (f + kSkinnyDepth < total) pf_next(wq0[d], wq1[d], sq[d]);
       if (f < total) {                                   // (uniform)
-        uint4 x0[MT], x1[MT];
+        const i32x8 bw = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          x0[mt] = *reinterpret_cast<const uint4*>(xrow + mt * 16 * kXPitchBytes + 128 * st);
-          x1[mt] = *reinterpret_cast<const uint4*>(xrow + mt * 16 * kXPitchBytes + 128 * st + 16);
-        }
-        bf16x8 a0, a1;
-        const bool pow2 = (__float_as_uint(sc) & 0x007fffffu) == 0u && sc > 0.0f && sc < INFINITY;
-        if (__ballot(!pow2) == 0ull) {                   // the conversion applies a power-of-two scale exactly
-          const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.x, sc, false));
-          const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.x, sc, true));
-          const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.y, sc, false));
-          const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.y, sc, true));
-          const unsigned o4 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.z, sc, false));
-          const unsigned o5 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.z, sc, true));
-          const unsigned o6 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.w, sc, false));
-          const unsigned o7 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wv.w, sc, true));
-          a0 = __builtin_bit_cast(bf16x8, make_uint4(o0, o1, o2, o3));
-          a1 = __builtin_bit_cast(bf16x8, make_uint4(o4, o5, o6, o7));
-        } else {                                         // general scale: fp32 multiply, round to bf16
-          const unsigned wd[4] = {wv.x, wv.y, wv.z, wv.w};
-          unsigned o[8];
+          const uint4 h0 = *reinterpret_cast<const uint4*>(ah + mt * 16 * kXPitch + 128 * b);
+          const uint4 h1 = *reinterpret_cast<const uint4*>(ah + mt * 16 * kXPitch + 128 * b + 16);
+          const uint4 l0 = *reinterpret_cast<const uint4*>(al + mt * 16 * kXPitch + 128 * b);
+          const uint4 l1 = *reinterpret_cast<const uint4*>(al + mt * 16 * kXPitch + 128 * b + 16);
+          const int e = ae[mt * 16 * kXBlocks + b];
+          const i32x8 ahi = {(int)h0.x, (int)h0.y, (int)h0.z, (int)h0.w, (int)h1.x, (int)h1.y, (int)h1.z, (int)h1.w};
+          const i32x8 alo = {(int)l0.x, (int)l0.y, (int)l0.z, (int)l0.w, (int)l1.x, (int)l1.y, (int)l1.z, (int)l1.w};
+          f32x4 t = {0.f, 0.f, 0.f, 0.f};
+          t = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ahi, bw, t, 0, 0, 0, e, 0, 0x7f7f7f7f);
+          t = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(alo, bw, t, 0, 0, 1, e, 0, 0x7f7f7f7f);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const f32x2 lo = e4m3x2_lo(wd[i]), hi = e4m3x2_hi(wd[i]);
-            typedef __attribute__((ext_vector_type(2))) __bf16 v2;
-            v2 r0, r1;
-            r0[0] = (__bf16)(lo[0] * sc); r0[1] = (__bf16)(lo[1] * sc);
-            r1[0] = (__bf16)(hi[0] * sc); r1[1] = (__bf16)(hi[1] * sc);
-            o[2 * i] = __builtin_bit_cast(unsigned, r0);
-            o[2 * i + 1] = __builtin_bit_cast(unsigned, r1);
-          }
-          a0 = __builtin_bit_cast(bf16x8, make_uint4(o[0], o[1], o[2], o[3]));
-          a1 = __builtin_bit_cast(bf16x8, make_uint4(o[4], o[5], o[6], o[7]));
+          for (int i = 0; i < 4; ++i) acc[mt][i] = fmaf(sc, t[i], acc[mt][i]);
         }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, __builtin_bit_cast(bf16x8, x0[mt]), acc[mt], 0, 0, 0);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, __builtin_bit_cast(bf16x8, x1[mt]), acc[mt], 0, 0, 0);
-        }
-        if (++st == steps) {                             // (uniform) tile finished: partial[split][m][row]
-          // lane (m = lane%16, g = lane/16) holds weight rows 4g + i of activation 16 mt + m
-          const int row0 = tile * 16;
+        if (++b == blocks) {                             // (uniform) tile finished: partial[split][m][row]
+          const int row = tile * 16 + r16;
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            const int m = 16 * mt + r16;
-            if (m < p.m) {
-              float* dst = p.partial + ((size_t)split * p.m + m) * p.n + row0 + 4 * kq;
-              if (row0 + 4 * kq + 3 < p.n && (p.n & 3) == 0) {
-                *reinterpret_cast<float4*>(dst) = make_float4(acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]);
-              } else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  if (row0 + 4 * kq + i < p.n) dst[i] = acc[mt][i];
-              }
+            for (int i = 0; i < 4; ++i) {
+              const int m = 16 * mt + 4 * g + i;
+              if (m < p.m && row < p.n) p.partial[((size_t)split * p.m + m) * p.n + row] = acc[mt][i];
             }
             acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
           }
-          st = 0;
+          b = 0;
           tile += kSkinnyWaves;
         }
       }
@@ -661,7 +689,7 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   if (rc) return rc;
   VecmatParams p;
   p.x = a.x; p.scale_x = a.scale_x; p.w = a.w; p.scale_w = a.scale_w; p.out = a.out;
-  p.partial = nullptr; p.counters = nullptr;
+  p.partial = nullptr;
   p.m = a.m; p.n = a.n; p.k = a.k; p.x_dtype = a.x_dtype; p.out_dtype = a.out_dtype;
   p.rows_per_wg = 0; p.k_splits = 1;
   rc = fill_scale_layout(a, p);
@@ -691,11 +719,11 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     p.rows_per_wg = per_wave * kSkinnyWaves;
     const dim3 grid((unsigned)((tiles + p.rows_per_wg - 1) / p.rows_per_wg), kSkinnySplits), block(kSkinnyWaves * 64);
     if (a.m <= 16) {
-      const int smem = 16 * kXPitchBytes;
+      const int smem = skinny_lds_bytes(1);
       CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
       hipLaunchKernelGGL(skinny_mfma_kernel<1>, grid, block, smem, stream, p);
     } else {
-      const int smem = 32 * kXPitchBytes;
+      const int smem = skinny_lds_bytes(2);
       CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
       hipLaunchKernelGGL(skinny_mfma_kernel<2>, grid, block, smem, stream, p);
     }
