@@ -413,6 +413,55 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   const int split = (int)blockIdx.y;
   const int k0 = split * kw;
   const int blocks = kw / 128;
+  // lane (r16, g): B operand = weight row r16 of the tile, channels 32 g .. 32 g + 31 of a block;
+  // A operand = activation row r16 (+ 16 mt), the same channels.  The result tile has weight row
+  // r16 in every register of the lane: register i is activation row 4 g + i.
+  const int r16 = lane & 15, g = lane >> 4;
+  const int perm_addr = 4 * (4 * r16 + g);               // source lane of this lane's weight bytes
+  const unsigned char* ah = xh + r16 * kXPitch + 16 * g;
+  const unsigned char* al = xl + r16 * kXPitch + 16 * g;
+  const int* ae = xe + r16 * kXBlocks;
+  const int tiles = (p.n + 15) / 16;
+  // this wavefront's tiles: first, first + kSkinnyWaves, ...; their blocks form one continuous
+  // stream so the weight prefetch never drains between tiles
+  const int first = (int)blockIdx.x * p.rows_per_wg + wave;
+  const int tile_end = min(tiles, ((int)blockIdx.x + 1) * p.rows_per_wg);
+  const int my_tiles = first < tile_end ? (tile_end - first + kSkinnyWaves - 1) / kSkinnyWaves : 0;
+  const int total = my_tiles * blocks;
+  // prefetch cursor: next weight bytes / scale of this lane, advanced block by block
+  int pf_tile = first, pf_b = 0;
+  const unsigned char* pf_w = nullptr;
+  const float* pf_s = nullptr;
+  auto pf_seek = [&]() {                                 // (per tile) row of this lane in tile pf_tile
+    const int n = min(pf_tile * 16 + r16, p.n - 1);
+    // (weights are fetched by lane 4 r + q = row r, bytes 16 q and 64 + 16 q of the block: four
+    // neighbouring lanes read 64 contiguous bytes, which the memory pipeline takes in one piece;
+    // a lane permutation then hands them to the matrix core's row-major lanes)
+    const int nl = min(pf_tile * 16 + (lane >> 2), p.n - 1);
+    pf_w = p.w + (size_t)nl * K + k0 + 16 * (lane & 3);
+    pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
+  };
+  auto pf_next = [&](uint4& w0, uint4& w1, float& sc) {
+    w0 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b);
+    w1 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b + 64);
+    sc = pf_s[(size_t)pf_b * p.scol_stride];
+    if (++pf_b == blocks) {                              // (uniform)
+      pf_b = 0;
+      pf_tile += kSkinnyWaves;
+      if (pf_tile < tile_end) pf_seek();
+    }
+  };
+  uint4 wq0[kSkinnyDepth], wq1[kSkinnyDepth];
+  float sq[kSkinnyDepth];
+  if (total > 0) {
+    pf_seek();
+#pragma unroll
+    for (int d = 0; d < kSkinnyDepth; ++d) {
+      if (d < total) pf_next(wq0[d], wq1[d], sq[d]);
+      else { wq0[d] = make_uint4(0, 0, 0, 0); wq1[d] = wq0[d]; sq[d] = 0.0f; }
+    }
+  }
+  // (the first weight blocks are already on their way: the conversion below runs in their shadow)
   // activation slice -> LDS: a quad of lanes per (row, block), 32 channels per lane (rows >= M are zero)
   for (int t = (int)threadIdx.x; t < 16 * MT * blocks * 4; t += kSkinnyWaves * 64) {
     const int q = t & 3, item = t >> 2;
@@ -437,49 +486,6 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   }
   __syncthreads();
 
-  // lane (r16, g): B operand = weight row r16 of the tile, channels 32 g .. 32 g + 31 of a block;
-  // A operand = activation row r16 (+ 16 mt), the same channels.  The result tile has weight row
-  // r16 in every register of the lane: register i is activation row 4 g + i.
-  const int r16 = lane & 15, g = lane >> 4;
-  const unsigned char* ah = xh + r16 * kXPitch + 32 * g;
-  const unsigned char* al = xl + r16 * kXPitch + 32 * g;
-  const int* ae = xe + r16 * kXBlocks;
-  const int tiles = (p.n + 15) / 16;
-  // this wavefront's tiles: first, first + kSkinnyWaves, ...; their blocks form one continuous
-  // stream so the weight prefetch never drains between tiles
-  const int first = (int)blockIdx.x * p.rows_per_wg + wave;
-  const int tile_end = min(tiles, ((int)blockIdx.x + 1) * p.rows_per_wg);
-  const int my_tiles = first < tile_end ? (tile_end - first + kSkinnyWaves - 1) / kSkinnyWaves : 0;
-  const int total = my_tiles * blocks;
-  // prefetch cursor: next weight bytes / scale of this lane, advanced block by block
-  int pf_tile = first, pf_b = 0;
-  const unsigned char* pf_w = nullptr;
-  const float* pf_s = nullptr;
-  auto pf_seek = [&]() {                                 // (per tile) row of this lane in tile pf_tile
-    const int n = min(pf_tile * 16 + r16, p.n - 1);
-    pf_w = p.w + (size_t)n * K + k0 + 32 * g;
-    pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
-  };
-  auto pf_next = [&](uint4& w0, uint4& w1, float& sc) {
-    w0 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b);
-    w1 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b + 16);
-    sc = pf_s[(size_t)pf_b * p.scol_stride];
-    if (++pf_b == blocks) {                              // (uniform)
-      pf_b = 0;
-      pf_tile += kSkinnyWaves;
-      if (pf_tile < tile_end) pf_seek();
-    }
-  };
-  uint4 wq0[kSkinnyDepth], wq1[kSkinnyDepth];
-  float sq[kSkinnyDepth];
-  if (total > 0) {
-    pf_seek();
-#pragma unroll
-    for (int d = 0; d < kSkinnyDepth; ++d) {
-      if (d < total) pf_next(wq0[d], wq1[d], sq[d]);
-      else { wq0[d] = make_uint4(0, 0, 0, 0); wq1[d] = wq0[d]; sq[d] = 0.0f; }
-    }
-  }
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -492,13 +498,16 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
       const float sc = sq[d];
       if (f + kSkinnyDepth < total) pf_next(wq0[d], wq1[d], sq[d]);
       if (f < total) {                                   // (uniform)
-        const i32x8 bw = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+        const i32x8 bw = {__builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.x), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.y),
+                          __builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.z), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.w),
+                          __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.x), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.y),
+                          __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.z), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.w)};
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const uint4 h0 = *reinterpret_cast<const uint4*>(ah + mt * 16 * kXPitch + 128 * b);
-          const uint4 h1 = *reinterpret_cast<const uint4*>(ah + mt * 16 * kXPitch + 128 * b + 16);
+          const uint4 h1 = *reinterpret_cast<const uint4*>(ah + mt * 16 * kXPitch + 128 * b + 64);
           const uint4 l0 = *reinterpret_cast<const uint4*>(al + mt * 16 * kXPitch + 128 * b);
-          const uint4 l1 = *reinterpret_cast<const uint4*>(al + mt * 16 * kXPitch + 128 * b + 16);
+          const uint4 l1 = *reinterpret_cast<const uint4*>(al + mt * 16 * kXPitch + 128 * b + 64);
           const int e = ae[mt * 16 * kXBlocks + b];
           const i32x8 ahi = {(int)h0.x, (int)h0.y, (int)h0.z, (int)h0.w, (int)h1.x, (int)h1.y, (int)h1.z, (int)h1.w};
           const i32x8 alo = {(int)l0.x, (int)l0.y, (int)l0.z, (int)l0.w, (int)l1.x, (int)l1.y, (int)l1.z, (int)l1.w};
