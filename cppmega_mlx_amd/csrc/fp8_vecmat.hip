@@ -201,7 +201,9 @@ struct StreamBuf {
   float sc[kStreamU][CH];
 };
 
-template <int M, int CH, int W>
+// XF8: the activations are e4m3 bytes with one fp32 scale (exactly representable as bf16 pairs;
+// the scale multiplies the finished sums)
+template <int M, int CH, int W, bool XF8 = false>
 __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams p) {
   constexpr int U = kStreamU;
   __shared__ float red[W][4][kStreamMaxRows][M];
@@ -223,13 +225,23 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       uint4 a = make_uint4(0, 0, 0, 0), b = a;
-      if (live) {
-        const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k);
-        a = src[0]; b = src[1];
-      }
-      const unsigned wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      if constexpr (XF8) {
+        if (live) a = *reinterpret_cast<const uint4*>((const unsigned char*)p.x + (size_t)m * K + k);
+        const unsigned wds[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
-      for (int i = 0; i < 8; ++i) xp[m][c][i] = __builtin_bit_cast(bf16x2, wds[i]);
+        for (int i = 0; i < 4; ++i) {
+          xp[m][c][2 * i] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, false);
+          xp[m][c][2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, true);
+        }
+      } else {
+        if (live) {
+          const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k);
+          a = src[0]; b = src[1];
+        }
+        const unsigned wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xp[m][c][i] = __builtin_bit_cast(bf16x2, wds[i]);
+      }
     }
   }
 
@@ -330,6 +342,7 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
       float s = 0.0f;
 #pragma unroll
       for (int w = 0; w < W; ++w) s += (red[w][0][r][m] + red[w][1][r][m]) + (red[w][2][r][m] + red[w][3][r][m]);
+      if constexpr (XF8) s *= p.scale_x[0];
       store_as(p.out, (size_t)m * p.n + row0 + r, p.out_dtype, s);
     }
   }
@@ -596,7 +609,8 @@ static bool vecmat_aligned(const cppmega_mi355_vecmat_args_t& a) {
   return (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) && (((size_t)a.k * xelt) % 16 == 0);
 }
 static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) {
-  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4 && (a.k % 16 == 0) && a.k <= kStreamMaxK;
+  const bool x_ok = (a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4) || (a.x_dtype == CPPMEGA_MI355_E4M3 && a.m == 1);
+  return x_ok && (a.k % 16 == 0) && a.k <= kStreamMaxK;
 }
 // the split-K MFMA kernel: bf16 activations, 2 <= M <= 32, K in eighths of whole scale blocks that fit the LDS slice
 static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
@@ -671,25 +685,25 @@ static void stream_split(int k, int* w_out, int* ch_out) {
   *w_out = best_w; *ch_out = best_ch;
 }
 
-template <int M, int W>
+template <int M, int W, bool XF8>
 static void stream_launch_ch(int ch, dim3 grid, hipStream_t stream, const VecmatParams& p) {
   const dim3 block(W * 64);
-  if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, W>), grid, block, 0, stream, p);
-  else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, W>), grid, block, 0, stream, p);
-  else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, W>), grid, block, 0, stream, p);
-  else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, W>), grid, block, 0, stream, p);
+  if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, W, XF8>), grid, block, 0, stream, p);
+  else if (ch == 2) hipLaunchKernelGGL((gemv_stream_kernel<M, 2, W, XF8>), grid, block, 0, stream, p);
+  else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, W, XF8>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, W, XF8>), grid, block, 0, stream, p);
 }
-template <int M>
+template <int M, bool XF8 = false>
 static void stream_launch(int w, int ch, dim3 grid, hipStream_t stream, const VecmatParams& p) {
   switch (w) {
-    case 1: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 1>), grid, dim3(64), 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 2>), grid, dim3(128), 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 3>), grid, dim3(192), 0, stream, p); break;
-    case 4: stream_launch_ch<M, 4>(ch, grid, stream, p); break;
-    case 5: stream_launch_ch<M, 5>(ch, grid, stream, p); break;
-    case 6: stream_launch_ch<M, 6>(ch, grid, stream, p); break;
-    case 7: stream_launch_ch<M, 7>(ch, grid, stream, p); break;
-    default: stream_launch_ch<M, 8>(ch, grid, stream, p); break;
+    case 1: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 1, XF8>), grid, dim3(64), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 2, XF8>), grid, dim3(128), 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 3, XF8>), grid, dim3(192), 0, stream, p); break;
+    case 4: stream_launch_ch<M, 4, XF8>(ch, grid, stream, p); break;
+    case 5: stream_launch_ch<M, 5, XF8>(ch, grid, stream, p); break;
+    case 6: stream_launch_ch<M, 6, XF8>(ch, grid, stream, p); break;
+    case 7: stream_launch_ch<M, 7, XF8>(ch, grid, stream, p); break;
+    default: stream_launch_ch<M, 8, XF8>(ch, grid, stream, p); break;
   }
 }
 
@@ -712,7 +726,8 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     if (w < 4 && ch != 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "vecmat: no streaming split for k=%d", a.k);
     p.rows_per_wg = stream_rows(a.n, a.m);
     const dim3 grid((unsigned)((a.n + p.rows_per_wg - 1) / p.rows_per_wg));
-    if (a.m == 1) stream_launch<1>(w, ch, grid, stream, p);
+    if (a.x_dtype == CPPMEGA_MI355_E4M3) stream_launch<1, true>(w, ch, grid, stream, p);
+    else if (a.m == 1) stream_launch<1>(w, ch, grid, stream, p);
     else if (a.m == 2) stream_launch<2>(w, ch, grid, stream, p);
     else if (a.m == 3) stream_launch<3>(w, ch, grid, stream, p);
     else stream_launch<4>(w, ch, grid, stream, p);

@@ -60,9 +60,9 @@ def test_block_scaled_bf16_activation(device, M, N, K, out_dtype):
     assert err <= (HALF_TOL if out_dtype != torch.float32 else f32_tol) * ref, (err, ref)
 
 
-def test_reference_shaped_fp8_activation_per_row_and_scalar_scales(device):
-    rng = np.random.default_rng(5)
-    N, K = 512, 4096
+@pytest.mark.parametrize("N,K", [(512, 4096), (130, 7168), (64, 16384), (77, 2048), (40, 1536), (300, 29696), (33, 100)])
+def test_reference_shaped_fp8_activation_per_row_and_scalar_scales(device, N, K):
+    rng = np.random.default_rng(5 + N + K)
     w = (rng.integers(0, 0x7F, (N, K)) | (rng.integers(0, 2, (N, K)) << 7)).astype(np.uint8)
     xc, xs = fp8.quantize_per_token(rng.standard_normal((1, K)).astype(np.float32))
     x = xc[0]
