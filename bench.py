@@ -212,6 +212,34 @@ def bench_vecmat(args, device, M: int):
     return res, (xs[0], ws[0], ss[0], outs[0])
 
 
+def bench_vecmat_fp8x(args, device):
+    """The reference's own vecmat form (fp8_vecmat_path_c.py:790-813): e4m3 activation vector with one
+    fp32 scale, e4m3 weights with one fp32 scale per output row, fp32 out."""
+    from cppmega_mlx_amd.nn._tilelang import fp8_vecmat_path_c as vm
+
+    N, K = 7168, 16384
+    gen = torch.Generator(device=device).manual_seed(177)
+    sets = []
+    for _ in range(3):
+        w = torch.randn((N, K), generator=gen, device=device).clamp(-3.5, 3.5).to(torch.float8_e4m3fn).view(torch.uint8)
+        x = torch.randn((K,), generator=gen, device=device).clamp(-3.5, 3.5).to(torch.float8_e4m3fn).view(torch.uint8)
+        sw = torch.rand((N,), generator=gen, device=device) + 0.5
+        sx = torch.full((1,), 0.37, device=device)
+        sets.append((x, w, sx, sw, torch.empty((N,), dtype=torch.float32, device=device)))
+    fns = [(lambda t=t: vm.fp8_scaled_vecmat_path_c_direct(t[0], t[1], scale_x=t[2], scale_w=t[3], out=t[4])) for t in sets]
+    steps = max(args.steps, 30)
+    secs, _ = timed_graph(fns, steps, args.warmup)
+    per = secs / steps
+    bytes_alg = N * K + N * 4 + K + N * 4
+    return {
+        "workload": "fp8_vecmat W e4m3[7168,16384] + fp32 scale per row, x e4m3[16384] + fp32 scale -> f32[7168]",
+        "us_per_launch": per * 1e6,
+        "algorithmic_bytes": bytes_alg,
+        "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+    }
+
+
 def cpu_baseline_vecmat(sample, rows: int = 1024):
     from oracle import vecmat as ov
 
@@ -420,6 +448,8 @@ def main() -> int:
             line["vecmat"][f"M{M}"] = res
             del sample
             torch.cuda.empty_cache()
+        line["vecmat"]["M1_fp8x"] = bench_vecmat_fp8x(args, device)
+        torch.cuda.empty_cache()
     if "topk" in parts:
         res, sample = bench_topk(args, device)
         if not args.no_cpu_baseline:
