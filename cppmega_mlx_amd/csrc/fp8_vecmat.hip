@@ -5,15 +5,12 @@
 // The weight is read from HBM exactly once; everything else is sized so that
 // the weight stream is the only traffic that matters.
 //
-//  * M == 1  (gemv_kernel): no matrix cores.  A workgroup of 4 wavefronts owns
-//    a few output rows; wavefront w owns the 1 KiB K-chunks c with c % 4 == w,
-//    so the four wavefronts read 4 KiB of one row contiguously.  The activation
-//    slice a wavefront needs is converted to fp32 once and stays in registers
-//    for all rows.  Per row a lane issues 16-byte weight loads, converts two
-//    bytes per instruction, accumulates in fp32 per 128-wide scale block, and
-//    the row sum is a wavefront reduction followed by a 4-way LDS combine.
-//  * 2 <= M <= 4, bf16 activations (gemv_stream_kernel): the same streaming shape with the
-//    M activation rows held in registers and v_dot2_f32_bf16 accumulation.
+//  * M <= 4 (M == 1 for e4m3 / fp32 activations), K a multiple of 16 up to 32768
+//    (gemv_stream_kernel): no matrix cores.  W wavefronts share a weight row and read it in
+//    contiguous 1 KiB pieces; the activation rows stay in registers; weights are converted two
+//    bytes per instruction and accumulated with v_dot2 (bf16 / fp16) or v_fma (fp32) in fp32 per
+//    128-wide scale block; a row pair's sums are reduced together across the wavefront.
+//  * M == 1, other K or misaligned rows (gemv_kernel): the same shape with bounds tests, fp32 math.
 //  * 5 <= M <= 32, bf16 activations (skinny_mfma_kernel): split-K over 8 workgroup columns with
 //    v_mfma_scale_f32_16x16x128_f8f6f4.  The weights feed the matrix cores as the e4m3 bytes
 //    they are; the activations are split once per workgroup into two e4m3 planes in LDS.  The
@@ -201,9 +198,13 @@ struct StreamBuf {
   float sc[kStreamU][CH];
 };
 
-// XF8: the activations are e4m3 bytes with one fp32 scale (exactly representable as bf16 pairs;
-// the scale multiplies the finished sums)
-template <int M, int CH, int W, bool XF8 = false>
+// XT, the activation type: bf16; e4m3 bytes with one fp32 scale (exactly representable as bf16
+// pairs; the scale multiplies the finished sums); fp16 (weights become fp16 pairs, exact, and meet
+// them in v_dot2_f32_f16); fp32 (weights become fp32, v_fma_f32).
+constexpr int kXBf16 = 0, kXF8 = 1, kXF16 = 2, kXF32 = 3;
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+template <int M, int CH, int W, int XT = kXBf16>
 __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams p) {
   constexpr int U = kStreamU;
   __shared__ float red[W][4][kStreamMaxRows][M];
@@ -216,7 +217,9 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
   const int last_row = p.n - 1;
 
   int koff[CH];
-  bf16x2 xp[M][CH][8];
+  constexpr bool XF8 = XT == kXF8;
+  constexpr int XW = XT == kXF32 ? 16 : 8;             // registers per activation row and chunk
+  unsigned xp[M][CH][XW];
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     const int k = (c * W + wave) * kChunk + lane * 16;
@@ -230,9 +233,18 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
         const unsigned wds[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          xp[m][c][2 * i] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, false);
-          xp[m][c][2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, true);
+          xp[m][c][2 * i] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, false));
+          xp[m][c][2 * i + 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, true));
         }
+      } else if constexpr (XT == kXF32) {
+        uint4 q[4] = {a, a, a, a};
+        if (live) {
+          const uint4* src = reinterpret_cast<const uint4*>((const float*)p.x + (size_t)m * K + k);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) q[i] = src[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { xp[m][c][4 * i] = q[i].x; xp[m][c][4 * i + 1] = q[i].y; xp[m][c][4 * i + 2] = q[i].z; xp[m][c][4 * i + 3] = q[i].w; }
       } else {
         if (live) {
           const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.x + (size_t)m * K + k);
@@ -240,7 +252,7 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
         }
         const unsigned wds[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xp[m][c][i] = __builtin_bit_cast(bf16x2, wds[i]);
+        for (int i = 0; i < 8; ++i) xp[m][c][i] = wds[i];
       }
     }
   }
@@ -278,18 +290,48 @@ __global__ __launch_bounds__(W * 64) void gemv_stream_kernel(const VecmatParams 
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         const unsigned wds[4] = {buf.w[u][c].x, buf.w[u][c].y, buf.w[u][c].z, buf.w[u][c].w};
-        bf16x2 wp[8];
+        if constexpr (XT == kXF32) {
+          f32x2 wf[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          wp[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, false);
-          wp[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, true);
-        }
+          for (int i = 0; i < 4; ++i) { wf[2 * i] = e4m3x2_lo(wds[i]); wf[2 * i + 1] = e4m3x2_hi(wds[i]); }
 #pragma unroll
-        for (int m = 0; m < M; ++m) {
-          float part = 0.0f;
+          for (int m = 0; m < M; ++m) {
+            float part = 0.0f;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) part = __builtin_amdgcn_fdot2_f32_bf16(wp[i], xp[m][c][i], part, false);
-          acc[u][m] = fmaf(buf.sc[u][c], part, acc[u][m]);
+            for (int i = 0; i < 8; ++i) {
+              part = fmaf(wf[i][0], __uint_as_float(xp[m][c][2 * i]), part);
+              part = fmaf(wf[i][1], __uint_as_float(xp[m][c][2 * i + 1]), part);
+            }
+            acc[u][m] = fmaf(buf.sc[u][c], part, acc[u][m]);
+          }
+        } else if constexpr (XT == kXF16) {
+          f16x2 wp[8];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            wp[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wds[i], 1.0f, false);
+            wp[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wds[i], 1.0f, true);
+          }
+#pragma unroll
+          for (int m = 0; m < M; ++m) {
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part = __builtin_amdgcn_fdot2(wp[i], __builtin_bit_cast(f16x2, xp[m][c][i]), part, false);
+            acc[u][m] = fmaf(buf.sc[u][c], part, acc[u][m]);
+          }
+        } else {
+          bf16x2 wp[8];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            wp[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, false);
+            wp[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wds[i], 1.0f, true);
+          }
+#pragma unroll
+          for (int m = 0; m < M; ++m) {
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part = __builtin_amdgcn_fdot2_f32_bf16(wp[i], __builtin_bit_cast(bf16x2, xp[m][c][i]), part, false);
+            acc[u][m] = fmaf(buf.sc[u][c], part, acc[u][m]);
+          }
         }
       }
     }
@@ -609,7 +651,8 @@ static bool vecmat_aligned(const cppmega_mi355_vecmat_args_t& a) {
   return (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) && (((size_t)a.k * xelt) % 16 == 0);
 }
 static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) {
-  const bool x_ok = (a.x_dtype == CPPMEGA_MI355_BF16 && a.m <= 4) || (a.x_dtype == CPPMEGA_MI355_E4M3 && a.m == 1);
+  const bool x_ok = ((a.x_dtype == CPPMEGA_MI355_BF16 || a.x_dtype == CPPMEGA_MI355_F16) && a.m <= 4) ||
+                    ((a.x_dtype == CPPMEGA_MI355_E4M3 || a.x_dtype == CPPMEGA_MI355_F32) && a.m == 1);
   return x_ok && (a.k % 16 == 0) && a.k <= kStreamMaxK;
 }
 // the split-K MFMA kernel: bf16 activations, 2 <= M <= 32, K in eighths of whole scale blocks that fit the LDS slice
@@ -685,7 +728,7 @@ static void stream_split(int k, int* w_out, int* ch_out) {
   *w_out = best_w; *ch_out = best_ch;
 }
 
-template <int M, int W, bool XF8>
+template <int M, int W, int XF8>
 static void stream_launch_ch(int ch, dim3 grid, hipStream_t stream, const VecmatParams& p) {
   const dim3 block(W * 64);
   if (ch == 1) hipLaunchKernelGGL((gemv_stream_kernel<M, 1, W, XF8>), grid, block, 0, stream, p);
@@ -693,7 +736,7 @@ static void stream_launch_ch(int ch, dim3 grid, hipStream_t stream, const Vecmat
   else if (ch == 3) hipLaunchKernelGGL((gemv_stream_kernel<M, 3, W, XF8>), grid, block, 0, stream, p);
   else hipLaunchKernelGGL((gemv_stream_kernel<M, 4, W, XF8>), grid, block, 0, stream, p);
 }
-template <int M, bool XF8 = false>
+template <int M, int XF8 = kXBf16>
 static void stream_launch(int w, int ch, dim3 grid, hipStream_t stream, const VecmatParams& p) {
   switch (w) {
     case 1: hipLaunchKernelGGL((gemv_stream_kernel<M, 1, 1, XF8>), grid, dim3(64), 0, stream, p); break;
@@ -726,7 +769,14 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     if (w < 4 && ch != 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "vecmat: no streaming split for k=%d", a.k);
     p.rows_per_wg = stream_rows(a.n, a.m);
     const dim3 grid((unsigned)((a.n + p.rows_per_wg - 1) / p.rows_per_wg));
-    if (a.x_dtype == CPPMEGA_MI355_E4M3) stream_launch<1, true>(w, ch, grid, stream, p);
+    if (a.x_dtype == CPPMEGA_MI355_E4M3) stream_launch<1, kXF8>(w, ch, grid, stream, p);
+    else if (a.x_dtype == CPPMEGA_MI355_F32) stream_launch<1, kXF32>(w, ch, grid, stream, p);
+    else if (a.x_dtype == CPPMEGA_MI355_F16) {
+      if (a.m == 1) stream_launch<1, kXF16>(w, ch, grid, stream, p);
+      else if (a.m == 2) stream_launch<2, kXF16>(w, ch, grid, stream, p);
+      else if (a.m == 3) stream_launch<3, kXF16>(w, ch, grid, stream, p);
+      else stream_launch<4, kXF16>(w, ch, grid, stream, p);
+    }
     else if (a.m == 1) stream_launch<1>(w, ch, grid, stream, p);
     else if (a.m == 2) stream_launch<2>(w, ch, grid, stream, p);
     else if (a.m == 3) stream_launch<3>(w, ch, grid, stream, p);

@@ -60,6 +60,22 @@ def test_block_scaled_bf16_activation(device, M, N, K, out_dtype):
     assert err <= (HALF_TOL if out_dtype != torch.float32 else f32_tol) * ref, (err, ref)
 
 
+@pytest.mark.parametrize("x_dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(1, 100, 4096), (1, 130, 7168), (1, 64, 16384), (1, 40, 1536), (1, 33, 29696),
+                                   (1, 7, 100), (2, 77, 2048), (3, 129, 7168), (4, 64, 16384), (5, 48, 1024)])
+def test_block_scaled_fp16_fp32_activation(device, M, N, K, x_dtype):
+    """fp16 / fp32 activations (exact inputs for the oracle: the values are rounded to the carrier first)."""
+    rng = np.random.default_rng(M * 7919 + N * 31 + K)
+    codes, scale = _weights(rng, N, K, pow2=False)
+    xt = to_dev(rng.standard_normal((M, K)).astype(np.float32), device).to(x_dtype)
+    xf = xt.float().cpu().numpy().astype(np.float64)
+    out = torch.zeros((M, N), dtype=torch.float32, device=device)
+    vm.fp8_scaled_vecmat_path_c(xt, to_dev(codes, device), scale_x=None, scale_w=to_dev(scale, device), out=out)
+    torch.cuda.synchronize()
+    err, ref = error_report(out.cpu().numpy(), _oracle_blocked(codes, scale, xf))
+    assert err <= F32_TOL * ref, (err, ref)
+
+
 @pytest.mark.parametrize("N,K", [(512, 4096), (130, 7168), (64, 16384), (77, 2048), (40, 1536), (300, 29696), (33, 100)])
 def test_reference_shaped_fp8_activation_per_row_and_scalar_scales(device, N, K):
     rng = np.random.default_rng(5 + N + K)
