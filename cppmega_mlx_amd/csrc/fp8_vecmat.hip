@@ -650,14 +650,20 @@ static bool vecmat_aligned(const cppmega_mi355_vecmat_args_t& a) {
   const size_t xelt = (size_t)dtype_size(a.x_dtype);
   return (a.k % 16 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) && (((size_t)a.k * xelt) % 16 == 0);
 }
-static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) {
-  const bool x_ok = ((a.x_dtype == CPPMEGA_MI355_BF16 || a.x_dtype == CPPMEGA_MI355_F16) && a.m <= 4) ||
-                    ((a.x_dtype == CPPMEGA_MI355_E4M3 || a.x_dtype == CPPMEGA_MI355_F32) && a.m == 1);
-  return x_ok && (a.k % 16 == 0) && a.k <= kStreamMaxK;
+// activation rows one launch of the streaming kernel takes (0: not a type it reads)
+static int stream_row_cap(int x_dtype) {
+  if (x_dtype == CPPMEGA_MI355_BF16 || x_dtype == CPPMEGA_MI355_F16) return 4;
+  if (x_dtype == CPPMEGA_MI355_E4M3 || x_dtype == CPPMEGA_MI355_F32) return 1;
+  return 0;
 }
-// the split-K MFMA kernel: bf16 activations, 2 <= M <= 32, K in eighths of whole scale blocks that fit the LDS slice
+static bool stream_k(const cppmega_mi355_vecmat_args_t& a) {
+  return stream_row_cap(a.x_dtype) > 0 && (a.k % 16 == 0) && a.k <= kStreamMaxK;
+}
+static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) { return stream_k(a) && a.m <= stream_row_cap(a.x_dtype); }
+// the split-K MFMA kernel: bf16 activations, M >= 5 (in passes of 32 rows), K in eighths of whole scale blocks that fit the LDS slice
+constexpr int kSkinnyMaxRows = 32;
 static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
-  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 2 && a.m <= 32 && !stream_shape(a) &&
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 &&
          (a.k % (kSkinnySplits * 128) == 0) && a.k / kSkinnySplits <= kSkinnyMaxKw;
 }
 static bool skinny_ok(const cppmega_mi355_vecmat_args_t& a) { return vecmat_aligned(a) && skinny_shape(a); }
@@ -666,7 +672,7 @@ int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* byt
   if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "vecmat: bytes is NULL");
   // pointers may be absent in a sizing call: decided from the shape alone (a misaligned call then
   // simply does not use the workspace)
-  *bytes = skinny_shape(a) ? (size_t)kSkinnySplits * a.m * a.n * sizeof(float) : 0;
+  *bytes = skinny_shape(a) ? (size_t)kSkinnySplits * (a.m < kSkinnyMaxRows ? a.m : kSkinnyMaxRows) * a.n * sizeof(float) : 0;
   return 0;
 }
 
@@ -762,27 +768,38 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   if (rc) return rc;
 
   const bool aligned = vecmat_aligned(a);
-  const bool stream_ok = aligned && stream_shape(a);
-  if (stream_ok) {
+  // one launch of the streaming kernel over `rows` activation rows starting at row m0
+  auto stream_pass = [&](VecmatParams q, int m0, int rows) -> int {
+    q.x = (const char*)a.x + (size_t)m0 * a.k * dtype_size(a.x_dtype);
+    q.out = (char*)a.out + (size_t)m0 * a.n * dtype_size(a.out_dtype);
+    q.m = rows;
     int w = 4, ch = 4;
     stream_split(a.k, &w, &ch);
     if (w < 4 && ch != 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "vecmat: no streaming split for k=%d", a.k);
-    p.rows_per_wg = stream_rows(a.n, a.m);
-    const dim3 grid((unsigned)((a.n + p.rows_per_wg - 1) / p.rows_per_wg));
-    if (a.x_dtype == CPPMEGA_MI355_E4M3) stream_launch<1, kXF8>(w, ch, grid, stream, p);
-    else if (a.x_dtype == CPPMEGA_MI355_F32) stream_launch<1, kXF32>(w, ch, grid, stream, p);
+    q.rows_per_wg = stream_rows(a.n, rows);
+    const dim3 grid((unsigned)((a.n + q.rows_per_wg - 1) / q.rows_per_wg));
+    if (a.x_dtype == CPPMEGA_MI355_E4M3) stream_launch<1, kXF8>(w, ch, grid, stream, q);
+    else if (a.x_dtype == CPPMEGA_MI355_F32) stream_launch<1, kXF32>(w, ch, grid, stream, q);
     else if (a.x_dtype == CPPMEGA_MI355_F16) {
-      if (a.m == 1) stream_launch<1, kXF16>(w, ch, grid, stream, p);
-      else if (a.m == 2) stream_launch<2, kXF16>(w, ch, grid, stream, p);
-      else if (a.m == 3) stream_launch<3, kXF16>(w, ch, grid, stream, p);
-      else stream_launch<4, kXF16>(w, ch, grid, stream, p);
+      if (rows == 1) stream_launch<1, kXF16>(w, ch, grid, stream, q);
+      else if (rows == 2) stream_launch<2, kXF16>(w, ch, grid, stream, q);
+      else if (rows == 3) stream_launch<3, kXF16>(w, ch, grid, stream, q);
+      else stream_launch<4, kXF16>(w, ch, grid, stream, q);
     }
-    else if (a.m == 1) stream_launch<1>(w, ch, grid, stream, p);
-    else if (a.m == 2) stream_launch<2>(w, ch, grid, stream, p);
-    else if (a.m == 3) stream_launch<3>(w, ch, grid, stream, p);
-    else stream_launch<4>(w, ch, grid, stream, p);
+    else if (rows == 1) stream_launch<1>(w, ch, grid, stream, q);
+    else if (rows == 2) stream_launch<2>(w, ch, grid, stream, q);
+    else if (rows == 3) stream_launch<3>(w, ch, grid, stream, q);
+    else stream_launch<4>(w, ch, grid, stream, q);
+    CM_HIP_CHECK(hipGetLastError());
+    return 0;
+  };
+  if (aligned && stream_shape(a)) {
+    rc = stream_pass(p, 0, a.m);
+    if (rc) return rc;
   } else if (skinny_ok(a)) {
-    const size_t need = (size_t)kSkinnySplits * a.m * a.n * sizeof(float);
+    // more than 32 activation rows: passes of 32 over the same workspace (stream order keeps them apart)
+    const int cap = a.m < kSkinnyMaxRows ? a.m : kSkinnyMaxRows;
+    const size_t need = (size_t)kSkinnySplits * cap * a.n * sizeof(float);
     if (!a.workspace || a.workspace_bytes < need)
       return fail(CPPMEGA_MI355_ERR_WORKSPACE, "vecmat: workspace of %zu bytes needed, %zu given", need, (size_t)a.workspace_bytes);
     p.partial = (float*)a.workspace;
@@ -792,17 +809,30 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     if (per_wave < 1) per_wave = 1;
     p.rows_per_wg = per_wave * kSkinnyWaves;
     const dim3 grid((unsigned)((tiles + p.rows_per_wg - 1) / p.rows_per_wg), kSkinnySplits), block(kSkinnyWaves * 64);
-    if (a.m <= 16) {
-      const int smem = skinny_lds_bytes(1);
-      CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-      hipLaunchKernelGGL(skinny_mfma_kernel<1>, grid, block, smem, stream, p);
-    } else {
-      const int smem = skinny_lds_bytes(2);
-      CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-      hipLaunchKernelGGL(skinny_mfma_kernel<2>, grid, block, smem, stream, p);
+    for (int m0 = 0; m0 < a.m; m0 += kSkinnyMaxRows) {
+      VecmatParams q = p;
+      q.m = a.m - m0 < kSkinnyMaxRows ? a.m - m0 : kSkinnyMaxRows;
+      q.x = (const char*)a.x + (size_t)m0 * a.k * dtype_size(a.x_dtype);
+      q.out = (char*)a.out + (size_t)m0 * a.n * dtype_size(a.out_dtype);
+      if (q.m <= 16) {
+        const int smem = skinny_lds_bytes(1);
+        CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        hipLaunchKernelGGL(skinny_mfma_kernel<1>, grid, block, smem, stream, q);
+      } else {
+        const int smem = skinny_lds_bytes(2);
+        CM_HIP_CHECK(hipFuncSetAttribute((const void*)skinny_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        hipLaunchKernelGGL(skinny_mfma_kernel<2>, grid, block, smem, stream, q);
+      }
+      CM_HIP_CHECK(hipGetLastError());
+      hipLaunchKernelGGL(skinny_reduce_kernel, dim3((unsigned)(((size_t)q.m * a.n + 255) / 256)), dim3(256), 0, stream, q);
     }
-    CM_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(skinny_reduce_kernel, dim3((unsigned)(((size_t)a.m * a.n + 255) / 256)), dim3(256), 0, stream, p);
+  } else if (aligned && stream_k(a)) {
+    // more rows than one launch takes: passes over the weights (which the last-level cache may keep)
+    const int cap = stream_row_cap(a.x_dtype);
+    for (int m0 = 0; m0 < a.m; m0 += cap) {
+      rc = stream_pass(p, m0, a.m - m0 < cap ? a.m - m0 : cap);
+      if (rc) return rc;
+    }
   } else if (a.m == 1 && aligned) {
     // rows per workgroup: keep at least ~3 workgroups per CU in the grid
     int rows = 16;

@@ -235,7 +235,7 @@ typedef struct cppmega_mi355_vecmat_args {
   int32_t out_dtype;
   int32_t reserved;
   void* out;
-  void* workspace;            /* split-K partials (5 <= M <= 32); may be NULL when
+  void* workspace;            /* split-K partials (M >= 5); may be NULL when
                                  *_workspace_bytes reports 0                   */
   size_t workspace_bytes;
 } cppmega_mi355_vecmat_args_t;
