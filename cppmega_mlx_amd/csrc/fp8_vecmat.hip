@@ -472,7 +472,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   // A operand = activation row r16 (+ 16 mt), the same channels.  The result tile has weight row
   // r16 in every register of the lane: register i is activation row 4 g + i.
   const int r16 = lane & 15, g = lane >> 4;
-  const int perm_addr = 4 * (4 * r16 + g);               // source lane of this lane's weight bytes
+  const int perm_addr = 4 * (8 * (r16 & 7) + g + (r16 >= 8 ? 4 : 0));   // source lane of this lane's weight bytes
   const unsigned char* ah = xh + r16 * kXPitch + 16 * g;
   const unsigned char* al = xl + r16 * kXPitch + 16 * g;
   const int* ae = xe + r16 * kXBlocks;
@@ -486,19 +486,23 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   // prefetch cursor: next weight bytes / scale of this lane, advanced block by block
   int pf_tile = first, pf_b = 0;
   const unsigned char* pf_w = nullptr;
+  const unsigned char* pf_w2 = nullptr;
   const float* pf_s = nullptr;
   auto pf_seek = [&]() {                                 // (per tile) row of this lane in tile pf_tile
     const int n = min(pf_tile * 16 + r16, p.n - 1);
-    // (weights are fetched by lane 4 r + q = row r, bytes 16 q and 64 + 16 q of the block: four
-    // neighbouring lanes read 64 contiguous bytes, which the memory pipeline takes in one piece;
-    // a lane permutation then hands them to the matrix core's row-major lanes)
-    const int nl = min(pf_tile * 16 + (lane >> 2), p.n - 1);
-    pf_w = p.w + (size_t)nl * K + k0 + 16 * (lane & 3);
+    // (weights are fetched by lane 8 r + q = bytes 16 q of the block's 128-byte line of row r
+    // (first load) and row 8 + r (second load): eight neighbouring lanes read a whole line, which
+    // the memory pipeline requests in one piece; two DPP moves and a lane permutation per
+    // register then hand the bytes to the matrix core's row-major lanes)
+    const int nl = min(pf_tile * 16 + (lane >> 3), p.n - 1);
+    const int nl2 = min(pf_tile * 16 + 8 + (lane >> 3), p.n - 1);
+    pf_w = p.w + (size_t)nl * K + k0 + 16 * (lane & 7);
+    pf_w2 = p.w + (size_t)nl2 * K + k0 + 16 * (lane & 7);
     pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
   };
   auto pf_next = [&](uint4& w0, uint4& w1, float& sc) {
     w0 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b);
-    w1 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b + 64);
+    w1 = *reinterpret_cast<const uint4*>(pf_w2 + 128 * pf_b);
     sc = pf_s[(size_t)pf_b * p.scol_stride];
     if (++pf_b == blocks) {                              // (uniform)
       pf_b = 0;
@@ -553,10 +557,17 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
       const float sc = sq[d];
       if (f + kSkinnyDepth < total) pf_next(wq0[d], wq1[d], sq[d]);
       if (f < total) {                                   // (uniform)
-        const i32x8 bw = {__builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.x), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.y),
-                          __builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.z), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w0.w),
-                          __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.x), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.y),
-                          __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.z), __builtin_amdgcn_ds_bpermute(perm_addr, (int)w1.w)};
+        // x0: pieces 0..3 of all 16 rows (the second load's, moved up four lanes, fill lanes 4..7 of
+        // every eight); x1: pieces 4..7 (the first load's, moved down four lanes, fill lanes 0..3)
+        const int a_[4] = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w}, b_[4] = {(int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+        i32x8 bw;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int x0 = __builtin_amdgcn_update_dpp(a_[d], b_[d], 0x114, 0xf, 0xa, false);   // row_shr:4 into banks 1, 3
+          const int x1 = __builtin_amdgcn_update_dpp(b_[d], a_[d], 0x104, 0xf, 0x5, false);   // row_shl:4 into banks 0, 2
+          bw[d] = __builtin_amdgcn_ds_bpermute(perm_addr, x0);
+          bw[4 + d] = __builtin_amdgcn_ds_bpermute(perm_addr, x1);
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const uint4 h0 = *reinterpret_cast<const uint4*>(ah + mt * 16 * kXPitch + 128 * b);
