@@ -236,7 +236,7 @@ def bench_vecmat_fp8x(args, device):
         "us_per_launch": per * 1e6,
         "algorithmic_bytes": bytes_alg,
         "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": None},
+                     "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic("fp8_vecmat_e4m3_activation")},
     }
 
 
