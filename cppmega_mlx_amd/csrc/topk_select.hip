@@ -142,9 +142,14 @@ __device__ BinHit find_bin(unsigned* smem, unsigned need, int mode) {
     int s; bool desc;
     if (mode == kAscending) { s = m; desc = false; }
     else if (mode == kDescending) { s = SEGS - 1 - m; desc = true; }
+    else if constexpr (SEGS == 1) {  // kSigned inside one segment: the lower half of the threads holds bins 2047..0
+      s = 0; desc = tid < THREADS / 2;
+    }
     else {  // kSigned: bins 2047..0 then 2048..4095 (SEGS is even here)
       if (m < SEGS / 2) { s = SEGS / 2 - 1 - m; desc = true; } else { s = m; desc = false; }
     }
+    // (one segment, signed walk: the wavefronts of the other half count as wholly before or after)
+    const bool split_walk = SEGS == 1 && mode == kSigned;
     // (the loop is unrolled and `s` selects among registers: keep it branch-free over s)
     unsigned my_sum = 0, my_incl = 0, my_wave_tot = 0, waves_before = 0;
     uint4 my_quad = make_uint4(0, 0, 0, 0);
@@ -155,7 +160,11 @@ __device__ BinHit find_bin(unsigned* smem, unsigned need, int mode) {
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
           if (w == wave) my_wave_tot = wtot[ss][w];
-          if (desc ? (w > wave) : (w < wave)) waves_before += wtot[ss][w];
+          if (split_walk) {
+            if (desc ? (w > wave && w < WAVES / 2) : (w < wave)) waves_before += wtot[ss][w];
+          } else if (desc ? (w > wave) : (w < wave)) {
+            waves_before += wtot[ss][w];
+          }
         }
       }
     }
@@ -617,7 +626,7 @@ int launch_kernel(K kernel, const TopkParams& p, int threads, size_t smem, hipSt
 static int wide_threads() {
   if (const char* e = getenv("CPPMEGA_MI355_TOPK_THREADS")) {
     const int v = atoi(e);
-    if (v == 256 || v == 512) return v;
+    if (v == 256 || v == 512 || v == 1024) return v;
   }
   return 512;
 }
@@ -627,7 +636,7 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
   const int T = p.width;
   const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
   const size_t out_words = sorted ? (size_t)p.sort_len * 2 : (size_t)p.k;
-  if (T <= 8192) {
+  if (T <= 32768) {
     auto tile_smem = [&](int E, int threads) {
       const size_t tile_words = (size_t)threads * (E + tile_pad(E));
       const size_t need = (size_t)kTileScratch + out_words;
@@ -646,8 +655,14 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
     if (T <= 4096) CM_TOPK_TILE(16, kTileThreads);
     // the widest rows: 512 threads x 16 columns (twice the wavefronts per row shorten every phase
     // of the row's pipeline, and the narrower runs need fewer registers)
-    if (wide_threads() == 512) CM_TOPK_TILE(16, 512);
-    CM_TOPK_TILE(32, kTileThreads);
+    if (T <= 8192) {
+      if (wide_threads() == 1024) CM_TOPK_TILE(8, 1024);
+      if (wide_threads() == 512) CM_TOPK_TILE(16, 512);
+      CM_TOPK_TILE(32, kTileThreads);
+    }
+    // up to 32768 columns: the same kernel on 1024 threads (half the time of the keyed-bin kernel below)
+    if (T <= 16384) CM_TOPK_TILE(16, 1024);
+    CM_TOPK_TILE(32, 1024);
 #undef CM_TOPK_TILE
   }
   const size_t smem = ((size_t)kWideScratch + out_words) * 4;

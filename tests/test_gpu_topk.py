@@ -38,7 +38,8 @@ def test_reference_known_answers(device, golden_dir):
 
 
 @pytest.mark.parametrize("rows,width,k", [(4, 64, 8), (3, 512, 64), (5, 2048, 256), (6, 8192, 2048), (2, 8192, 1),
-                                          (2, 8192, 8192), (3, 100, 7), (2, 1001, 500), (2, 4096, 2048), (1, 4, 4), (2, 20000, 3000), (1, 65536, 2048), (2, 9001, 100)])
+                                          (2, 8192, 8192), (3, 100, 7), (2, 1001, 500), (2, 4096, 2048), (1, 4, 4), (2, 20000, 3000), (1, 65536, 2048), (2, 9001, 100),
+                                          (3, 16384, 2048), (2, 12288, 4096), (2, 32768, 2048), (2, 20004, 5000), (1, 30001, 7), (2, 16384, 16384), (2, 16380, 1), (2, 8196, 8000)])
 @pytest.mark.parametrize("masked", [False, True])
 @pytest.mark.parametrize("order", ["index", "value"])
 def test_random_rows_bit_exact(device, rows, width, k, masked, order):
