@@ -62,6 +62,20 @@ def test_block_scaled_bf16_activation(device, M, N, K, out_dtype):
     assert err <= (HALF_TOL if out_dtype != torch.float32 else f32_tol) * ref, (err, ref)
 
 
+@pytest.mark.parametrize("M,N,K", [(2, 40, 2048), (4, 33, 8192), (3, 20, 14336), (4, 130, 12288), (2, 9, 10240),
+                                   (4, 300, 16384), (3, 64, 7168), (2, 5000, 4096), (4, 28, 6144)])
+def test_block_scaled_bf16_small_batch_arbitrary_scales(device, M, N, K):
+    """2 <= M <= 4 on the streaming kernel: arbitrary (not power-of-two) block scales, fp32 out."""
+    rng = np.random.default_rng(M * 104729 + N * 13 + K)
+    codes, scale = _weights(rng, N, K, pow2=False)
+    xt, xf = bf16_pair(rng.standard_normal((M, K)), device)
+    out = torch.zeros((M, N), dtype=torch.float32, device=device)
+    vm.fp8_scaled_vecmat_path_c(xt, to_dev(codes, device), scale_x=None, scale_w=to_dev(scale, device), out=out)
+    torch.cuda.synchronize()
+    err, ref = error_report(out.cpu().numpy(), _oracle_blocked(codes, scale, xf))
+    assert err <= F32_TOL * ref, (err, ref)
+
+
 @pytest.mark.parametrize("x_dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("M,N,K", [(1, 100, 4096), (1, 130, 7168), (1, 64, 16384), (1, 40, 1536), (1, 33, 29696),
                                    (1, 7, 100), (2, 77, 2048), (3, 129, 7168), (4, 64, 16384), (5, 48, 1024), (7, 64, 2048), (3, 50, 1040)])
