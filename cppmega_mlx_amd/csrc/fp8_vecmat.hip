@@ -501,8 +501,8 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
     pf_s = p.scale_w + (size_t)(n >> p.srow_shift) * p.srow_stride + (size_t)(k0 >> 7) * p.scol_stride;
   };
   auto pf_next = [&](uint4& w0, uint4& w1, float& sc) {
-    w0 = *reinterpret_cast<const uint4*>(pf_w + 128 * pf_b);
-    w1 = *reinterpret_cast<const uint4*>(pf_w2 + 128 * pf_b);
+    w0 = load_w16(pf_w + 128 * pf_b);
+    w1 = load_w16(pf_w2 + 128 * pf_b);
     sc = pf_s[(size_t)pf_b * p.scol_stride];
     if (++pf_b == blocks) {                              // (uniform)
       pf_b = 0;
