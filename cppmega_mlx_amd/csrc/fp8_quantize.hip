@@ -3,8 +3,9 @@
 //
 //   per token   scale[row] = max(amax(row) * (1/448), 1e-12); code = rne(clamp(x / scale, +-448))
 //   per tensor  the same with one amax over the whole tensor, the scale replicated per row
-//   mxfp8       per 32 channels: byte = clamp(127 + ceil(log2(amax / 448)), 1, 254) (127 for an
-//               all-zero block); code = rne(clamp(x / 2^(byte-127), +-448))
+//   mxfp8       per 32 channels: byte = clamp(127 + rint(log2(amax / 448)), 1, 254) (127 for an
+//               all-zero block; the exponent rounds to nearest, so values up to sqrt(2) above
+//               the scaled range saturate); code = rne(clamp(x / 2^(byte-127), +-448))
 //
 // One wavefront per row.  Besides codes and scales a call can ask for the round trip
 // dec(code) * scale in the input's dtype, which is what the float-carrier attention wrappers
@@ -79,12 +80,14 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const QuantParams p,
       float am = fabsf(v);
 #pragma unroll
       for (int off = 16; off >= 1; off >>= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
-      // smallest e with 448 * 2^e >= amax:  amax = m * 2^E, m in [1,2)  ->  e = E - 8 + (m > 1.75)
+      // e = rint(log2(amax / 448)):  amax = fr * 2^ex, fr in [0.5, 1), 448 = 0.875 * 2^9, so
+      // log2(amax / 448) = (ex - 9) + log2(fr / 0.875) with the last term in [-0.81, 0.19): it
+      // rounds to -1 iff fr / 0.875 < 2^-0.5, i.e. fr^2 < 0.875^2 / 2 (exact in double).
       int e = 0;
       if (am > 0.0f) {
         int ex;
-        const float fr = frexpf(am, &ex);       // am = fr * 2^ex, fr in [0.5, 1)
-        e = (ex - 1) - 8 + (fr > 0.875f ? 1 : 0);
+        const float fr = frexpf(am, &ex);
+        e = ex - 10 + ((double)fr * (double)fr > 0.3828125 ? 1 : 0);
       }
       const int byte = min(max(e + 127, 1), 254);
       const float inv = ldexpf(1.0f, 127 - byte), sc = ldexpf(1.0f, byte - 127);

@@ -7,9 +7,11 @@ trip of q and kv through e4m3 with one E8M0 scale per 32 channels, back to the c
 dtype, then the plain sparse attention; a width not divisible by 32 skips the round
 trip) and ``sparse_mla_blockscaled_apply`` :246-273.
 
-The packed form is four e4m3 bytes per uint32, byte 0 in the low bits; the scale byte
-choice of the reference's quantiser lives in MLX and is not restated anywhere in the
-reference, so this module uses byte = clamp(127 + ceil(log2(amax / 448)), 1, 254).
+The packed form is four e4m3 bytes per uint32, byte 0 in the low bits.  The scale byte of
+the reference's quantiser (``mx.quantize(mode="mxfp8")``) is
+byte = clamp(127 + rint(log2(amax / 448)), 1, 254) with codes saturating at +-448: the rule
+that reproduces the reference's seeded receipt
+``bench/tilelang_ports/sparse_mla_blockscaled.json`` (``parity.blockscaled_vs_bf16``).
 """
 
 from __future__ import annotations

@@ -254,7 +254,10 @@ int cppmega_mi355_fp8_vecmat(const cppmega_mi355_vecmat_args_t* args, size_t arg
  *   PER_TENSOR  _to_fp8_with_per_tensor_scale (sparse_mla_fp8.py:123-145): one amax over
  *               the tensor, the scale replicated per row
  *   MXFP8       _quantize_mxfp8 (sparse_mla_blockscaled.py:60-76): one E8M0 byte per 32
- *               channels, byte = clamp(127 + ceil(log2(amax/448)), 1, 254)
+ *               channels, byte = clamp(127 + rint(log2(amax/448)), 1, 254): the exponent
+ *               rounds to nearest (the rule that reproduces the reference's seeded receipt
+ *               bench/tilelang_ports/sparse_mla_blockscaled.json parity.blockscaled_vs_bf16),
+ *               codes saturate at +-448
  *   DEQUANT_*   _from_fp8_with_scale (sparse_mla_fp8.py:148-157) / _dequantize_mxfp8
  *               (sparse_mla_blockscaled.py:79-87): recovered = dec(codes) * scale
  * x is [rows, k] float32/float16/bfloat16, dense.  Any of codes / scale / recovered may be

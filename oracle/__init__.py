@@ -12,12 +12,18 @@ Pinning status (what fixes each function besides its own formula):
   ``float8_e4m3fn`` decoder for all 254 non-NaN bytes.
 * ``fp8.e8m0_decode``            -- pinned against the reference-held table
   rule (byte 0 or 255 -> 0, else 2**(b-127)).
-* ``fp8.e4m3_encode``, ``fp8.quantize_*`` -- producer side (input generation
-  only).  The reference delegates to MLX ``mx.to_fp8`` / ``mx.quantize`` whose
-  source is not in the tree: **parity unpinned** for the quantiser's rounding;
-  kernels consume prepared bytes + scales, so no kernel result depends on it.
-  Mathematically pinned here by round-trip exactness on the e4m3 grid and by
-  nearest-value brute force.
+* ``fp8.e4m3_encode``, ``fp8.quantize_*`` -- producer side.  The reference
+  delegates to MLX ``mx.to_fp8`` / ``mx.quantize`` whose source is not in the
+  tree; ``quantize_per_tensor`` and ``quantize_mxfp8`` are pinned by the two
+  seeded receipts the reference holds (bench/tilelang_ports/sparse_mla_fp8.json
+  ``parity.fp8_vs_bf16`` and sparse_mla_blockscaled.json
+  ``parity.blockscaled_vs_bf16``, regenerated in
+  tests/test_oracle_reference_receipts.py), ``quantize_per_token`` by the
+  reference's own producer kernel text, ``e4m3_encode`` by round-trip exactness
+  on the e4m3 grid and nearest-value brute force.  Left open by the receipts:
+  the rounding of an MXFP8 exponent exactly half-way between two integers
+  (cannot occur for a float amax) and ties of ``mx.to_fp8`` on exact code
+  midpoints (assumed to-even, as every IEEE-style converter).
 * ``topk.topk_selector_oracle``  -- pinned by the reference tests' exact-order
   known answers, sentinel cases and an O(T^2) brute-force ranker.
 * ``sparse_mla.sparse_mla_oracle`` -- pinned against a per-token loop

@@ -101,8 +101,11 @@ def quantize_per_token(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
 def quantize_per_tensor(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
     """One amax scale for the whole tensor, replicated per row: the float-carrier producer
     cppmega_mlx/nn/_tilelang/sparse_mla_fp8.py:123-145 (scale = max(amax/448, 1e-12), float32
-    arithmetic).  The rounding of ``mx.to_fp8`` is not in the tree (parity unpinned); this uses
-    round-to-nearest-even with saturation like the per-token producer kernel."""
+    arithmetic), codes round-to-nearest-even with saturation like the per-token producer kernel.
+    ``mx.to_fp8`` is not in the tree; pinned by the reference's seeded receipt
+    bench/tilelang_ports/sparse_mla_fp8.json ``parity.fp8_vs_bf16.max_abs_err`` =
+    0.0030034519731998444 (scripts/bench_tilelang_sparse_mla_fp8.py:105-125,443-444), which this
+    reproduces to 1.4e-8 (float32 matmul-order noise of the reference's run)."""
     x = np.asarray(x, dtype=np.float32)
     amax = np.float32(np.max(np.abs(x))) if x.size else np.float32(0)
     scale = np.maximum(amax * np.float32(1.0 / 448.0), np.float32(1e-12)).astype(np.float32)
@@ -149,12 +152,18 @@ def quantize_block(x: np.ndarray, block: int = 128, pow2: bool = True) -> tuple[
 
 
 def quantize_mxfp8(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
-    """E8M0-per-32 quantiser used to build block-scaled (MXFP8) test inputs.
+    """E8M0-per-32 quantiser: ``mx.quantize(mode="mxfp8")`` as the reference calls it
+    (cppmega_mlx/nn/_tilelang/sparse_mla_blockscaled.py:75).
 
-    scale byte = 127 + ceil(log2(amax/448)) clamped to [1, 254]; codes =
-    encode(x / 2**(byte-127)).  The reference calls ``mx.quantize(mode="mxfp8")``
-    (cppmega_mlx/nn/_tilelang/sparse_mla_blockscaled.py:75), whose scale choice
-    is not in the tree: parity unpinned, inputs only.
+    scale byte = 127 + rint(log2(amax/448)) clamped to [1, 254] (the exponent is rounded to
+    the NEAREST integer, so up to sqrt(2) of a block's range saturates at +-448); codes =
+    rne(clamp(x / 2**(byte-127), +-448)).  MLX's source is not in the tree; the rule is pinned
+    by the seeded receipt the reference holds, bench/tilelang_ports/sparse_mla_blockscaled.json
+    ``parity.blockscaled_vs_bf16.max_abs_err`` = 0.011328823864459991 (written by
+    scripts/bench_tilelang_sparse_mla_fp8.py:105-125,443-445): round reproduces it to 4e-9,
+    ceil gives 2.16e-3, floor 1.77e-2, the OCP floor(log2 amax) - 8 rule 2.17e-3.  Left open by
+    the receipt: which way an exponent exactly half-way between two integers rounds
+    (amax = 448 * 2**(n + 0.5) is not a float, so the case cannot occur).
     """
     x = np.asarray(x, dtype=np.float32)
     k = x.shape[-1]
@@ -163,10 +172,10 @@ def quantize_mxfp8(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
     xb = x.reshape(x.shape[:-1] + (k // 32, 32)).astype(np.float64)
     amax = np.max(np.abs(xb), axis=-1)
     with np.errstate(divide="ignore"):
-        expo = np.where(amax > 0, np.ceil(np.log2(np.where(amax > 0, amax / E4M3_MAX, 1.0))), 0.0)
+        expo = np.where(amax > 0, np.rint(np.log2(np.where(amax > 0, amax / E4M3_MAX, 1.0))), 0.0)
     byte = np.clip(expo + 127, 1, 254).astype(np.uint8)
     scale = np.exp2(byte.astype(np.float64) - 127)
-    codes = e4m3_encode(xb / scale[..., None]).reshape(x.shape)
+    codes = e4m3_encode(np.clip(xb / scale[..., None], -E4M3_MAX, E4M3_MAX)).reshape(x.shape)
     return codes, byte
 
 

@@ -55,8 +55,11 @@ def test_mxfp8_matches_oracle(device, carrier):
     rng = np.random.default_rng(6)
     rows, k = 21, 160
     x = _values(rng, rows, k)
-    x[5, :32] = 448.0 * 2.0 ** -3                        # amax exactly on a power-of-two boundary
+    x[5, :32] = 448.0 * 2.0 ** -3                        # amax exactly 448 * 2^e
     x[5, 32:64] = np.nextafter(np.float32(448.0 * 2.0 ** -3), np.float32(1e9))
+    # either side of the exponent's rounding point amax = 448 * 2^(e + 1/2)
+    half = np.float32(448.0 * 2.0 ** -2.5)
+    x[6, :32] = np.nextafter(half, np.float32(0)); x[6, 32:64] = half; x[6, 64:96] = np.nextafter(half, np.float32(1e9))
     xt = to_dev(x, device).to(carrier)
     xf = xt.float().cpu().numpy()
     want_codes, want_bytes = fp8.quantize_mxfp8(xf)
@@ -107,3 +110,23 @@ def test_float_carrier_attention_wrappers(device):
     np.testing.assert_array_equal(scale.cpu().numpy(), want_scale)
     rec = ff8._from_fp8_with_scale(codes, scale, dtype=torch.float32)
     np.testing.assert_array_equal(rec.cpu().numpy(), fp8.roundtrip_per_tensor(qf))
+
+
+def test_reference_parity_receipts_on_the_gpu(device):
+    """The reference's two seeded receipts (scripts/bench_tilelang_sparse_mla_fp8.py:105-125, 443-445;
+    bench/tilelang_ports/sparse_mla_fp8.json and sparse_mla_blockscaled.json, ``parity``) through the
+    float-carrier entry points: max|quantised - plain| on float32 carriers."""
+    from cppmega_mlx_amd.nn.sparse_mla import sparse_mla_attention_reference
+    from tests.test_oracle_reference_receipts import BLOCKSCALED_VS_PLAIN, FP8_VS_PLAIN, receipt_inputs
+
+    q, kv, idx = receipt_inputs()
+    qt, kt, it = to_dev(q, device), to_dev(kv, device), to_dev(idx, device)
+    plain = sparse_mla_attention_reference(qt, kt, it, d_v=32)
+    fp8_out = ff8.sparse_mla_fp8_apply(qt, kt, it, d_v=32)
+    bs_out = fbs.sparse_mla_blockscaled_apply(qt, kt, it, d_v=32)
+    fp8_ref = ff8.sparse_mla_fp8_reference(qt, kt, it, d_v=32)
+    bs_ref = fbs.sparse_mla_blockscaled_reference(qt, kt, it, d_v=32)
+    torch.cuda.synchronize()
+    assert plain.dtype == torch.float32
+    for got, want in ((fp8_out, FP8_VS_PLAIN), (fp8_ref, FP8_VS_PLAIN), (bs_out, BLOCKSCALED_VS_PLAIN), (bs_ref, BLOCKSCALED_VS_PLAIN)):
+        assert abs(float((got - plain).abs().max()) - want) <= 1e-6

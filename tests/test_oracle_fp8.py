@@ -111,13 +111,15 @@ def test_producer_quantisers_closed_forms():
     r = fp8.roundtrip_per_tensor(y)
     np.testing.assert_array_equal(fp8.roundtrip_per_tensor(r), r)
     assert np.abs(r - y).max() <= np.abs(y).max() / 448.0 * 16.0      # half an ulp of the top binade (ulp 32 at 448)
-    # MXFP8: 448 * 2^e is the largest amax a block with exponent e holds
-    z = np.zeros((1, 96), dtype=np.float32)
+    # MXFP8: the block exponent is log2(amax / 448) rounded to nearest; what exceeds 448 * 2^e saturates
+    z = np.zeros((1, 128), dtype=np.float32)
     z[0, 0] = 448.0
     z[0, 32] = 448.0 * 2.0 ** -5
     z[0, 64] = np.nextafter(np.float32(448.0), np.float32(1e9))
+    z[0, 96] = 448.0 * 1.5                                            # log2(1.5) = 0.585 -> exponent 1
     mcodes, mbytes = fp8.quantize_mxfp8(z)
-    assert list(mbytes[0]) == [127, 122, 128]
-    assert mcodes[0, 0] == 0x7E and mcodes[0, 32] == 0x7E and mcodes[0, 64] == 0x76   # 448.00003/2 = 224 -> 0x76
+    assert list(mbytes[0]) == [127, 122, 127, 128]
+    assert mcodes[0, 0] == 0x7E and mcodes[0, 32] == 0x7E and mcodes[0, 64] == 0x7E   # 448.00003 saturates
+    assert mcodes[0, 96] == 0x7A                                      # 672 / 2 = 336 -> rne to 320 (1.25 * 2^8)
     rm = fp8.roundtrip_mxfp8(y)
     np.testing.assert_array_equal(fp8.roundtrip_mxfp8(rm), rm)
