@@ -58,4 +58,10 @@ void sparse_mla_latent_plan(MlaParams& p);
 int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream);   // includes its combine step
 size_t sparse_mla_latent_workspace_bytes(const MlaParams& p);
 
+// producer/consumer kernel for FP8 latent caches (sparse_mla_latent_pc.hip): 64 heads per workgroup
+bool sparse_mla_latent_pc_supported(const MlaParams& p);
+void sparse_mla_latent_pc_plan(MlaParams& p);
+int sparse_mla_latent_pc_launch(const MlaParams& p, hipStream_t stream);   // includes its combine step
+size_t sparse_mla_latent_pc_workspace_bytes(const MlaParams& p);
+
 }  // namespace cm

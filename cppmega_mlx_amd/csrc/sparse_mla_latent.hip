@@ -923,6 +923,16 @@ int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream) {
   return 0;
 }
 
+// the combine step alone (partials in the layout of hg 32-head groups per workgroup)
+int sparse_mla_latent_combine_launch(const MlaParams& p, int hg, hipStream_t stream) {
+  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const dim3 cgrid((unsigned)((size_t)p.B * p.S * p.G * chunks), (unsigned)(4 * hg));
+  if (hg == 4) hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
+  CM_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
 size_t sparse_mla_latent_workspace_bytes(const MlaParams& p) {
   if (p.num_splits <= 1) return 0;
   const int hg = p.heads_per_wg / 32;

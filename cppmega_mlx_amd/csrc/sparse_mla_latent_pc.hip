@@ -1,0 +1,952 @@
+// Sparse MLA forward over an FP8 latent KV cache on the matrix cores (gfx950), with the
+// wavefronts of a workgroup split into score producers and value consumers.
+//
+// Shapes served: bf16 queries of 576 = 512 latent + 64 rope channels, d_v = 512, keys as e4m3
+// latent [512] with fp32 scales (per 128 / 256 / 512 channels, per row, or none) plus a bf16
+// rope tail [64]; more than 32 heads per KV group.
+//
+// Workgroup = (query, KV group, chunk of 64 heads, key split), 8 wavefronts, key tiles of 32
+// rows in a ring of five LDS slots filled by the load unit (global_load_lds) three tiles ahead.
+// Two wavefronts share a SIMD: one producer and one consumer, so the matrix passes of one run
+// under the vector instructions of the other.
+//
+//   producers (wavefronts 0..3): producer p owns heads 16p..16p+15 of the chunk.
+//     S^T = K.Q^T on v_mfma_scale_f32_16x16x128_f8f6f4: the key bytes are the A operand as they
+//     lie in the tile (no conversion instructions); the power-of-two part of a key's block scale
+//     is the operand exponent, the mantissa part multiplies the block's fp32 partial sum.  Q^T is
+//     split once per workgroup into two e4m3 planes hi + lo (hi + lo = the bf16 value, one
+//     exponent per head and 128 channels), kept in registers.  The rope tail is a bf16 product.
+//     Softmax in base 2 with a lazily moved private running maximum per head; P goes to LDS as
+//     bf16 in the B-operand layout of the value product, once per scale block with V's block
+//     scale folded in.
+//   consumers (wavefronts 4..7): consumer c owns value channels 128c..128c+127 (= scale block c
+//     when there are four) for all 64 heads: O^T += V^T.P^T on v_mfma_f32_32x32x16_bf16, V^T
+//     fragments by transposing LDS reads of the raw tile, converted unscaled (exactly).  They
+//     also issue the row loads.
+//   pipeline  iteration t: barrier; producers: scores and P of tile t+1; consumers: issue tile
+//             t+4, value product of tile t.  One barrier per tile.
+//
+// Key splits write their accumulators (rounded to bf16) to the workspace as the lanes hold them
+// plus (max, sum) per head; sparse_mla_latent_combine_kernel (HG = 2 layout) merges them.
+
+#include <type_traits>
+
+#include "sparse_mla_common.h"
+#include "mfma_util.h"
+
+namespace cm {
+
+int sparse_mla_latent_combine_launch(const MlaParams& p, int hg, hipStream_t stream);
+
+#if defined(CM_PC_TIMING) || defined(CM_PC_DEBUG)
+#ifndef CM_PC_TICK_WG
+#define CM_PC_TICK_WG 0
+#endif
+__device__ unsigned long long g_pc_ticks[64];
+#endif
+#ifdef CM_PC_TIMING
+#define TICK(i) do { if (blockIdx.x == CM_PC_TICK_WG && lane == 0) g_pc_ticks[i] = __builtin_amdgcn_s_memtime(); } while (0)
+#define TACC(i, t0) do { if (blockIdx.x == CM_PC_TICK_WG && lane == 0) g_pc_ticks[i] += __builtin_amdgcn_s_memtime() - (t0); } while (0)
+#define TNOW() __builtin_amdgcn_s_memtime()
+#else
+#define TICK(i)
+#define TACC(i, t0)
+#define TNOW() 0ull
+#endif
+#ifdef CM_PC_TIMING_LIGHT
+#undef TACC
+#undef TNOW
+#define TACC(i, t0)
+#define TNOW() 0ull
+#endif
+
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kLat = 512;
+constexpr int kRope = 64;
+constexpr int kDqk = kLat + kRope;
+constexpr int kTK = 32;                         // keys per tile
+#ifndef CM_RING
+#define CM_RING 5
+#endif
+#ifndef CM_MAXKEYS
+#define CM_MAXKEYS 2048
+#endif
+constexpr int kRing = CM_RING;                  // tile slots
+constexpr int kAhead = kRing - 1;               // tiles issued ahead of the value product
+// A tile slot holds the rows in matrix-operand order.  Latent: for sub-tile sj (16 keys) and
+// 128-channel block blk, two planes j of 64 lanes x 16 bytes: lane (key n = lane % 16, kg = lane / 16)
+// of plane j holds channels 128 blk + 32 kg + 16 j .. + 15 of key 16 sj + n.  A plane is what one
+// load instruction writes (the load unit stores lane after lane) and what one 16-byte-per-lane
+// LDS read of a K operand fetches, contiguously.  Plane 1 starts 128 bytes after the end of plane
+// 0, so that the two neighbouring chunks a V^T read takes from eight rows fall on different banks.
+// Rope: for sub-tile sj and 32-channel step s one plane: lane (n, kq) holds channels 32 s + 8 kq .. + 7.
+constexpr int kPlane = 1024 + 128;              // bytes from plane 0 to plane 1 of a pair
+constexpr int kPair = 2 * kPlane;               // one (sub-tile, block)
+constexpr int kLatBytes = 8 * kPair;            // 18432
+constexpr int kRopeBytes = 4 * 1024;            // [sj][s] planes
+constexpr int kScaleBytes = kTK * 4 * 4;        // 512: up to four fp32 scales per row, [row][block]
+constexpr int kSlotBytes = kLatBytes + kRopeBytes + kScaleBytes;   // 23040
+constexpr int kRingBytes = kRing * kSlotBytes;  // 104960
+constexpr int kMaxKeys = CM_MAXKEYS;            // keys of one split (their rows are staged in LDS)
+constexpr int kKeyInts = kMaxKeys + kTK;
+constexpr int kHeadsWg = 64;
+constexpr int kXPitch = 132;                    // floats per head row of the output transpose (128 + 4)
+constexpr int kPartFloats = 4 * 16 * 64 * 4;    // partial values of one 32-head group: [4 consumers][16 rows][64 lanes][4]
+constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
+
+constexpr int kPVarBytes = 2 * 2 * 1024;        // one scale variant of P: [k-step][head block][64 lanes x 16 B]
+constexpr int kPBytes = 4 * kPVarBytes;         // one parity
+constexpr int kPOff = kRingBytes;
+constexpr int kFacOff = kPOff + 2 * kPBytes;        // [parity][4 producers][16 heads] fp32
+constexpr int kFlagOff = kFacOff + 2 * 4 * 16 * 4;  // [parity][4 producers] int
+constexpr int kStatOff = kFlagOff + 2 * 4 * 4;      // [4 producers][16 heads][2] fp32
+constexpr int kValidOff = kStatOff + 4 * 16 * 2 * 4;  // [tile] int: every key of the tile is valid
+constexpr int kKeyOff = kValidOff + (kMaxKeys / kTK) * 4;
+constexpr int kSmem = kKeyOff + kKeyInts * 4;
+static_assert(kSmem <= 160 * 1024, "LDS budget");
+static_assert(4 * 32 * kXPitch * 4 <= kRingBytes, "the output transpose reuses the ring");
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ bf16x8 cvt8(unsigned w0, unsigned w1) {
+  const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, 1.0f, false));
+  const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, 1.0f, true));
+  const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, false));
+  const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, true));
+  return __builtin_bit_cast(bf16x8, make_uint4(o0, o1, o2, o3));
+}
+
+// sign and mantissa of a scale with the exponent of 1.0: scale = 2^(exponent field - 127) * this
+__device__ __forceinline__ float scale_mant(float s) {
+  return __uint_as_float((__float_as_uint(s) & 0x807fffffu) | 0x3f800000u);
+}
+
+// 16 x 16 x 128 over e4m3 bytes, operands scaled by 2^(byte - 127): the byte is byte SEL of `a_exp`
+// for A and of `b_exp` for B, and must be the same in the four lanes of a row (l, l+16, ..).
+template <int SEL>
+__device__ __forceinline__ void mfma_s8(f32x4& acc, const i32x8& a, const i32x8& b, int a_exp, int b_exp) {
+  acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, SEL, a_exp, SEL, b_exp);
+}
+__device__ __forceinline__ void mfma_s(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mfma_o(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
+
+// 32 bf16 (four 16-byte pieces, channel order) of each lane -> e4m3 hi + e4m3 lo with hi + lo = x,
+// both in units of 2^(e - 127); returns e, common to lanes l, l^16, l^32, l^48 (one head's 128
+// channels).  hi carries the upper four significant bits of a bf16 value and lo the lower four, so
+// the pair is exact for every element within ~2^-14 of the largest of the 128 and off by less
+// than 2^-18 of that largest one otherwise.
+__device__ __forceinline__ int split_q32(const uint4 (&x)[4], i32x8& hi, i32x8& lo) {
+  u16x2 top = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned w[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2, w[d] & 0x7fff7fffu));
+  }
+  int amax_bits = max((int)top[0], (int)top[1]);             // bf16 bits of the largest magnitude
+  amax_bits = max(amax_bits, __float_as_int(xor16(__int_as_float(amax_bits))));
+  amax_bits = max(amax_bits, __float_as_int(xor32(__int_as_float(amax_bits))));
+  const int e = max((amax_bits >> 7) - 7, 1);                 // |x| / 2^(e-127) < 256
+  const float unit = __uint_as_float((unsigned)e << 23);
+  const i16x2 zero = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned w[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      const unsigned w0 = w[2 * d], w1 = w[2 * d + 1];
+      i16x2 h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(zero, __builtin_bit_cast(bf16x2, w0), unit, false);
+      h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(h, __builtin_bit_cast(bf16x2, w1), unit, true);
+      const unsigned hw = __builtin_bit_cast(unsigned, h);
+      const f32x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(hw, unit, false);
+      const f32x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(hw, unit, true);
+      i16x2 l = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(zero, __uint_as_float(w0 << 16) - d0[0],
+                                                         __uint_as_float(w0 & 0xffff0000u) - d0[1], unit, false);
+      l = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(l, __uint_as_float(w1 << 16) - d1[0],
+                                                   __uint_as_float(w1 & 0xffff0000u) - d1[1], unit, true);
+      hi[2 * j + d] = (int)hw;
+      lo[2 * j + d] = __builtin_bit_cast(int, l);
+    }
+  }
+  return e;
+}
+
+// v_max_f32 as it is (fmaxf first passes every operand through a canonicalising max with itself).
+// Only for operands that ordinary vector instructions produced: never for matrix results, whose
+// read-after-write wait states the compiler pads only for instructions it can see.
+__device__ __forceinline__ float vmax(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// maximum over lanes l, l^16, l^32, l^48 (every lane gets it): a row swap leaves each value next
+// to its partner's
+__device__ __forceinline__ float max_rows(float v) {
+  unsigned u = __float_as_uint(v);
+  u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = vmax(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  u = __float_as_uint(v);
+  r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return vmax(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// NBLK: fp32 scales per key row (1, 2 or 4)
+template <int NBLK>
+__global__ __launch_bounds__(512, 2) void sparse_mla_latent_pc_kernel(const MlaParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = (int)threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave < 4;
+  const int role = wave & 3;                    // producer p / consumer c
+  constexpr int nblk = NBLK;
+  TICK(producer ? 0 : 32);
+
+  // ---- which (query, KV group, head chunk, split).  Workgroup ids that are equal modulo 8 run on
+  //      the same XCD and share its L2: every workgroup of one (query, KV group) gets such ids, so
+  //      the gathered key rows are fetched from HBM once for both head chunks and the query rows
+  //      once for all key splits ----
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
+  const long long per_q = (long long)p.num_splits * chunks;    // workgroups of one (query, KV group)
+  const long long nq = (long long)p.B * p.S * p.G;
+  const long long nq8 = nq & ~7ll;
+  long long qg;
+  int chunk, split;
+  {
+    const long long id = blockIdx.x;
+    long long r;
+    if (id < nq8 * per_q) {
+      const long long slot = id >> 3;
+      qg = (slot / per_q) * 8 + (id & 7);
+      r = slot % per_q;
+    } else {
+      const long long rest = id - nq8 * per_q;
+      qg = nq8 + rest / per_q;
+      r = rest % per_q;
+    }
+    split = (int)(r / chunks);
+    chunk = (int)(r % chunks);
+  }
+  const int g = (int)(qg % p.G);
+  const size_t bs = (size_t)(qg / p.G);           // b*S + s
+  const int b = (int)(bs / p.S);
+  const int head0 = g * p.heads_per_group + chunk * kHeadsWg;
+  const int heads_here = min(kHeadsWg, p.heads_per_group - chunk * kHeadsWg);
+  const size_t idx_base = (bs * p.G + g) * (size_t)p.topk;
+  const int key_begin = split * p.keys_per_split;
+  const int key_end = min(p.topk, key_begin + p.keys_per_split);
+  const int n_keys = max(0, key_end - key_begin);
+  const int list_tiles = (n_keys + kTK - 1) / kTK;
+
+  const bool has_scale = p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;   // otherwise the scale area holds ones
+
+  int* keys = reinterpret_cast<int*>(smem + kKeyOff);
+  float* facbuf = reinterpret_cast<float*>(smem + kFacOff);
+  int* flagbuf = reinterpret_cast<int*>(smem + kFlagOff);
+  float* stats = reinterpret_cast<float*>(smem + kStatOff);
+  int* tvalid = reinterpret_cast<int*>(smem + kValidOff);
+
+  if (!has_scale) {                               // no scales in memory: every slot's scale area is 1.0 for good
+    for (int i = tid; i < kRing * kTK; i += 512)
+      reinterpret_cast<float*>(smem + (i / kTK) * kSlotBytes + kLatBytes + kRopeBytes)[i % kTK] = 1.0f;
+  }
+  // ---- cache rows of this split's keys -> LDS (-1 = skipped) ----
+  int* last_valid = reinterpret_cast<int*>(stats);          // [8], one per wavefront (the statistics come much later)
+  // thread t takes list entries t, t + 512, ..: every index word is requested before the first one
+  // is looked at (one memory round trip), unconditionally, with positions clamped to the list.
+  // The producers put their query-row requests between the two halves: the load unit then
+  // moves the 74 KB of query rows while the index words are on their way, instead of in front of
+  // the first key tile.
+  constexpr int kRounds = kMaxKeys / 512;
+  const bool wide = p.index_dtype == CPPMEGA_MI355_I64;
+  int idx_lo[kRounds], idx_hi[kRounds];
+  {
+    const int* words = (const int*)p.indices;
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+      idx_lo[r] = 0; idx_hi[r] = 0;
+      if (r * 512 < list_tiles * kTK) {           // (uniform)
+        const size_t at = idx_base + (size_t)min(key_begin + tid + 512 * r, p.topk - 1);
+        const size_t w0 = wide ? 2 * at : at;
+        idx_lo[r] = words[w0];
+        idx_hi[r] = words[w0 + (wide ? 1 : 0)];
+      }
+    }
+  }
+  auto stage_keys = [&]() {
+    const int ctid = tid;
+    int* lo = idx_lo; int* hi = idx_hi;
+    int mine = -1;
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+      if (r * 512 < list_tiles * kTK) {
+        const int i = ctid + 512 * r;
+        const long long k = wide ? (long long)(((unsigned long long)(unsigned)hi[r] << 32) | (unsigned)lo[r]) : (long long)lo[r];
+        const bool ok = i < n_keys && k >= 0 && k < p.Skv;
+        int row = ok ? (int)k : -1;
+#ifdef CM_PC_HOT_ROWS
+        if (row >= 0) row = row & 1023;
+#endif
+        if (i < list_tiles * kTK) keys[i] = row;
+        if (ok) mine = i;
+        // a tile is the 32 consecutive entries of half a wavefront; the masked-key path also serves a
+        // non-positive softmax scale (the plain path takes maxima before scaling)
+        const unsigned long long okm = __ballot(ok && p.sm_scale > 0.0f);
+        if ((lane & 31) == 0 && i < list_tiles * kTK) tvalid[i / kTK] = (unsigned)(okm >> (lane & 32)) == 0xffffffffu;
+      }
+    }
+    mine = max(mine, __shfl_xor(mine, 1, 64));
+    mine = max(mine, __shfl_xor(mine, 2, 64));
+    mine = max(mine, __shfl_xor(mine, 4, 64));
+    mine = max(mine, __shfl_xor(mine, 8, 64));
+    mine = max(mine, __shfl_xor(mine, 16, 64));
+    mine = max(mine, __shfl_xor(mine, 32, 64));
+    if (lane == 0) last_valid[wave] = mine;
+  };
+  // causal padding puts the skipped (-1) slots at the end of a list: tiles past the last valid key do nothing
+  auto count_tiles = [&]() {
+    int m = -1;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) m = max(m, last_valid[w]);
+    return __builtin_amdgcn_readfirstlane((m + kTK) / kTK);
+  };
+  const size_t q_index = bs;
+  // key-split partials: one block per (query, KV group, head chunk, split)
+  const size_t part_block = (size_t)(((long long)bs * p.G + g) * chunks + chunk) * p.num_splits + split;
+  const size_t part_blocks_total = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
+
+#ifdef CM_PC_TIMING
+  if (blockIdx.x == 0 && lane == 0) g_pc_ticks[48 + wave] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+#endif
+  if (producer) {
+    // =====================================================================================
+    // producer p = role: heads 16p .. 16p+15 of the chunk
+    // =====================================================================================
+    const int n = lane & 15, kg = lane >> 4;
+    // Q^T operands: lane (head n, kg) holds channels 128 blk + 32 kg .. +31 of the latent and
+    // channels 512 + 32 r + 8 kg .. +7 of the rope tail
+    uint4 qraw[4][4];
+    bf16x8 qr[2];
+    {
+      const int h = 16 * role + n;
+      // heads past the end of the group repeat head 0: their columns stay finite and are never stored
+      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (h < heads_here ? h : 0)) * (size_t)kDqk;
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qraw[blk][j] = *reinterpret_cast<const uint4*>(qrow + 128 * blk + 32 * kg + 8 * j);
+#pragma unroll
+      for (int r = 0; r < 2; ++r) qr[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kg));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    stage_keys();
+    if (wave == 0) TICK(16);
+    __syncthreads();                                // keys[] is complete
+    if (wave == 0) TICK(17);
+    const int n_tiles = count_tiles();
+    i32x8 qh[4], ql[4];
+    int qexp = 0;
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) qexp |= split_q32(qraw[blk], qh[blk], ql[blk]) << (8 * blk);
+    if (role == 0) TICK(1);
+    float m_run = -INFINITY;                      // base-2 running reference of head n
+    float l_run = 0.0f;                           // this lane's share of its denominator
+    const float qk_scale = p.sm_scale * kLog2e;
+
+    // K operands of a tile -> registers: per sub-tile four 32-byte block fragments, two rope
+    // fragments and the scales of this lane's key row (they give the operand exponents).  They are
+    // requested one tile ahead, right after the previous tile's products, so that they land
+    // under its softmax.
+    i32x8 kf[2][4];
+    bf16x8 rf[2][2];
+    float own[2][nblk];
+    auto load_k = [&](int tau) {
+      const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
+      const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        const float* scl = scl_base + (16 * sj + n) * nblk;
+        if (nblk == 4) {
+          const float4 o4 = *reinterpret_cast<const float4*>(scl);
+          own[sj][0] = o4.x; own[sj][1 % nblk] = o4.y; own[sj][2 % nblk] = o4.z; own[sj][3 % nblk] = o4.w;
+        } else if (nblk == 2) {
+          const float2 o2 = *reinterpret_cast<const float2*>(scl);
+          own[sj][0] = o2.x; own[sj][1 % nblk] = o2.y;
+        } else {
+          own[sj][0] = scl[0];
+        }
+      }
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        // the lane's 32 bytes of a block are its 16 bytes of the block's two planes
+        const unsigned char* lat = slot + sj * (4 * kPair) + lane * 16;
+        const unsigned char* rope = slot + kLatBytes + sj * 2048 + lane * 16;
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+          const uint4 c0 = *reinterpret_cast<const uint4*>(lat + blk * kPair);
+          const uint4 c1 = *reinterpret_cast<const uint4*>(lat + blk * kPair + kPlane);
+          kf[sj][blk] = i32x8{(int)c0.x, (int)c0.y, (int)c0.z, (int)c0.w, (int)c1.x, (int)c1.y, (int)c1.z, (int)c1.w};
+        }
+        rf[sj][0] = *reinterpret_cast<const bf16x8*>(rope);
+        rf[sj][1] = *reinterpret_cast<const bf16x8*>(rope + 1024);
+      }
+    };
+
+    // scores and probabilities of tile tau (whose K operands are in registers) -> P(tau) in LDS;
+    // `next`: tile tau+1 exists (it has landed)
+    auto produce = [&](int tau, bool next) {
+      const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
+      const int spar = tau & 1;
+      const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
+      const bool all_valid = tvalid[tau] != 0;      // (uniform) no skipped key in this tile
+      float ksc[2][4][nblk];                        // scales of keys 16 sj + 4 kg + i (partial sums, P)
+      int4 kk[2] = {make_int4(0, 0, 0, 0), make_int4(0, 0, 0, 0)};
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        const float* sclc = scl_base + (16 * sj + 4 * kg) * nblk;
+        if (nblk == 4) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float4 v4 = *reinterpret_cast<const float4*>(sclc + 4 * i);
+            ksc[sj][i][0] = v4.x; ksc[sj][i][1 % nblk] = v4.y; ksc[sj][i][2 % nblk] = v4.z; ksc[sj][i][3 % nblk] = v4.w;
+          }
+        } else if (nblk == 2) {
+          const float4 a = *reinterpret_cast<const float4*>(sclc), bq = *reinterpret_cast<const float4*>(sclc + 4);
+          ksc[sj][0][0] = a.x; ksc[sj][0][1 % nblk] = a.y; ksc[sj][1][0] = a.z; ksc[sj][1][1 % nblk] = a.w;
+          ksc[sj][2][0] = bq.x; ksc[sj][2][1 % nblk] = bq.y; ksc[sj][3][0] = bq.z; ksc[sj][3][1 % nblk] = bq.w;
+        } else {
+          const float4 a = *reinterpret_cast<const float4*>(sclc);
+          ksc[sj][0][0] = a.x; ksc[sj][1][0] = a.y; ksc[sj][2][0] = a.z; ksc[sj][3][0] = a.w;
+        }
+        if (!all_valid) kk[sj] = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * sj + 4 * kg);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // exponent bytes of this lane's key rows, and whether any row of the tile has a mantissa part
+      int kexp[2];
+      bool plain = true;
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        kexp[sj] = 0;
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+          const unsigned sc = __float_as_uint(own[sj][(blk * nblk) >> 2]);
+          kexp[sj] |= (int)(((sc >> 23) & 0xffu) << (8 * blk));
+          plain = plain && ((sc & 0x807fffffu) == 0u);
+        }
+      }
+      const bool all_plain = __ballot(!plain) == 0ull;       // (uniform)
+      f32x4 st[2];
+      st[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+      st[1] = st[0];
+#ifdef CM_PC_NO_MFMA
+      for (int sj = 0; sj < 2; ++sj) for (int b2 = 0; b2 < 4; ++b2) st[sj][b2] = __int_as_float(kf[sj][b2][0] ^ kf[sj][b2][7]) + (float)rf[sj][0][0] + (float)rf[sj][1][0];
+      if (false) {
+#else
+      if (all_plain) {
+#endif
+        // one sub-tile after the other: the second one's operands are still landing
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          mfma_s8<0>(st[sj], kf[sj][0], qh[0], kexp[sj], qexp);
+          mfma_s8<0>(st[sj], kf[sj][0], ql[0], kexp[sj], qexp);
+          mfma_s8<1>(st[sj], kf[sj][1], qh[1], kexp[sj], qexp);
+          mfma_s8<1>(st[sj], kf[sj][1], ql[1], kexp[sj], qexp);
+          mfma_s8<2>(st[sj], kf[sj][2], qh[2], kexp[sj], qexp);
+          mfma_s8<2>(st[sj], kf[sj][2], ql[2], kexp[sj], qexp);
+          mfma_s8<3>(st[sj], kf[sj][3], qh[3], kexp[sj], qexp);
+          mfma_s8<3>(st[sj], kf[sj][3], ql[3], kexp[sj], qexp);
+          mfma_s(st[sj], rf[sj][0], qr[0]);
+          mfma_s(st[sj], rf[sj][1], qr[1]);
+        }
+      } else {
+        // each block is accumulated apart and enters the score times its keys' mantissa factors; the
+        // two sub-tiles alternate so that a block's factors are applied under the other's products
+        auto block = [&](auto blk_c) {
+          constexpr int blk = decltype(blk_c)::value;
+          f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0;
+          mfma_s8<blk>(a0, kf[0][blk], qh[blk], kexp[0], qexp);
+          mfma_s8<blk>(a1, kf[1][blk], qh[blk], kexp[1], qexp);
+          mfma_s8<blk>(a0, kf[0][blk], ql[blk], kexp[0], qexp);
+          mfma_s8<blk>(a1, kf[1][blk], ql[blk], kexp[1], qexp);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            st[0][i] += scale_mant(ksc[0][i][(blk * nblk) >> 2]) * a0[i];
+            st[1][i] += scale_mant(ksc[1][i][(blk * nblk) >> 2]) * a1[i];
+          }
+        };
+        block(std::integral_constant<int, 0>{});
+        block(std::integral_constant<int, 1>{});
+        block(std::integral_constant<int, 2>{});
+        block(std::integral_constant<int, 3>{});
+        mfma_s(st[0], rf[0][0], qr[0]);
+        mfma_s(st[1], rf[1][0], qr[0]);
+        mfma_s(st[0], rf[0][1], qr[1]);
+        mfma_s(st[1], rf[1][1], qr[1]);
+      }
+
+      __builtin_amdgcn_sched_barrier(0);
+      // The scale reads issued before the products have long landed: say so before the next batch of
+      // reads.  (The LDS counter holds 15 at most; without this the compiler, unable to name "all
+      // but the last 22", makes the first use of a scale wait for most of that batch.)
+      __builtin_amdgcn_s_waitcnt(0xc07f);           // lgkmcnt(0)
+#ifndef CM_PC_NO_LOADK
+      if (next) load_k(tau + 1);                    // (the fragment registers are free again)
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+#ifdef CM_PC_NO_SOFTMAX
+      if (st[0][0] + st[1][0] == 1.2345f) l_run += 1.0f;
+      return;
+#endif
+      // ---- softmax: this lane holds head n, keys 16 sj + 4 kg + i ----
+      float mx;
+      float mul = qk_scale;                         // what turns a held sum into a base-2 score
+      if (all_valid) {
+        // no skipped key: the maximum is taken on the raw sums (qk_scale > 0 on this path)
+        // (fmaxf, not the raw instruction: the compiler pads the wait states a vector instruction
+        // needs before it may read matrix results only for instructions it can see)
+        mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
+                   fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
+      } else {
+        mx = -INFINITY;
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          const bool ok[4] = {kk[sj].x >= 0, kk[sj].y >= 0, kk[sj].z >= 0, kk[sj].w >= 0};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            st[sj][e] = ok[e] ? st[sj][e] * qk_scale : -INFINITY;
+            mx = fmaxf(mx, st[sj][e]);
+          }
+        }
+        mul = 1.0f;
+      }
+      mx = max_rows(mx) * mul;                 // over the four key quarters (lanes n, n+16, n+32, n+48)
+      {
+        const bool grow = mx > m_run + kLazy;
+        // accumulators of a head whose reference was -inf are still zero: nothing to rescale
+        const bool rescale = grow && m_run != -INFINITY;
+        const bool any_rescale = __ballot(rescale) != 0ull;
+        float fac = 1.0f;
+        if (grow) {
+          fac = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - mx);
+          l_run *= fac;
+          m_run = mx;
+        }
+        if (any_rescale && lane < 16) facbuf[(spar * 4 + role) * 16 + n] = fac;
+        if (lane == 0) flagbuf[spar * 4 + role] = any_rescale ? 1 : 0;
+      }
+      // exp2(-inf - m) is 0 for a finite m; a head with no valid key yet keeps m_run = -inf
+      const float neg_m = -vmax(m_run, -1.0e30f);
+      unsigned char* pdst = smem + kPOff + spar * kPBytes;
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        float pr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pr[i] = fast_exp2(__builtin_fmaf(st[sj][i], mul, neg_m));
+          l_run += pr[i];
+        }
+        // P (x V's block scale) -> LDS in the B-operand layout of the 32x32x16 product: lane
+        // (head of a 32-head block, key/8) owns 16 bytes = 8 keys; this lane holds keys 4kg..4kg+3
+        unsigned char* dst = pdst + ((sj * 2 + (role >> 1)) * 64 + (role & 1) * 16 + n + (kg >> 1) * 32) * 16 + (kg & 1) * 8;
+#pragma unroll
+        for (int v = 0; v < nblk; ++v) {
+          const uint2 w = make_uint2(pack_bf16(pr[0] * ksc[sj][0][v], pr[1] * ksc[sj][1][v]),
+                                     pack_bf16(pr[2] * ksc[sj][2][v], pr[3] * ksc[sj][3][v]));
+          *reinterpret_cast<uint2*>(dst + v * kPVarBytes) = w;
+        }
+      }
+    };
+
+    // t = -1: [X] tile 0 has landed.  t >= 0: [B_t] tile t+2 has landed, P(t) is complete, the value
+    // product of tile t-1 is done.
+    for (int t = -1; t < n_tiles; ++t) {
+      __syncthreads();
+      if (t == -1 && role == 0) TICK(2);
+      // (the first barrier only promises tile 0: tile 1's operands are read a round late, once)
+      if (t <= 0 && t + 1 < n_tiles) load_k(t + 1);
+#ifndef CM_PC_NO_PRODUCE
+      if (t + 1 < n_tiles) produce(t + 1, t >= 0 && t + 2 < n_tiles);
+#endif
+      if (t == -1 && role == 0) TICK(3);
+    }
+    if (role == 0) TICK(4);
+    l_run += xor16(l_run);
+    l_run += xor32(l_run);
+    if (lane < 16) {
+      stats[(role * 16 + lane) * 2 + 0] = m_run;
+      stats[(role * 16 + lane) * 2 + 1] = l_run;
+    }
+#ifdef CM_PC_DEBUG
+    if (blockIdx.x == CM_PC_TICK_WG && tid == 0) {
+      g_pc_ticks[60] = (unsigned long long)__float_as_uint(m_run) | ((unsigned long long)__float_as_uint(l_run) << 32);
+      g_pc_ticks[61] = (unsigned long long)n_tiles;
+    }
+#endif
+    __syncthreads();                              // [E] statistics are visible; the ring is free
+    return;
+  }
+
+  // =======================================================================================
+  // consumer c = role: value channels 128c .. 128c+127 of all 64 heads; also the row loads
+  // =======================================================================================
+  stage_keys();
+  __syncthreads();                                // keys[] is complete
+  const int n_tiles = count_tiles();
+#if defined(CM_PC_TIMING) || defined(CM_PC_DEBUG)
+  if (blockIdx.x == CM_PC_TICK_WG && tid == 256) {
+    g_pc_ticks[56] = (unsigned long long)n_tiles;
+    g_pc_ticks[57] = (unsigned long long)(unsigned)last_valid[0] | ((unsigned long long)(unsigned)last_valid[7] << 32);
+    g_pc_ticks[58] = (unsigned long long)(unsigned)keys[0] | ((unsigned long long)(unsigned)keys[1] << 32);
+    g_pc_ticks[59] = (unsigned long long)(unsigned)n_keys | ((unsigned long long)(unsigned)list_tiles << 32);
+  }
+#endif
+  // HBM -> LDS: this wavefront brings rows 8c .. 8c+7 of a tile.  A skipped key fetches cache
+  // row 0 instead (its probability is zero), so every tile is the same number of load
+  // instructions and the in-order load counter can be waited on by count.  The loads are inline
+  // assembly: the compiler would otherwise order every later LDS read behind them.
+  //   latent : block c of both sub-tiles, two planes each: lane (n, kg) of plane j fetches bytes
+  //            128 c + 32 kg + 16 j .. + 15 of key 16 sj + n
+  //   rope   : plane (sj = c / 2, s = c % 2): lane (n, kq) fetches bytes 64 s + 16 kq .. + 15 of the rope row
+  //   scales : element 64c + lane of [32 rows][nblk]
+  const bool scale_op = has_scale && 64 * role < kTK * nblk;
+  const size_t group_row0 = ((size_t)b * p.Skv) * p.G + g;     // cache row of key 0; key k is G rows further per step
+  const int sc_elem = 64 * role + lane;
+  const int sc_row = min(sc_elem / nblk, kTK - 1);
+  const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + 128 * role + 32 * (lane >> 4);
+  const unsigned char* rope_src = (const unsigned char*)p.rope + group_row0 * (kRope * 2) + 64 * (role & 1) + 16 * (lane >> 4);
+  const unsigned char* sc_src = (const unsigned char*)p.kv_scale + (group_row0 * nblk + (unsigned)(sc_elem % nblk)) * 4;
+  const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = (unsigned)p.G * nblk * 4;
+  auto dma16 = [&](const unsigned char* src, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+  };
+  auto dma4 = [&](const unsigned char* src, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+  };
+  const unsigned smem_base = (unsigned)(size_t)(lds_void*)smem;                 // LDS byte address of the ring
+  // one tile is six load instructions (five without a scale instruction): prepare computes the
+  // row numbers, part(i) issues instruction i.  The value product spreads the parts between its
+  // matrix instructions: issuing blocks while the load unit's queue is full.
+  unsigned dma_slot = 0;
+  size_t dma_r0 = 0, dma_r1 = 0, dma_rs = 0;
+  auto dma_prepare = [&](int tau) {
+    dma_slot = smem_base + (unsigned)(tau % kRing) * kSlotBytes;
+    const int* tk = keys + tau * kTK;
+    const int k0 = tk[lane & 15], k1 = tk[16 + (lane & 15)];        // this lane's key of sub-tile 0 / 1
+    const int ksc_row = scale_op ? tk[sc_row] : 0;
+    dma_r0 = (size_t)(unsigned)max(k0, 0);
+    dma_r1 = (size_t)(unsigned)max(k1, 0);
+    dma_rs = (size_t)(unsigned)max(ksc_row, 0);
+  };
+  auto dma_part = [&](int i) {
+    if (i == 0) dma16(lat_src + dma_r0 * lat_step, dma_slot + role * kPair);
+    else if (i == 1) dma16(lat_src + dma_r0 * lat_step + 16, dma_slot + role * kPair + kPlane);
+    else if (i == 2) dma16(lat_src + dma_r1 * lat_step, dma_slot + (4 + role) * kPair);
+    else if (i == 3) dma16(lat_src + dma_r1 * lat_step + 16, dma_slot + (4 + role) * kPair + kPlane);
+    else if (i == 4) dma16(rope_src + ((role >> 1) ? dma_r1 : dma_r0) * rope_step, dma_slot + kLatBytes + role * 1024);
+    else if (scale_op) {
+      if (sc_elem < kTK * nblk) dma4(sc_src + dma_rs * sc_step, dma_slot + kLatBytes + kRopeBytes + 256 * role);
+    }
+  };
+  auto issue_tile = [&](int tau) {
+    dma_prepare(tau);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) dma_part(i);
+  };
+  // wait until at most `tiles` of the most recently issued tiles are still in flight
+  auto wait_outstanding = [&](int tiles) {
+    const int per = scale_op ? 6 : 5;
+    switch (min(tiles, 5) * per) {
+      case 30: asm volatile("s_waitcnt vmcnt(30)" ::: "memory"); break;
+      case 25: asm volatile("s_waitcnt vmcnt(25)" ::: "memory"); break;
+      case 24: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+      case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+      case 18: asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); break;
+      case 15: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
+      case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+  };
+
+  // ---- value side state: o[dvb][hb] = O^T[32 channels x 32 heads] ----
+  f32x16 o[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) o[i][hb][j] = 0.0f;
+  const int pvar = (role * nblk) >> 2;                         // scale block of channels 128c..
+  int pv_off[4];                                               // transposing-read offsets per 32-channel block
+  {
+    // lanes t = 0..15 of a group read 8 bytes each from eight consecutive keys' 16-byte pieces (128
+    // contiguous bytes); half selects the plane, kq2 the upper eight keys of the step
+    const int t = lane & 15, half = (lane >> 4) & 1, kq2 = lane >> 5;
+    const int r = 8 * kq2 + (t >> 1);                          // key within the 16-key step
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) pv_off[dvb] = role * kPair + half * kPlane + (dvb * 16 + r) * 16 + 8 * (t & 1);
+  }
+  // V^T fragments of one 16-key step (four 32-channel blocks), raw
+  auto load_v = [&](int tau, int kstep, i32x2 (&vr)[4]) {
+    const unsigned char* vslot = smem + (tau % kRing) * kSlotBytes + kstep * (4 * kPair);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb)
+      vr[dvb] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(vslot + pv_off[dvb]));
+  };
+  i32x2 v0[4];                                    // first step of the tile about to be consumed (read ahead of the barrier)
+  // value product of tile tv; `next`: tile tv+1 exists (it has landed: the producers are reading it)
+  auto consume = [&](int tv, bool next, bool dma) {
+    const int vpar = tv & 1;
+    if (dma) dma_prepare(tv + kAhead);
+    const unsigned char* pfrag = smem + kPOff + vpar * kPBytes + pvar * kPVarBytes + lane * 16;
+    bf16x8 pb[2][2];
+#pragma unroll
+    for (int kstep = 0; kstep < 2; ++kstep)
+#pragma unroll
+      for (int hb = 0; hb < 2; ++hb) pb[kstep][hb] = *reinterpret_cast<const bf16x8*>(pfrag + (kstep * 2 + hb) * 1024);
+    const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
+    i32x2 v1[4];
+    load_v(tv, 1, v1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (__builtin_amdgcn_readfirstlane(fl.x | fl.y | fl.z | fl.w) != 0) {      // producers moved a reference: rescale (rare)
+#pragma unroll
+      for (int hb = 0; hb < 2; ++hb) {
+        const int hd = lane & 31;
+        const int fl_p = hb == 0 ? ((hd >> 4) ? fl.y : fl.x) : ((hd >> 4) ? fl.w : fl.z);
+        const float fsc = fl_p ? facbuf[(vpar * 4 + 2 * hb + (hd >> 4)) * 16 + (hd & 15)] : 1.0f;
+#pragma unroll
+        for (int dvb = 0; dvb < 4; ++dvb)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) o[dvb][hb][j] *= fsc;
+      }
+    }
+    bf16x8 a[4];
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) a[dvb] = cvt8((unsigned)v0[dvb][0], (unsigned)v0[dvb][1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+      mfma_o(o[dvb][0], a[dvb], pb[0][0]);
+      mfma_o(o[dvb][1], a[dvb], pb[0][1]);
+      if (dma) dma_part(dvb);
+    }
+    if (next) load_v(tv + 1, 0, v0);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) a[dvb] = cvt8((unsigned)v1[dvb][0], (unsigned)v1[dvb][1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+      mfma_o(o[dvb][0], a[dvb], pb[1][0]);
+      mfma_o(o[dvb][1], a[dvb], pb[1][1]);
+      if (dma && dvb < 2) dma_part(4 + dvb);
+    }
+  };
+
+  // ---- pipeline ----
+  // only the first tile is requested ahead of the first barrier (issuing blocks while the load
+  // unit's queue is full, and the producers cannot start before this wavefront gets there)
+  if (role == 0) TICK(18);
+  if (n_tiles > 0) issue_tile(0);
+  if (role == 0) TICK(19);
+  wait_outstanding(0);                            // tile 0 has landed
+  if (role == 0) TICK(20);
+  __syncthreads();                                // [X]
+#pragma unroll
+  for (int tau = 1; tau < kAhead; ++tau)
+    if (tau < n_tiles) issue_tile(tau);
+  if (n_tiles > 0) load_v(0, 0, v0);
+  wait_outstanding(max(min(kAhead, n_tiles) - 3, 0));   // tile 2 has landed
+  if (role == 0) TICK(33);
+  for (int t = 0; t < n_tiles; ++t) {
+    __syncthreads();                              // [B_t]
+#ifdef CM_PC_NO_DMA
+    const bool more = false;
+#else
+    const bool more = t + kAhead < n_tiles;
+#endif
+#ifdef CM_PC_NO_CONSUME
+    if (more) issue_tile(t + kAhead);
+#else
+    consume(t, t + 1 < n_tiles, more);            // (tile t+4 goes into the slot of tile t-1)
+#endif
+    // tile t+3 must have landed before the next barrier; the tile issued after it may stay in flight
+    wait_outstanding(max(min(t + kAhead, n_tiles - 1) - (t + 3), 0));
+  }
+  if (role == 0) TICK(34);
+  __syncthreads();                                // [E] statistics are visible; the ring is free
+  if (role == 0) TICK(35);
+
+  // ---- epilogue ----
+  const int hd = lane & 31, gq2 = lane >> 5;
+  const bool direct = p.num_splits == 1;
+  float* xbuf = reinterpret_cast<float*>(smem) + role * 32 * kXPitch;     // private to this wavefront
+#pragma unroll
+  for (int hb = 0; hb < 2; ++hb) {
+    const float m_all = stats[((2 * hb + (hd >> 4)) * 16 + (hd & 15)) * 2];
+    const float l_all = stats[((2 * hb + (hd >> 4)) * 16 + (hd & 15)) * 2 + 1];
+    const int h_local = 32 * hb + hd;
+#ifdef CM_PC_NO_PARTIALS
+    if (!direct) continue;
+#endif
+    if (!direct) {
+      // key split: the unnormalised accumulators leave exactly as the lanes hold them (rounded to
+      // bf16: the values are relative to the split's own maximum, so their range is that of the
+      // output times the split's probability mass)
+      unsigned short* blk = (unsigned short*)p.workspace + part_block * (size_t)(2 * kPartFloats) +
+                            ((size_t)((role * 2 + hb) * 16) * 64 + lane) * 4;
+#pragma unroll
+      for (int dvb = 0; dvb < 4; ++dvb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x16& acc = o[dvb][hb];
+          *reinterpret_cast<uint2*>(blk + (size_t)(dvb * 4 + j) * 256) =
+              make_uint2(pack_bf16(acc[4 * j], acc[4 * j + 1]), pack_bf16(acc[4 * j + 2], acc[4 * j + 3]));
+        }
+      }
+      if (role == 0 && lane < 32) {
+        float* ml = (float*)((unsigned short*)p.workspace + part_blocks_total * (size_t)(2 * kPartFloats)) + (part_block * kHeadsWg + h_local) * 2;
+        ml[0] = m_all;
+        ml[1] = l_all;
+      }
+      continue;
+    }
+    float out_scale = 1.0f, lse_val = 0.0f;
+    {
+      float m_fin = m_all, l_fin = l_all;
+      if (p.sinks && h_local < heads_here) {
+        const float sk = p.sinks[head0 + h_local] * kLog2e;
+        const float m2 = fmaxf(m_fin, sk);
+        const float keep = (m_fin == -INFINITY) ? 0.0f : exp2f(m_fin - m2);
+        l_fin = l_fin * keep + exp2f(sk - m2);
+        out_scale = keep;
+        m_fin = m2;
+      }
+      if (l_fin > 0.0f) {
+        out_scale = out_scale / l_fin;
+        lse_val = (m_fin + log2f(l_fin)) * kLn2;
+      } else {
+        out_scale = 0.0f;
+      }
+    }
+    // transpose through LDS: lane (head hd, gq2) holds channels 32dvb + 8j + 4gq2 + (0..3) in o[.][4j..4j+3]
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x16& acc = o[dvb][hb];
+        const float4 v = make_float4(acc[4 * j] * out_scale, acc[4 * j + 1] * out_scale, acc[4 * j + 2] * out_scale,
+                                     acc[4 * j + 3] * out_scale);
+        *reinterpret_cast<float4*>(xbuf + hd * kXPitch + 32 * dvb + 8 * j + 4 * gq2) = v;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // rows of 128 channels leave coalesced: 32 lanes x 4 channels, two heads per step
+#pragma unroll 4
+    for (int it = 0; it < 16; ++it) {
+      const int row = 2 * it + gq2;
+      const int hl = 32 * hb + row;
+      if (hl >= heads_here) continue;
+      const float4 v = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + hd * 4);
+      const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + 128 * role + hd * 4;
+      if (p.out_dtype == CPPMEGA_MI355_F32) {
+        *reinterpret_cast<float4*>((float*)p.out + off) = v;
+      } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
+        *reinterpret_cast<uint2*>((unsigned short*)p.out + off) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
+      } else {
+        unsigned short* dst = (unsigned short*)p.out + off;
+        dst[0] = f32_to_f16_bits(v.x); dst[1] = f32_to_f16_bits(v.y);
+        dst[2] = f32_to_f16_bits(v.z); dst[3] = f32_to_f16_bits(v.w);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (role == 0 && lane < 32 && h_local < heads_here && p.lse) p.lse[q_index * p.H + head0 + h_local] = lse_val;
+  }
+  if (role == 0) TICK(36);
+}
+
+}  // namespace
+
+#if defined(CM_PC_TIMING) || defined(CM_PC_DEBUG)
+extern "C" int cm_dbg_pc_ticks(unsigned long long* host, int reset) {
+  if (reset) {
+    unsigned long long z[64] = {0};
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pc_ticks), z, sizeof(z));
+  }
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pc_ticks), 64 * sizeof(unsigned long long));
+}
+#endif
+
+bool sparse_mla_latent_pc_supported(const MlaParams& p) {
+  if (p.q_dtype != CPPMEGA_MI355_BF16 || p.q_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
+  if (p.d_qk != kDqk || p.d_v != kLat || p.d_kv != kLat) return false;
+  if (p.kv_dtype != CPPMEGA_MI355_E4M3) return false;
+  if (p.rope_dim != kRope || p.rope_dtype != CPPMEGA_MI355_BF16) return false;
+  if (p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK) {
+    if (p.kv_scale_block != 128 && p.kv_scale_block != 256 && p.kv_scale_block != 512) return false;
+  } else if (p.kv_scale_kind != CPPMEGA_MI355_SCALE_PER_TOKEN && p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE) {
+    return false;
+  }
+  if (p.heads_per_group <= 32) return false;      // a single 32-head group gains nothing from sharing
+  if (p.topk < 1 || (size_t)p.B * p.S == 0) return false;
+  if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
+  if (p.kv_scale && ((uintptr_t)p.kv_scale & 3)) return false;
+  if ((unsigned long long)p.B * p.Skv * p.G >= 0x7fffffffull) return false;   // cache rows are counted in 32 bits
+  if (p.topk > 16 * kMaxKeys) return false;       // the combine step merges at most 16 key splits
+  return true;
+}
+
+void sparse_mla_latent_pc_plan(MlaParams& p) {
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
+  const long long base = (long long)p.B * p.S * p.G * chunks;
+  int splits = 1;
+  while (base * splits < 256 && p.topk / (splits * 2) >= 4 * kTK && splits < 16) splits *= 2;
+  while ((p.topk + splits - 1) / splits > kMaxKeys && splits < 16) splits *= 2;
+  p.heads_per_wg = kHeadsWg + 1;                  // (marks this kernel)
+  const int tiles = (p.topk + kTK - 1) / kTK;
+  const int tiles_per_split = (tiles + splits - 1) / splits;
+  p.num_splits = splits;
+  p.keys_per_split = tiles_per_split * kTK;
+}
+
+int sparse_mla_latent_pc_launch(const MlaParams& p, hipStream_t stream) {
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
+  const long long wgs = (long long)p.B * p.S * p.G * p.num_splits * chunks;
+  if (wgs > 0x7fffffffll || p.keys_per_split > kMaxKeys || p.num_splits > 16)
+    return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse MLA: launch too large");
+  const dim3 grid((unsigned)wgs), block(512);
+  const int nblk = p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK ? kLat / p.kv_scale_block : 1;
+#define CM_LAUNCH_PC(NB_)                                                                                          \
+  do {                                                                                                             \
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_pc_kernel<NB_>,                                 \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmem));                           \
+    hipLaunchKernelGGL((sparse_mla_latent_pc_kernel<NB_>), grid, block, kSmem, stream, p);                          \
+  } while (0)
+  if (nblk == 4) CM_LAUNCH_PC(4);
+  else if (nblk == 2) CM_LAUNCH_PC(2);
+  else CM_LAUNCH_PC(1);
+#undef CM_LAUNCH_PC
+  CM_HIP_CHECK(hipGetLastError());
+  if (p.num_splits > 1) return sparse_mla_latent_combine_launch(p, 2, stream);
+  return 0;
+}
+
+size_t sparse_mla_latent_pc_workspace_bytes(const MlaParams& p) {
+  if (p.num_splits <= 1) return 0;
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
+  const size_t blocks = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
+  return blocks * ((size_t)2 * kPartFloats * sizeof(unsigned short) + kHeadsWg * 2 * sizeof(float));
+}
+
+}  // namespace cm
