@@ -40,7 +40,6 @@ FILE_FLAGS: dict[str, list[str]] = {}
 # asynchronous loads by count, and spill traffic would be counted with them.
 NO_SCRATCH = {
     "sparse_mla_latent.hip": ("sparse_mla_latent_kernel",),
-    "sparse_mla_latent_pc.hip": ("sparse_mla_latent_pc_kernel",),
 }
 
 

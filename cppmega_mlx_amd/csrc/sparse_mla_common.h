@@ -26,7 +26,7 @@ struct MlaParams {
   int heads_per_group;
   int num_splits;       // split-KV factor of the MFMA kernel
   int keys_per_split;
-  int heads_per_wg;     // 0: 32-head tile kernel; 64 / 128: shared-tile latent kernel
+  int heads_per_wg;     // 0: 32-head tile kernel; 64: shared-tile latent kernel (sparse_mla_latent.hip)
   float sm_scale;
 };
 
@@ -57,11 +57,5 @@ bool sparse_mla_latent_supported(const MlaParams& p);
 void sparse_mla_latent_plan(MlaParams& p);
 int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream);   // includes its combine step
 size_t sparse_mla_latent_workspace_bytes(const MlaParams& p);
-
-// producer/consumer kernel for FP8 latent caches (sparse_mla_latent_pc.hip): 64 heads per workgroup
-bool sparse_mla_latent_pc_supported(const MlaParams& p);
-void sparse_mla_latent_pc_plan(MlaParams& p);
-int sparse_mla_latent_pc_launch(const MlaParams& p, hipStream_t stream);   // includes its combine step
-size_t sparse_mla_latent_pc_workspace_bytes(const MlaParams& p);
 
 }  // namespace cm

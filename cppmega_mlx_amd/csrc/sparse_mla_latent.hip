@@ -1,127 +1,192 @@
-// Sparse MLA forward over an FP8 latent KV cache on the matrix cores (gfx950):
-// 64 or 128 heads share every gathered key row.
+// Sparse MLA forward over an FP8 latent KV cache on the matrix cores (gfx950), with the
+// wavefronts of a workgroup split into score producers and value consumers.
 //
-// Shapes served: bf16 queries of 576 = 512 latent + 64 rope channels, d_v = 512,
-// keys as e4m3 latent [512] with fp32 scales (per 128 / 256 / 512 channels, or
-// per row, or none) plus a bf16 rope tail [64]; at least 33 heads per KV group.
+// Shapes served: bf16 queries of 576 = 512 latent + 64 rope channels, d_v = 512, keys as e4m3
+// latent [512] with fp32 scales (per 128 / 256 / 512 channels, per row, or none) plus a bf16
+// rope tail [64]; more than 32 heads per KV group.
 //
-// Workgroup = (query, KV group, chunk of 32*HG heads, key split), 4 wavefronts,
-// key tiles of 32 rows.
+// Workgroup = (query, KV group, chunk of 64 heads, key split), 8 wavefronts, key tiles of 32
+// rows in a ring of five LDS slots filled by the load unit (global_load_lds) three tiles ahead.
+// Two wavefronts share a SIMD: one producer and one consumer, so the matrix passes of one run
+// under the vector instructions of the other.
 //
-//   HBM -> LDS   Rows travel as raw bytes (e4m3 latent, bf16 rope, fp32 scales)
-//                straight into a ring of four LDS tile slots by the load unit
-//                (global_load_lds), three tiles ahead.  Nothing is ever
-//                rewritten in LDS: both matrix products dequantise in the
-//                operand path, in registers.  The 16-byte chunk c of row r lives
-//                at chunk c ^ (r & 7), which makes both access patterns below
-//                conflict-free; the swizzle costs nothing because each lane of
-//                a load instruction picks which source chunk it fetches.
-//   S^T = K.Q^T  Wavefront w owns 32 heads (their Q^T fragments stay in 144
-//                VGPRs) and HG/2 sub-tiles of 16 keys.  A K fragment is one
-//                16-byte LDS read of e4m3 bytes, converted to bf16 by
-//                v_cvt_scalef32_pk_bf16_fp8 with the power-of-two part of the
-//                block scale (exact); the mantissa part of the scale multiplies
-//                the fp32 partial sum of that 128-channel block.  The contraction
-//                order inside a 64-channel step is permuted (the same way for K
-//                and Q) so that one 16-byte read feeds two MFMA k-steps.
-//   softmax      base 2, running maximum per (wavefront, head) moved lazily.
-//                P is written to LDS as bf16 in the B-operand layout of the
-//                second product, once per scale block with V's block scale
-//                folded in (so V itself is converted unscaled, exactly).
-//   O^T += V^T.P^T  Wavefront w owns value channels 128w..128w+127 for all heads
-//                of the workgroup: V^T fragments are transposing 8-byte LDS reads
-//                (ds_read_b64_tr_b8) of the raw tile.  Accumulators are kept per
-//                producing wavefront (its running maximum is private), 256 AGPRs
-//                in all, so the key loop needs one barrier per tile and no
-//                agreement on maxima; the two accumulator sets of a head (HG = 2)
-//                are merged once at the end, in registers.
-//   pipeline     iteration t: barrier; issue tile t+3; QK + softmax of tile t+1;
-//                PV of tile t.
+//   producers (wavefronts 0..3): producer p owns heads 16p..16p+15 of the chunk.
+//     S^T = K.Q^T on v_mfma_scale_f32_16x16x128_f8f6f4: the key bytes are the A operand as they
+//     lie in the tile (no conversion instructions); the power-of-two part of a key's block scale
+//     is the operand exponent, the mantissa part multiplies the block's fp32 partial sum.  Q^T is
+//     split once per workgroup into two e4m3 planes hi + lo (hi + lo = the bf16 value, one
+//     exponent per head and 128 channels), kept in registers.  The rope tail is a bf16 product.
+//     Softmax in base 2 with a lazily moved private running maximum per head; P goes to LDS as
+//     bf16 in the B-operand layout of the value product, once per scale block with V's block
+//     scale folded in.
+//   consumers (wavefronts 4..7): consumer c owns value channels 128c..128c+127 (= scale block c
+//     when there are four) for all 64 heads: O^T += V^T.P^T on v_mfma_f32_32x32x16_bf16, V^T
+//     fragments by transposing LDS reads of the raw tile, converted unscaled (exactly).  They
+//     also issue the row loads.
+//   pipeline  iteration t: barrier; producers: scores and P of tile t+1; consumers: issue tile
+//             t+4, value product of tile t.  One barrier per tile.
 //
-// Key splits write their accumulators (rounded to bf16) to the workspace exactly as the lanes
-// hold them (512 B per store), plus (max, sum) per head; sparse_mla_latent_combine_kernel merges the
-// splits and does the transposition to [head][channel] that the single-split path does in LDS.
+// Key splits write their accumulators (rounded to bf16) to the workspace as the lanes hold them
+// plus (max, sum) per head; sparse_mla_latent_combine_kernel merges them and does the transposition
+// to [head][channel] that the single-split path does in LDS.
 
-#include <cstdlib>
+#include <type_traits>
 
 #include "sparse_mla_common.h"
 #include "mfma_util.h"
 
 namespace cm {
+
 namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kLat = 512;
 constexpr int kRope = 64;
 constexpr int kDqk = kLat + kRope;
 constexpr int kTK = 32;                         // keys per tile
-constexpr int kRing = 4;                        // tile slots
-constexpr int kLatBytes = kTK * kLat;           // 16384
-constexpr int kRopeBytes = kTK * kRope * 2;     // 4096
-constexpr int kScaleBytes = kTK * 4 * 4;        // 512: up to four fp32 scales per row
-constexpr int kSlotBytes = kLatBytes + kRopeBytes + kScaleBytes;   // 20992
-constexpr int kRingBytes = kRing * kSlotBytes;  // 83968
+constexpr int kRing = 5;                        // tile slots
+constexpr int kAhead = kRing - 1;               // tiles issued ahead of the value product
+// A tile slot holds the rows in matrix-operand order.  Latent: for sub-tile sj (16 keys) and
+// 128-channel block blk, two planes j of 64 lanes x 16 bytes: lane (key n = lane % 16, kg = lane / 16)
+// of plane j holds channels 128 blk + 32 kg + 16 j .. + 15 of key 16 sj + n.  A plane is what one
+// load instruction writes (the load unit stores lane after lane) and what one 16-byte-per-lane
+// LDS read of a K operand fetches, contiguously.  Plane 1 starts 128 bytes after the end of plane
+// 0, so that the two neighbouring chunks a V^T read takes from eight rows fall on different banks.
+// Rope: for sub-tile sj and 32-channel step s one plane: lane (n, kq) holds channels 32 s + 8 kq .. + 7.
+constexpr int kPlane = 1024 + 128;              // bytes from plane 0 to plane 1 of a pair
+constexpr int kPair = 2 * kPlane;               // one (sub-tile, block)
+constexpr int kLatBytes = 8 * kPair;            // 18432
+constexpr int kRopeBytes = 4 * 1024;            // [sj][s] planes
+constexpr int kScaleBytes = 2 * kTK * 4 * 4;    // up to four fp32 scales per row, twice: [row][block], then [block][row]
+constexpr int kScaleT = kTK * 4 * 4;            // offset of the [block][row] copy inside the scale area
+constexpr int kSlotBytes = kLatBytes + kRopeBytes + kScaleBytes;   // 23552
+constexpr int kRingBytes = kRing * kSlotBytes;  // 104960
 constexpr int kMaxKeys = 2048;                  // keys of one split (their rows are staged in LDS)
-constexpr int kKeyInts = kMaxKeys + 4 * kTK;    // + the tiles the pipeline prefetches past the end
+constexpr int kKeyInts = kMaxKeys + kTK;
+constexpr int kHeadsWg = 64;
 constexpr int kXPitch = 132;                    // floats per head row of the output transpose (128 + 4)
-constexpr int kPartFloats = 4 * 16 * 64 * 4;         // partial values (bf16) of one 32-head group: [4 wavefronts][16 rows][64 lanes][4]
+constexpr int kPartFloats = 4 * 16 * 64 * 4;    // partial values of one 32-head group: [4 consumers][16 rows][64 lanes][4]
 constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
 
-template <int HG>
-struct Geo {
-  static constexpr int kSpw = HG / 2;                       // 16-key sub-tiles per wavefront and tile
-  static constexpr int kSlots = 2 * HG;                     // (k-step, head group) pairs of a tile
-  static constexpr int kPBytes = 4 * kSlots * 1024;         // one parity: 4 scale variants
-  static constexpr int kPOff = kRingBytes;
-  static constexpr int kFacOff = kPOff + 2 * kPBytes;       // [parity][4 producers][32 heads] fp32
-  static constexpr int kFlagOff = kFacOff + 2 * 4 * 32 * 4; // [parity][4 producers] int
-  static constexpr int kStatOff = kFlagOff + 2 * 4 * 4;     // [4 producers][32 heads][2] fp32
-  static constexpr int kKeyOff = kStatOff + 4 * 32 * 2 * 4;
-  static constexpr int kSmem = kKeyOff + kKeyInts * 4;
-  static_assert(kSmem <= 160 * 1024, "LDS budget");
-  static_assert(4 * 32 * kXPitch * 4 <= kRingBytes, "the output transpose reuses the ring");
-};
+constexpr int kPBytes = 2 * 2 * 1024;           // P of one tile: [k-step][head block][64 lanes x 16 B]
+constexpr int kPOff = kRingBytes;
+constexpr int kFacOff = kPOff + 2 * kPBytes;        // [parity][4 producers][16 heads] fp32
+constexpr int kFlagOff = kFacOff + 2 * 4 * 16 * 4;  // [parity][4 producers] int
+constexpr int kStatOff = kFlagOff + 2 * 4 * 4;      // [4 producers][16 heads][2] fp32
+constexpr int kValidOff = kStatOff + 4 * 16 * 2 * 4;  // [tile] int: every key of the tile is valid
+constexpr int kKeyOff = kValidOff + (kMaxKeys / kTK) * 4;
+constexpr int kSmem = kKeyOff + kKeyInts * 4;
+static_assert(kSmem <= 160 * 1024, "LDS budget");
+static_assert(4 * 32 * kXPitch * 4 <= kRingBytes, "the output transpose reuses the ring");
 
-// 2^x by the hardware instruction alone (x <= ~8 here; tiny results may flush to zero)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ bf16x8 cvt8(unsigned w0, unsigned w1, float pow2_scale) {
-  const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, pow2_scale, false));
-  const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, pow2_scale, true));
-  const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, pow2_scale, false));
-  const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, pow2_scale, true));
+__device__ __forceinline__ bf16x8 cvt8(unsigned w0, unsigned w1) {
+  const unsigned o0 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, 1.0f, false));
+  const unsigned o1 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w0, 1.0f, true));
+  const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, false));
+  const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, true));
   return __builtin_bit_cast(bf16x8, make_uint4(o0, o1, o2, o3));
 }
 
-// scale = pow2 * mant: pow2 keeps the exponent field (what the converter applies, exactly),
-// mant the sign and mantissa.  A zero or denormal scale comes out as ~2^-127 (its products
-// vanish either way); inf / nan scales stay non-finite.
-__device__ __forceinline__ float scale_pow2(float s) { return __uint_as_float(__float_as_uint(s) & 0x7f800000u); }
+// sign and mantissa of a scale with the exponent of 1.0: scale = 2^(exponent field - 127) * this
 __device__ __forceinline__ float scale_mant(float s) {
   return __uint_as_float((__float_as_uint(s) & 0x807fffffu) | 0x3f800000u);
 }
 
-// The score product uses the compiler's own MFMA (this file is built with
-// -mllvm -amdgpu-mfma-vgpr-form, so its accumulators are ordinary VGPRs): the compiler then
-// knows the instruction's latency and pads its hazards exactly.  The value product keeps the
-// inline form: its 256 accumulator registers must be AGPRs.
+// 16 x 16 x 128 over e4m3 bytes, operands scaled by 2^(byte - 127): the byte is byte SEL of `a_exp`
+// for A and of `b_exp` for B, and must be the same in the four lanes of a row (l, l+16, ..).
+template <int SEL>
+__device__ __forceinline__ void mfma_s8(f32x4& acc, const i32x8& a, const i32x8& b, int a_exp, int b_exp) {
+  acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, SEL, a_exp, SEL, b_exp);
+}
 __device__ __forceinline__ void mfma_s(f32x4& acc, const bf16x8& a, const bf16x8& b) {
   acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
 }
+__device__ __forceinline__ void mfma_o(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
 
-// HG: 32-head groups per workgroup (2 or 4); NBLK: fp32 scales per key row (1, 2 or 4)
-template <int HG, int NBLK>
-__global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaParams p) {
-  using G_ = Geo<HG>;
-  constexpr int SPW = G_::kSpw;
+// 32 bf16 (four 16-byte pieces, channel order) of each lane -> e4m3 hi + e4m3 lo with hi + lo = x,
+// both in units of 2^(e - 127); returns e, common to lanes l, l^16, l^32, l^48 (one head's 128
+// channels).  hi carries the upper four significant bits of a bf16 value and lo the lower four, so
+// the pair is exact for every element within ~2^-14 of the largest of the 128 and off by less
+// than 2^-18 of that largest one otherwise.
+__device__ __forceinline__ int split_q32(const uint4 (&x)[4], i32x8& hi, i32x8& lo) {
+  u16x2 top = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned w[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2, w[d] & 0x7fff7fffu));
+  }
+  int amax_bits = max((int)top[0], (int)top[1]);             // bf16 bits of the largest magnitude
+  amax_bits = max(amax_bits, __float_as_int(xor16(__int_as_float(amax_bits))));
+  amax_bits = max(amax_bits, __float_as_int(xor32(__int_as_float(amax_bits))));
+  const int e = max((amax_bits >> 7) - 7, 1);                 // |x| / 2^(e-127) < 256
+  const float unit = __uint_as_float((unsigned)e << 23);
+  const i16x2 zero = {0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const unsigned w[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      const unsigned w0 = w[2 * d], w1 = w[2 * d + 1];
+      i16x2 h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(zero, __builtin_bit_cast(bf16x2, w0), unit, false);
+      h = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(h, __builtin_bit_cast(bf16x2, w1), unit, true);
+      const unsigned hw = __builtin_bit_cast(unsigned, h);
+      const f32x2 d0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(hw, unit, false);
+      const f32x2 d1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(hw, unit, true);
+      i16x2 l = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(zero, __uint_as_float(w0 << 16) - d0[0],
+                                                         __uint_as_float(w0 & 0xffff0000u) - d0[1], unit, false);
+      l = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(l, __uint_as_float(w1 << 16) - d1[0],
+                                                   __uint_as_float(w1 & 0xffff0000u) - d1[1], unit, true);
+      hi[2 * j + d] = (int)hw;
+      lo[2 * j + d] = __builtin_bit_cast(int, l);
+    }
+  }
+  return e;
+}
+
+// v_max_f32 as it is (fmaxf first passes every operand through a canonicalising max with itself).
+// Only for operands that ordinary vector instructions produced: never for matrix results, whose
+// read-after-write wait states the compiler pads only for instructions it can see.
+__device__ __forceinline__ float vmax(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// maximum over lanes l, l^16, l^32, l^48 (every lane gets it): a row swap leaves each value next
+// to its partner's
+__device__ __forceinline__ float max_rows(float v) {
+  unsigned u = __float_as_uint(v);
+  u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = vmax(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  u = __float_as_uint(v);
+  r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return vmax(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// NBLK: fp32 scales per key row (1, 2 or 4)
+template <int NBLK>
+__global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = (int)threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave < 4;
+  const int role = wave & 3;                    // producer p / consumer c
+  constexpr int nblk = NBLK;
 
   // ---- which (query, KV group, head chunk, split).  Workgroup ids that are equal modulo 8 run on
   //      the same XCD and share its L2: every workgroup of one (query, KV group) gets such ids, so
-  //      its query rows are fetched from HBM once (all key splits read them) and the head chunks
-  //      of a split find the gathered key rows of their sibling in cache ----
-  const int chunks = (p.heads_per_group + 32 * HG - 1) / (32 * HG);
+  //      the gathered key rows are fetched from HBM once for both head chunks and the query rows
+  //      once for all key splits ----
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
   const long long per_q = (long long)p.num_splits * chunks;    // workgroups of one (query, KV group)
   const long long nq = (long long)p.B * p.S * p.G;
   const long long nq8 = nq & ~7ll;
@@ -145,94 +210,67 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
   const int g = (int)(qg % p.G);
   const size_t bs = (size_t)(qg / p.G);           // b*S + s
   const int b = (int)(bs / p.S);
-  const int head0 = g * p.heads_per_group + chunk * 32 * HG;
-  const int heads_here = min(32 * HG, p.heads_per_group - chunk * 32 * HG);
+  const int head0 = g * p.heads_per_group + chunk * kHeadsWg;
+  const int heads_here = min(kHeadsWg, p.heads_per_group - chunk * kHeadsWg);
   const size_t idx_base = (bs * p.G + g) * (size_t)p.topk;
   const int key_begin = split * p.keys_per_split;
   const int key_end = min(p.topk, key_begin + p.keys_per_split);
   const int n_keys = max(0, key_end - key_begin);
-  const int list_tiles = (n_keys + kTK - 1) / kTK;   // tiles the index list spans; trailing all-skipped tiles are dropped below
+  const int list_tiles = (n_keys + kTK - 1) / kTK;
 
-  constexpr int nblk = NBLK;
   const bool has_scale = p.kv_scale_kind != CPPMEGA_MI355_SCALE_NONE;   // otherwise the scale area holds ones
 
-  // roles: this wavefront produces scores for head group hgq and sub-tiles sub0.., and
-  // accumulates value channels 128*wave.. for every head group
-  const int hgq = wave % HG;
-  const int sub0 = (wave / HG) * SPW;
+  int* keys = reinterpret_cast<int*>(smem + kKeyOff);
+  float* facbuf = reinterpret_cast<float*>(smem + kFacOff);
+  int* flagbuf = reinterpret_cast<int*>(smem + kFlagOff);
+  float* stats = reinterpret_cast<float*>(smem + kStatOff);
+  int* tvalid = reinterpret_cast<int*>(smem + kValidOff);
 
-  int* keys = reinterpret_cast<int*>(smem + G_::kKeyOff);
-  float* facbuf = reinterpret_cast<float*>(smem + G_::kFacOff);
-  int* flagbuf = reinterpret_cast<int*>(smem + G_::kFlagOff);
-  float* stats = reinterpret_cast<float*>(smem + G_::kStatOff);
-
-  // The first index entries are requested before the (much larger) query fragments: loads return
-  // in order, and the key rows can only be fetched once the indices are known.  Every load of
-  // this prologue is unconditional (positions and heads are clamped instead): only then can
-  // the compiler wait for the index words by count and leave the query loads in flight.
-  int early_lo[2], early_hi[2];
-  {
-    const bool wide = p.index_dtype == CPPMEGA_MI355_I64;
-    const int* words = (const int*)p.indices;
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const size_t at = idx_base + (size_t)min(key_begin + tid + 256 * e, p.topk - 1);
-      const size_t w0 = wide ? 2 * at : at;
-      early_lo[e] = words[w0];
-      early_hi[e] = words[w0 + (wide ? 1 : 0)];
-    }
-  }
-
-  // ---- Q^T fragments: lane (head n = lane%16, kq = lane/16), heads n and 16+n of group hgq.
-  //      latent step ks (64 channels): fragments 2ks, 2ks+1 hold channels 64ks + 16kq + {0..7}, {8..15};
-  //      rope step r: fragment 16+r holds channels 512 + 32r + 8kq + {0..7} ----
-  bf16x8 qf[2][18];
-  {
-    const int n = lane & 15, kq = lane >> 4;
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      const int h = 32 * hgq + hh * 16 + n;
-      // heads past the end of the group repeat head 0: their columns stay finite and are never stored
-      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (h < heads_here ? h : 0)) * (size_t)kDqk;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const uint4 t0 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq);
-        const uint4 t1 = *reinterpret_cast<const uint4*>(qrow + 64 * ks + 16 * kq + 8);
-        qf[hh][2 * ks] = __builtin_bit_cast(bf16x8, t0);
-        qf[hh][2 * ks + 1] = __builtin_bit_cast(bf16x8, t1);
-      }
-#pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        const uint4 t = *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kq);
-        qf[hh][16 + r] = __builtin_bit_cast(bf16x8, t);
-      }
-    }
+  if (!has_scale) {                               // no scales in memory: every slot's scale area is 1.0 for good
+    for (int i = tid; i < kRing * kTK; i += 512)
+      reinterpret_cast<float*>(smem + (i / kTK) * kSlotBytes + kLatBytes + kRopeBytes)[i % kTK] = 1.0f;
   }
   // ---- cache rows of this split's keys -> LDS (-1 = skipped) ----
-  int* last_valid = reinterpret_cast<int*>(smem);          // (ring memory, not yet in use)
-  if (tid == 0) *last_valid = -1;
-  __syncthreads();
+  int* last_valid = reinterpret_cast<int*>(stats);          // [8], one per wavefront (the statistics come much later)
+  // thread t takes list entries t, t + 512, ..: every index word is requested before the first one
+  // is looked at (one memory round trip), unconditionally, with positions clamped to the list.
+  // The producers put their query-row requests between the two halves: the load unit then
+  // moves the 74 KB of query rows while the index words are on their way, instead of in front of
+  // the first key tile.
+  constexpr int kRounds = kMaxKeys / 512;
+  const bool wide = p.index_dtype == CPPMEGA_MI355_I64;
+  int idx_lo[kRounds], idx_hi[kRounds];
   {
-    int mine = -1;
+    const int* words = (const int*)p.indices;
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int i = tid + 256 * e;
-      if (i < list_tiles * kTK + 4 * kTK) {
-        const long long k = p.index_dtype == CPPMEGA_MI355_I64
-                                ? (long long)(((unsigned long long)(unsigned)early_hi[e] << 32) | (unsigned)early_lo[e])
-                                : (long long)early_lo[e];
-        const bool ok = i < n_keys && k >= 0 && k < p.Skv;
-        keys[i] = ok ? (int)k : -1;
-        if (ok) mine = i;
+    for (int r = 0; r < kRounds; ++r) {
+      idx_lo[r] = 0; idx_hi[r] = 0;
+      if (r * 512 < list_tiles * kTK) {           // (uniform)
+        const size_t at = idx_base + (size_t)min(key_begin + tid + 512 * r, p.topk - 1);
+        const size_t w0 = wide ? 2 * at : at;
+        idx_lo[r] = words[w0];
+        idx_hi[r] = words[w0 + (wide ? 1 : 0)];
       }
     }
-    for (int i = tid + 512; i < list_tiles * kTK + 4 * kTK; i += 256) {
-      int row = -1;
-      if (i < n_keys) {
-        const long long k = load_index(p, idx_base + key_begin + i);
-        if (k >= 0 && k < p.Skv) { row = (int)k; mine = i; }
+  }
+  auto stage_keys = [&]() {
+    const int ctid = tid;
+    int* lo = idx_lo; int* hi = idx_hi;
+    int mine = -1;
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+      if (r * 512 < list_tiles * kTK) {
+        const int i = ctid + 512 * r;
+        const long long k = wide ? (long long)(((unsigned long long)(unsigned)hi[r] << 32) | (unsigned)lo[r]) : (long long)lo[r];
+        const bool ok = i < n_keys && k >= 0 && k < p.Skv;
+        int row = ok ? (int)k : -1;
+        if (i < list_tiles * kTK) keys[i] = row;
+        if (ok) mine = i;
+        // a tile is the 32 consecutive entries of half a wavefront; the masked-key path also serves a
+        // non-positive softmax scale (the plain path takes maxima before scaling)
+        const unsigned long long okm = __ballot(ok && p.sm_scale > 0.0f);
+        if ((lane & 31) == 0 && i < list_tiles * kTK) tvalid[i / kTK] = (unsigned)(okm >> (lane & 32)) == 0xffffffffu;
       }
-      keys[i] = row;
     }
     mine = max(mine, __shfl_xor(mine, 1, 64));
     mine = max(mine, __shfl_xor(mine, 2, 64));
@@ -240,417 +278,502 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
     mine = max(mine, __shfl_xor(mine, 8, 64));
     mine = max(mine, __shfl_xor(mine, 16, 64));
     mine = max(mine, __shfl_xor(mine, 32, 64));
-    if (lane == 0 && mine >= 0) atomicMax(last_valid, mine);
-  }
-
-  if (!has_scale) {                               // no scales in memory: every slot's scale area is 1.0 for good
-    for (int i = tid; i < kRing * kTK; i += 256)
-      reinterpret_cast<float*>(smem + (i / kTK) * kSlotBytes + kLatBytes + kRopeBytes)[i % kTK] = 1.0f;
-  }
-  __syncthreads();                                // keys[] is complete
+    if (lane == 0) last_valid[wave] = mine;
+  };
   // causal padding puts the skipped (-1) slots at the end of a list: tiles past the last valid key do nothing
-  const int n_tiles = __builtin_amdgcn_readfirstlane((*last_valid + kTK) / kTK);
-  __syncthreads();                                // everyone has read it before the ring is written
-
-  // ---- HBM -> LDS: this wavefront brings rows 8*wave .. 8*wave+7 of a tile.  A skipped key
-  //      fetches cache row 0 instead (its probability is zero), so every wavefront issues
-  //      the same number of loads for every tile and the in-order load counter can be
-  //      waited on by count. ----
-  // Row numbers fit 32 bits (checked on the host).  The loads are written as inline assembly:
-  // the compiler would otherwise order every later LDS read behind them (vmcnt(0)), which
-  // serialises the pipeline this kernel is built around.
-  //   latent : instruction i of wavefront w carries rows 8i+2w (lanes 0..31) and 8i+2w+1, so a
-  //            lane's swizzle term (row & 7) is the same for all i
-  //   rope   : one instruction, rows 8w + lane/8
-  //   scales : element 64w + lane of [32 rows][nblk]
-  const bool scale_op = has_scale && 64 * wave < kTK * nblk;
-  const size_t group_row0 = ((size_t)b * p.Skv) * p.G + g;     // cache row of key 0; key k is G rows further per step
-  const int lat_row = 2 * wave + (lane >> 5);                 // + 8i
-  const int rope_row = 8 * wave + (lane >> 3);
-  const int sc_elem = 64 * wave + lane;
-  const int sc_row = min(sc_elem / nblk, kTK - 1);
-  const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + (((lane & 31) ^ (lat_row & 7)) << 4);
-  const unsigned char* rope_src = (const unsigned char*)p.rope + group_row0 * (kRope * 2) + (((lane & 7) ^ (rope_row & 7)) << 4);
-  const unsigned char* sc_src = (const unsigned char*)p.kv_scale + (group_row0 * nblk + (unsigned)(sc_elem % nblk)) * 4;
-  const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = (unsigned)p.G * nblk * 4;
-  auto dma16 = [&](const unsigned char* src, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "memory", "m0");
+  auto count_tiles = [&]() {
+    int m = -1;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) m = max(m, last_valid[w]);
+    return __builtin_amdgcn_readfirstlane((m + kTK) / kTK);
   };
-  auto dma4 = [&](const unsigned char* src, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src) : "memory", "m0");
-  };
-  const unsigned smem_base = (unsigned)(size_t)(lds_void*)smem;                 // LDS byte address of the ring
-  auto issue_tile = [&](int tau) {
-    const unsigned slot = smem_base + (unsigned)(tau & (kRing - 1)) * kSlotBytes;
-    const int* tk = keys + tau * kTK;
-    int rows[6];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rows[i] = tk[8 * i + lat_row];
-    rows[4] = tk[rope_row];
-    rows[5] = scale_op ? tk[sc_row] : 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      dma16(lat_src + (size_t)(unsigned)max(rows[i], 0) * lat_step, slot + (8 * i + 2 * wave) * kLat);
-    dma16(rope_src + (size_t)(unsigned)max(rows[4], 0) * rope_step, slot + kLatBytes + 8 * wave * (kRope * 2));
-    if (scale_op) {
-      if (sc_elem < kTK * nblk)
-        dma4(sc_src + (size_t)(unsigned)max(rows[5], 0) * sc_step, slot + kLatBytes + kRopeBytes + 256 * wave);
-    }
-  };
-  auto wait_tiles_but_one = [&]() {               // everything but the most recently issued tile has landed
-    if (scale_op) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-  };
-
-  // ---- score side state ----
-  float m_run[2] = {-INFINITY, -INFINITY};        // base-2 running reference of heads n and 16+n
-  float l_run[2] = {0.0f, 0.0f};                  // this lane's share of the denominators
-  const float qk_scale = p.sm_scale * kLog2e;
-
-  // S^T of tile tau for this wavefront's head group and sub-tiles
-  auto qk_tile = [&](int tau, f32x4 (&st)[SPW][2]) {
-    const unsigned char* slot = smem + (tau & (kRing - 1)) * kSlotBytes;
-    const int m = lane & 15, kq = lane >> 4;
-#pragma unroll
-    for (int sj = 0; sj < SPW; ++sj) {
-      const int r = 16 * (sub0 + sj) + m;         // tile row of this lane's K fragment
-      const int r7 = r & 7;
-      const unsigned char* lat0 = slot + r * kLat + ((kq ^ r7) << 4);
-      const unsigned char* lat1 = slot + r * kLat + (((4 + kq) ^ r7) << 4);
-      const unsigned char* rope = slot + kLatBytes + r * (kRope * 2);
-      const float* scl = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + r * nblk;
-      // the power-of-two part of a key's scale goes into the conversion of its K fragment (this
-      // lane's row r); the mantissa part multiplies the partial sums, which this lane holds for
-      // keys 4*(lane/16) + i
-      const float* sclc = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * kq) * nblk;
-      auto load_k = [&](int ks) {                 // raw bytes of the 64-channel step ks
-        return *reinterpret_cast<const uint4*>(((ks & 1) ? lat1 : lat0) + 128 * (ks >> 1));
-      };
-      uint4 raw_a = load_k(0), raw_b = load_k(1);
-      float pw[4];
-      bool plain = true;                          // every scale of this row is a power of two
-#pragma unroll
-      for (int grp = 0; grp < 4; ++grp) {
-        const float sc = scl[(grp * nblk) >> 2];
-        pw[grp] = scale_pow2(sc);
-        plain = plain && (pw[grp] == sc);
-      }
-      const bool all_plain = __ballot(!plain) == 0ull;     // (uniform) no mantissa factors in this sub-tile
-      f32x4 tot0 = {0.f, 0.f, 0.f, 0.f}, tot1 = {0.f, 0.f, 0.f, 0.f};
-      f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
-      // software pipeline: step ks multiplies fragments converted during step ks-1 from bytes
-      // read during step ks-2
-      bf16x8 f0 = cvt8(raw_a.x, raw_a.y, pw[0]), f1 = cvt8(raw_a.z, raw_a.w, pw[0]);
-      bf16x8 rf0 = f0, rf1 = f0;                  // rope fragments (read during the last two steps)
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        uint4 raw_c = raw_b;
-        if (ks + 2 < 8) raw_c = load_k(ks + 2);
-        else if (ks == 6) rf0 = *reinterpret_cast<const bf16x8*>(rope + ((kq ^ r7) << 4));
-        else rf1 = *reinterpret_cast<const bf16x8*>(rope + (((4 + kq) ^ r7) << 4));
-        bf16x8 n0 = f0, n1 = f1;
-        if (ks + 1 < 8) {
-          n0 = cvt8(raw_b.x, raw_b.y, pw[(ks + 1) >> 1]);
-          n1 = cvt8(raw_b.z, raw_b.w, pw[(ks + 1) >> 1]);
-        }
-        mfma_s(a0, f0, qf[0][2 * ks]);
-        mfma_s(a1, f0, qf[1][2 * ks]);
-        mfma_s(a0, f1, qf[0][2 * ks + 1]);
-        mfma_s(a1, f1, qf[1][2 * ks + 1]);
-        // one LDS read, then MFMA and conversion pairs alternating
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-        }
-        if ((ks & 1) && !all_plain) {             // end of a 128-channel block: apply its mantissa factors
-          const int grp = ks >> 1;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float mant = scale_mant(sclc[i * nblk + ((grp * nblk) >> 2)]);
-            tot0[i] += mant * a0[i];
-            tot1[i] += mant * a1[i];
-            a0[i] = 0.0f;
-            a1[i] = 0.0f;
-          }
-        }
-        f0 = n0; f1 = n1;
-        raw_b = raw_c;
-      }
-      mfma_s(a0, rf0, qf[0][16]);
-      mfma_s(a1, rf0, qf[1][16]);
-      mfma_s(a0, rf1, qf[0][17]);
-      mfma_s(a1, rf1, qf[1][17]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        tot0[i] += a0[i];
-        tot1[i] += a1[i];
-      }
-      st[sj][0] = tot0;
-      st[sj][1] = tot1;
-    }
-  };
-
-  // ---- value side state: o[4*dvb + producer] = O^T[32 channels x 32 heads] ----
-  f32x16 o[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i)
-#pragma unroll
-    for (int j = 0; j < 16; ++j) o[i][j] = 0.0f;
-  const int pvar = (wave * nblk) >> 2;                         // scale block of channels 128*wave..
-  int pv_off[4];                                               // transposing-read offsets per 32-channel block
-  {
-    const int t = lane & 15, half = (lane >> 4) & 1, kq2 = lane >> 5;
-    const int r = 8 * kq2 + (t >> 1);                          // row within a 16-key step (r & 7 = t >> 1)
-#pragma unroll
-    for (int dvb = 0; dvb < 4; ++dvb) {
-      const int c = 8 * wave + 2 * dvb + half;                 // 16-byte chunk of the row
-      pv_off[dvb] = r * kLat + ((c ^ (r & 7)) << 4) + 8 * (t & 1);
-    }
-  }
-  // One pipeline stage: the value product of tile tv (8 steps of one V^T fragment and HG MFMAs)
-  // with the softmax of tile ts cut into pieces that run in the shadow of those MFMAs.
-  // do_s / do_v are uniform.
-  auto stage = [&](int tv, bool do_v, int ts, bool do_s) {
-    typedef __attribute__((ext_vector_type(2))) int i32x2;
-    const int n = lane & 15, gq = lane >> 4;
-    const unsigned char* vslot = smem + (tv & (kRing - 1)) * kSlotBytes;
-    const unsigned char* sslot = smem + (ts & (kRing - 1)) * kSlotBytes;
-    const int vpar = tv & 1, spar = ts & 1;
-    f32x4 st[SPW][2];
-    const unsigned char* pfrag = smem + G_::kPOff + vpar * G_::kPBytes + (pvar * G_::kSlots * 64 + lane) * 16;
-    unsigned char* pdst = smem + G_::kPOff + spar * G_::kPBytes;
-    float sv[SPW][2][4];
-    float pr[2][4];
-    float mx[2] = {-INFINITY, -INFINITY};
-    // V's block scales of this lane's keys (4gq + i of each sub-tile) and their validity: read once, up front
-    // (with two sub-tiles per wavefront there are no registers to spare: those read when needed)
-    constexpr bool kHoist = SPW == 1;
-    float vsc[SPW][4][nblk];
-    int4 kvalid[SPW];
-    auto read_scales = [&](int sj) {
-      const float* scl = reinterpret_cast<const float*>(sslot + kLatBytes + kRopeBytes) + (16 * (sub0 + sj) + 4 * gq) * nblk;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (nblk == 4) {
-          const float4 v4 = *reinterpret_cast<const float4*>(scl + 4 * i);
-          vsc[sj][i][0] = v4.x; vsc[sj][i][1 % nblk] = v4.y; vsc[sj][i][2 % nblk] = v4.z; vsc[sj][i][3 % nblk] = v4.w;
-        } else if (nblk == 2) {
-          const float2 v2 = *reinterpret_cast<const float2*>(scl + 2 * i);
-          vsc[sj][i][0] = v2.x; vsc[sj][i][1 % nblk] = v2.y;
-        } else {
-          vsc[sj][i][0] = scl[i];
-        }
-      }
-    };
-    if (do_v) {                                   // producers moved their reference: rescale (rare)
-      const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
-      if (__builtin_amdgcn_readfirstlane(fl.x | fl.y | fl.z | fl.w) != 0) {
-        mfma_settle_acc(o);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          // one accumulator block at a time: the values pass through ordinary VGPRs
-          const float fsc = facbuf[(vpar * 4 + (i & 3)) * 32 + (lane & 31)];
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int j = 0; j < 16; ++j) o[i][j] *= fsc;
-          asm volatile("" : "+a"(o[i]));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_settle_acc(o);
-      }
-    }
-    bf16x8 pb[HG];
-    i32x2 vraw = {0, 0};
-    auto load_v = [&](int i) {                    // V^T fragment of step i = (k-step i/4, channel block i%4)
-      return __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (__attribute__((address_space(3))) i32x2*)(vslot + 16 * (i >> 2) * kLat + pv_off[i & 3]));
-    };
-    auto load_p = [&](int kstep) {
-#pragma unroll
-      for (int hg = 0; hg < HG; ++hg) pb[hg] = *reinterpret_cast<const bf16x8*>(pfrag + (kstep * HG + hg) * 1024);
-    };
-    auto probs = [&](int sj) {                    // pr = exp2(score - reference), denominators
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pr[hh][i] = (sv[sj][hh][i] == -INFINITY) ? 0.0f : fast_exp2(sv[sj][hh][i] - m_run[hh]);
-          l_run[hh] += pr[hh][i];
-        }
-    };
-    // P (x V's block scale) -> LDS in the B-operand layout of the 32x32x16 product: lane
-    // (head, key/8) owns 16 bytes = 8 keys; this lane holds keys 4gq..4gq+3 of sub-tile sj
-    auto write_p = [&](int sj, int v0, int v1) {
-      const int slot_id = (sub0 + sj) * HG + hgq;
-#pragma unroll
-      for (int v = v0; v < v1; ++v) {
-        if (v >= nblk) break;
-        float sc[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) sc[i] = vsc[sj][i][v % nblk];
-        unsigned char* dst = pdst + ((v * G_::kSlots + slot_id) * 64 + (gq >> 1) * 32) * 16 + (gq & 1) * 8;
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          const uint2 w = make_uint2(pack_bf16(pr[hh][0] * sc[0], pr[hh][1] * sc[1]),
-                                     pack_bf16(pr[hh][2] * sc[2], pr[hh][3] * sc[3]));
-          *reinterpret_cast<uint2*>(dst + (hh * 16 + n) * 16) = w;
-        }
-      }
-    };
-    auto softmax_piece = [&](int i) {
-      if (i == 0) {                               // mask, scale, local maxima
-#pragma unroll
-        for (int sj = 0; sj < SPW; ++sj) {
-          const int4 kk = kHoist ? kvalid[sj] : *reinterpret_cast<const int4*>(keys + ts * kTK + 16 * (sub0 + sj) + 4 * gq);
-          const bool ok[4] = {kk.x >= 0, kk.y >= 0, kk.z >= 0, kk.w >= 0};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            sv[sj][0][e] = ok[e] ? st[sj][0][e] * qk_scale : -INFINITY;
-            sv[sj][1][e] = ok[e] ? st[sj][1][e] * qk_scale : -INFINITY;
-            mx[0] = fmaxf(mx[0], sv[sj][0][e]);
-            mx[1] = fmaxf(mx[1], sv[sj][1][e]);
-          }
-        }
-      } else if (i == 1) {                        // maxima across the four key quarters; lazy reference
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          mx[hh] = fmaxf(mx[hh], xor16(mx[hh]));
-          mx[hh] = fmaxf(mx[hh], xor32(mx[hh]));
-        }
-        const bool grow = (mx[0] > m_run[0] + kLazy) || (mx[1] > m_run[1] + kLazy);
-        const bool any_grow = __ballot(grow) != 0ull;
-        // accumulators of a head whose reference was -inf are still zero: nothing to rescale
-        const bool rescale = (mx[0] > m_run[0] + kLazy && m_run[0] != -INFINITY) || (mx[1] > m_run[1] + kLazy && m_run[1] != -INFINITY);
-        const bool any_rescale = __ballot(rescale) != 0ull;
-        if (any_grow) {                           // consumers rescale their accumulators by fac first
-          float fac[2];
-#pragma unroll
-          for (int hh = 0; hh < 2; ++hh) {
-            const float m_new = (mx[hh] > m_run[hh] + kLazy) ? mx[hh] : m_run[hh];
-            fac[hh] = (m_run[hh] == -INFINITY) ? 1.0f : exp2f(m_run[hh] - m_new);
-            l_run[hh] *= fac[hh];
-            m_run[hh] = m_new;
-          }
-          if (any_rescale && lane < 16) {
-            facbuf[(spar * 4 + wave) * 32 + n] = fac[0];
-            facbuf[(spar * 4 + wave) * 32 + 16 + n] = fac[1];
-          }
-        }
-        if (!any_rescale && lane < 32) facbuf[(spar * 4 + wave) * 32 + lane] = 1.0f;
-        if (lane == 0) flagbuf[spar * 4 + wave] = any_rescale ? 1 : 0;
-      } else if (i == 2) {
-        if (!kHoist) read_scales(0);
-        probs(0);
-      } else if (i == 3) {
-        write_p(0, 0, 2);
-      } else if (i == 4) {
-        write_p(0, 2, 4);
-      } else if (SPW == 2) {
-        if (i == 5) { read_scales(1); probs(1); }
-        else if (i == 6) write_p(1, 0, 2);
-        else write_p(1, 2, 4);
-      }
-    };
-    if (do_s) qk_tile(ts, st);
-    __builtin_amdgcn_sched_barrier(0);
-    if (do_s && kHoist) {
-#pragma unroll
-      for (int sj = 0; sj < SPW; ++sj) {
-        kvalid[sj] = *reinterpret_cast<const int4*>(keys + ts * kTK + 16 * (sub0 + sj) + 4 * gq);
-        read_scales(sj);
-      }
-    }
-    if (do_v) {
-      load_p(0);
-      vraw = load_v(0);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_barrier(0);
-      i32x2 vnext = vraw;
-      if (do_v && i < 7) vnext = load_v(i + 1);
-      if (do_s) softmax_piece(i);
-      if (do_v) {
-        const bf16x8 a = cvt8((unsigned)vraw[0], (unsigned)vraw[1], 1.0f);
-        const int kstep = i >> 2, dvb = i & 3;
-#pragma unroll
-        for (int hg = 0; hg < HG; ++hg) {
-          const int prod = HG == 4 ? hg : hg + 2 * kstep;      // the wavefront that produced this P
-          mfma_pv(o[4 * dvb + prod], a, pb[hg]);
-        }
-        if (i == 3) load_p(1);
-      }
-      vraw = vnext;
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  // ---- pipeline ----
-  issue_tile(0);
-  issue_tile(1);
-  issue_tile(2);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  stage(0, false, 0, true);
-  for (int t = 0; t < n_tiles; ++t) {
-    wait_tiles_but_one();                         // tile t+1 (issued two iterations ago) has landed
-    __syncthreads();                              // ... for every wavefront; P(t) is complete; PV(t-1) is done
-    issue_tile(t + 3);                            // into the slot of tile t-1
-    __builtin_amdgcn_sched_barrier(0);
-    stage(t, true, t + 1, t + 1 < n_tiles);
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the prefetches past the end
-  mfma_settle_acc(o);
-
-  // ---- epilogue ----
-#pragma unroll
-  for (int hh = 0; hh < 2; ++hh) {                // a head's denominator is spread over lanes n, n+16, n+32, n+48
-    l_run[hh] += xor16(l_run[hh]);
-    l_run[hh] += xor32(l_run[hh]);
-  }
-  if (lane < 16) {
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      stats[(wave * 32 + hh * 16 + lane) * 2 + 0] = m_run[hh];
-      stats[(wave * 32 + hh * 16 + lane) * 2 + 1] = l_run[hh];
-    }
-  }
-  __syncthreads();                                // statistics are visible; the ring is free
-
-  const int hd = lane & 31, gq2 = lane >> 5;
-  const bool direct = p.num_splits == 1;
-  float* xbuf = reinterpret_cast<float*>(smem) + wave * 32 * kXPitch;     // private to this wavefront
   const size_t q_index = bs;
   // key-split partials: one block per (query, KV group, head chunk, split)
   const size_t part_block = (size_t)(((long long)bs * p.G + g) * chunks + chunk) * p.num_splits + split;
   const size_t part_blocks_total = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
+
+  if (producer) {
+    // =====================================================================================
+    // producer p = role: heads 16p .. 16p+15 of the chunk
+    // =====================================================================================
+    const int n = lane & 15, kg = lane >> 4;
+    // Q^T operands: lane (head n, kg) holds channels 128 blk + 32 kg .. +31 of the latent and
+    // channels 512 + 32 r + 8 kg .. +7 of the rope tail
+    uint4 qraw[4][4];
+    bf16x8 qr[2];
+    {
+      const int h = 16 * role + n;
+      // heads past the end of the group repeat head 0: their columns stay finite and are never stored
+      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (h < heads_here ? h : 0)) * (size_t)kDqk;
 #pragma unroll
-  for (int hg = 0; hg < HG; ++hg) {
-    float m_all, l_all;
-    if (HG == 4) {
-      m_all = stats[(hg * 32 + hd) * 2];
-      l_all = stats[(hg * 32 + hd) * 2 + 1];
-    } else {                                      // two producers per head group: hg and hg + 2
-      const float ma = stats[(hg * 32 + hd) * 2], la = stats[(hg * 32 + hd) * 2 + 1];
-      const float mb = stats[((hg + 2) * 32 + hd) * 2], lb = stats[((hg + 2) * 32 + hd) * 2 + 1];
-      m_all = fmaxf(ma, mb);
-      const float fa = (ma == -INFINITY) ? 0.0f : exp2f(ma - m_all);
-      const float fb = (mb == -INFINITY) ? 0.0f : exp2f(mb - m_all);
-      l_all = la * fa + lb * fb;
+      for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
-      for (int dvb = 0; dvb < 4; ++dvb) {
-        __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < 4; ++j) qraw[blk][j] = *reinterpret_cast<const uint4*>(qrow + 128 * blk + 32 * kg + 8 * j);
 #pragma unroll
-        for (int j = 0; j < 16; ++j) o[4 * dvb + hg][j] = o[4 * dvb + hg][j] * fa + o[4 * dvb + hg + 2][j] * fb;
-        asm volatile("" : "+a"(o[4 * dvb + hg]));
+      for (int r = 0; r < 2; ++r) qr[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kg));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    stage_keys();
+    __syncthreads();                                // keys[] is complete
+    const int n_tiles = count_tiles();
+    i32x8 qh[4], ql[4];
+    int qexp = 0;
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) qexp |= split_q32(qraw[blk], qh[blk], ql[blk]) << (8 * blk);
+    float m_run = -INFINITY;                      // base-2 running reference of head n
+    float l_run = 0.0f;                           // this lane's share of its denominator
+    const float qk_scale = p.sm_scale * kLog2e;
+
+    // K operands of a tile -> registers: per sub-tile four 32-byte block fragments, two rope
+    // fragments and the scales of this lane's key row (they give the operand exponents).  They are
+    // requested one tile ahead, right after the previous tile's products, so that they land
+    // under its softmax.
+    i32x8 kf[2][4];
+    bf16x8 rf[2][2];
+    float own[2][nblk];
+    auto load_k = [&](int tau) {
+      const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
+      const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        const float* scl = scl_base + (16 * sj + n) * nblk;
+        if (nblk == 4) {
+          const float4 o4 = *reinterpret_cast<const float4*>(scl);
+          own[sj][0] = o4.x; own[sj][1 % nblk] = o4.y; own[sj][2 % nblk] = o4.z; own[sj][3 % nblk] = o4.w;
+        } else if (nblk == 2) {
+          const float2 o2 = *reinterpret_cast<const float2*>(scl);
+          own[sj][0] = o2.x; own[sj][1 % nblk] = o2.y;
+        } else {
+          own[sj][0] = scl[0];
+        }
+      }
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        // the lane's 32 bytes of a block are its 16 bytes of the block's two planes
+        const unsigned char* lat = slot + sj * (4 * kPair) + lane * 16;
+        const unsigned char* rope = slot + kLatBytes + sj * 2048 + lane * 16;
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+          const uint4 c0 = *reinterpret_cast<const uint4*>(lat + blk * kPair);
+          const uint4 c1 = *reinterpret_cast<const uint4*>(lat + blk * kPair + kPlane);
+          kf[sj][blk] = i32x8{(int)c0.x, (int)c0.y, (int)c0.z, (int)c0.w, (int)c1.x, (int)c1.y, (int)c1.z, (int)c1.w};
+        }
+        rf[sj][0] = *reinterpret_cast<const bf16x8*>(rope);
+        rf[sj][1] = *reinterpret_cast<const bf16x8*>(rope + 1024);
+      }
+    };
+
+    // scores and probabilities of tile tau (whose K operands are in registers) -> P(tau) in LDS;
+    // `next`: tile tau+1 exists (it has landed)
+    auto produce = [&](int tau, bool next) {
+      const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
+      const int spar = tau & 1;
+      const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
+      const bool all_valid = tvalid[tau] != 0;      // (uniform) no skipped key in this tile
+      int4 kk[2] = {make_int4(0, 0, 0, 0), make_int4(0, 0, 0, 0)};
+      if (!all_valid) {
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) kk[sj] = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * sj + 4 * kg);
       }
       __builtin_amdgcn_sched_barrier(0);
+      // exponent bytes of this lane's key rows, and whether any row of the tile has a mantissa part
+      int kexp[2];
+      bool plain = true;
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        kexp[sj] = 0;
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+          const unsigned sc = __float_as_uint(own[sj][(blk * nblk) >> 2]);
+          kexp[sj] |= (int)(((sc >> 23) & 0xffu) << (8 * blk));
+          plain = plain && ((sc & 0x807fffffu) == 0u);
+        }
+      }
+      const bool all_plain = __ballot(!plain) == 0ull;       // (uniform)
+      float ksc[2][4][nblk];                        // scales of keys 16 sj + 4 kg + i: their mantissa parts multiply the partial sums
+      if (!all_plain) {
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          const float* sclc = scl_base + (16 * sj + 4 * kg) * nblk;
+          if (nblk == 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float4 v4 = *reinterpret_cast<const float4*>(sclc + 4 * i);
+              ksc[sj][i][0] = v4.x; ksc[sj][i][1 % nblk] = v4.y; ksc[sj][i][2 % nblk] = v4.z; ksc[sj][i][3 % nblk] = v4.w;
+            }
+          } else if (nblk == 2) {
+            const float4 a = *reinterpret_cast<const float4*>(sclc), bq = *reinterpret_cast<const float4*>(sclc + 4);
+            ksc[sj][0][0] = a.x; ksc[sj][0][1 % nblk] = a.y; ksc[sj][1][0] = a.z; ksc[sj][1][1 % nblk] = a.w;
+            ksc[sj][2][0] = bq.x; ksc[sj][2][1 % nblk] = bq.y; ksc[sj][3][0] = bq.z; ksc[sj][3][1 % nblk] = bq.w;
+          } else {
+            const float4 a = *reinterpret_cast<const float4*>(sclc);
+            ksc[sj][0][0] = a.x; ksc[sj][1][0] = a.y; ksc[sj][2][0] = a.z; ksc[sj][3][0] = a.w;
+          }
+        }
+      }
+      f32x4 st[2];
+      st[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+      st[1] = st[0];
+      if (all_plain) {
+        // one sub-tile after the other: the second one's operands are still landing
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          mfma_s8<0>(st[sj], kf[sj][0], qh[0], kexp[sj], qexp);
+          mfma_s8<0>(st[sj], kf[sj][0], ql[0], kexp[sj], qexp);
+          mfma_s8<1>(st[sj], kf[sj][1], qh[1], kexp[sj], qexp);
+          mfma_s8<1>(st[sj], kf[sj][1], ql[1], kexp[sj], qexp);
+          mfma_s8<2>(st[sj], kf[sj][2], qh[2], kexp[sj], qexp);
+          mfma_s8<2>(st[sj], kf[sj][2], ql[2], kexp[sj], qexp);
+          mfma_s8<3>(st[sj], kf[sj][3], qh[3], kexp[sj], qexp);
+          mfma_s8<3>(st[sj], kf[sj][3], ql[3], kexp[sj], qexp);
+          mfma_s(st[sj], rf[sj][0], qr[0]);
+          mfma_s(st[sj], rf[sj][1], qr[1]);
+        }
+      } else {
+        // each block is accumulated apart and enters the score times its keys' mantissa factors; the
+        // two sub-tiles alternate so that a block's factors are applied under the other's products
+        auto block = [&](auto blk_c) {
+          constexpr int blk = decltype(blk_c)::value;
+          f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0;
+          mfma_s8<blk>(a0, kf[0][blk], qh[blk], kexp[0], qexp);
+          mfma_s8<blk>(a1, kf[1][blk], qh[blk], kexp[1], qexp);
+          mfma_s8<blk>(a0, kf[0][blk], ql[blk], kexp[0], qexp);
+          mfma_s8<blk>(a1, kf[1][blk], ql[blk], kexp[1], qexp);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            st[0][i] += scale_mant(ksc[0][i][(blk * nblk) >> 2]) * a0[i];
+            st[1][i] += scale_mant(ksc[1][i][(blk * nblk) >> 2]) * a1[i];
+          }
+        };
+        block(std::integral_constant<int, 0>{});
+        block(std::integral_constant<int, 1>{});
+        block(std::integral_constant<int, 2>{});
+        block(std::integral_constant<int, 3>{});
+        mfma_s(st[0], rf[0][0], qr[0]);
+        mfma_s(st[1], rf[1][0], qr[0]);
+        mfma_s(st[0], rf[0][1], qr[1]);
+        mfma_s(st[1], rf[1][1], qr[1]);
+      }
+
+      __builtin_amdgcn_sched_barrier(0);
+      // The scale reads issued before the products have long landed: say so before the next batch of
+      // reads.  (The LDS counter holds 15 at most; without this the compiler, unable to name "all
+      // but the last 22", makes the first use of a scale wait for most of that batch.)
+      __builtin_amdgcn_s_waitcnt(0xc07f);           // lgkmcnt(0)
+      if (next) load_k(tau + 1);                    // (the fragment registers are free again)
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- softmax: this lane holds head n, keys 16 sj + 4 kg + i ----
+      float mx;
+      float mul = qk_scale;                         // what turns a held sum into a base-2 score
+      if (all_valid) {
+        // no skipped key: the maximum is taken on the raw sums (qk_scale > 0 on this path)
+        // (fmaxf, not the raw instruction: the compiler pads the wait states a vector instruction
+        // needs before it may read matrix results only for instructions it can see)
+        mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
+                   fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
+      } else {
+        mx = -INFINITY;
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) {
+          const bool ok[4] = {kk[sj].x >= 0, kk[sj].y >= 0, kk[sj].z >= 0, kk[sj].w >= 0};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            st[sj][e] = ok[e] ? st[sj][e] * qk_scale : -INFINITY;
+            mx = fmaxf(mx, st[sj][e]);
+          }
+        }
+        mul = 1.0f;
+      }
+      mx = max_rows(mx) * mul;                 // over the four key quarters (lanes n, n+16, n+32, n+48)
+      {
+        const bool grow = mx > m_run + kLazy;
+        // accumulators of a head whose reference was -inf are still zero: nothing to rescale
+        const bool rescale = grow && m_run != -INFINITY;
+        const bool any_rescale = __ballot(rescale) != 0ull;
+        float fac = 1.0f;
+        if (grow) {
+          fac = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - mx);
+          l_run *= fac;
+          m_run = mx;
+        }
+        if (any_rescale && lane < 16) facbuf[(spar * 4 + role) * 16 + n] = fac;
+        if (lane == 0) flagbuf[spar * 4 + role] = any_rescale ? 1 : 0;
+      }
+      // exp2(-inf - m) is 0 for a finite m; a head with no valid key yet keeps m_run = -inf
+      const float neg_m = -vmax(m_run, -1.0e30f);
+      unsigned char* pdst = smem + kPOff + spar * kPBytes;
+#pragma unroll
+      for (int sj = 0; sj < 2; ++sj) {
+        float pr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pr[i] = fast_exp2(__builtin_fmaf(st[sj][i], mul, neg_m));
+          l_run += pr[i];
+        }
+        // P -> LDS in the B-operand layout of the 32x32x16 product: lane (head of a 32-head block,
+        // key/8) owns 16 bytes = 8 keys; this lane holds keys 4kg..4kg+3.  (V's block scales are
+        // applied by the consumers, each for its own channel block.)
+        unsigned char* dst = pdst + ((sj * 2 + (role >> 1)) * 64 + (role & 1) * 16 + n + (kg >> 1) * 32) * 16 + (kg & 1) * 8;
+        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(pr[0], pr[1]), pack_bf16(pr[2], pr[3]));
+      }
+    };
+
+    // t = -1: [X] tile 0 has landed.  t >= 0: [B_t] tile t+2 has landed, P(t) is complete, the value
+    // product of tile t-1 is done.
+    for (int t = -1; t < n_tiles; ++t) {
+      __syncthreads();
+      // (the first barrier only promises tile 0: tile 1's operands are read a round late, once)
+      if (t <= 0 && t + 1 < n_tiles) load_k(t + 1);
+      if (t + 1 < n_tiles) produce(t + 1, t >= 0 && t + 2 < n_tiles);
     }
-    const int h_local = 32 * hg + hd;
+    l_run += xor16(l_run);
+    l_run += xor32(l_run);
+    if (lane < 16) {
+      stats[(role * 16 + lane) * 2 + 0] = m_run;
+      stats[(role * 16 + lane) * 2 + 1] = l_run;
+    }
+    __syncthreads();                              // [E] statistics are visible; the ring is free
+    return;
+  }
+
+  // =======================================================================================
+  // consumer c = role: value channels 128c .. 128c+127 of all 64 heads; also the row loads
+  // =======================================================================================
+  stage_keys();
+  __syncthreads();                                // keys[] is complete
+  const int n_tiles = count_tiles();
+  // HBM -> LDS: this wavefront brings rows 8c .. 8c+7 of a tile.  A skipped key fetches cache
+  // row 0 instead (its probability is zero), so every tile is the same number of load
+  // instructions and the in-order load counter can be waited on by count.  The loads are inline
+  // assembly: the compiler would otherwise order every later LDS read behind them.
+  //   latent : block c of both sub-tiles, two planes each: lane (n, kg) of plane j fetches bytes
+  //            128 c + 32 kg + 16 j .. + 15 of key 16 sj + n
+  //   rope   : plane (sj = c / 2, s = c % 2): lane (n, kq) fetches bytes 64 s + 16 kq .. + 15 of the rope row
+  //   scales : element 64c + lane of [32 rows][nblk]
+  //   scales, transposed : (nblk > 1) the wavefronts after those: element 64 (c - nblk/2) + lane of [nblk][32 rows]
+  const bool scale_op = has_scale && 64 * role < kTK * nblk;
+  const bool tr_op = has_scale && nblk > 1 && !scale_op && 64 * (role - nblk / 2) < kTK * nblk;
+  const int tr_elem = 64 * (role - nblk / 2) + lane;          // (block, row) = (tr_elem / 32, tr_elem % 32)
+  const size_t group_row0 = ((size_t)b * p.Skv) * p.G + g;     // cache row of key 0; key k is G rows further per step
+  const int sc_elem = 64 * role + lane;
+  const int sc_row = min(sc_elem / nblk, kTK - 1);
+  const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + 128 * role + 32 * (lane >> 4);
+  const unsigned char* rope_src = (const unsigned char*)p.rope + group_row0 * (kRope * 2) + 64 * (role & 1) + 16 * (lane >> 4);
+  const unsigned char* sc_src = (const unsigned char*)p.kv_scale +
+                                (group_row0 * nblk + (unsigned)(tr_op ? (tr_elem >> 5) & (nblk - 1) : sc_elem % nblk)) * 4;
+  const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = (unsigned)p.G * nblk * 4;
+  auto dma16 = [&](const unsigned char* src, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+  };
+  auto dma4 = [&](const unsigned char* src, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+  };
+  const unsigned smem_base = (unsigned)(size_t)(lds_void*)smem;                 // LDS byte address of the ring
+  // one tile is six load instructions (five without a scale instruction): prepare computes the
+  // row numbers, part(i) issues instruction i.  The value product spreads the parts between its
+  // matrix instructions: issuing blocks while the load unit's queue is full.
+  unsigned dma_slot = 0;
+  size_t dma_r0 = 0, dma_r1 = 0, dma_rs = 0;
+  auto dma_prepare = [&](int tau) {
+    dma_slot = smem_base + (unsigned)(tau % kRing) * kSlotBytes;
+    const int* tk = keys + tau * kTK;
+    const int k0 = tk[lane & 15], k1 = tk[16 + (lane & 15)];        // this lane's key of sub-tile 0 / 1
+    const int ksc_row = scale_op ? tk[sc_row] : tr_op ? tk[tr_elem & 31] : 0;
+    dma_r0 = (size_t)(unsigned)max(k0, 0);
+    dma_r1 = (size_t)(unsigned)max(k1, 0);
+    dma_rs = (size_t)(unsigned)max(ksc_row, 0);
+  };
+  auto dma_part = [&](int i) {
+    if (i == 0) dma16(lat_src + dma_r0 * lat_step, dma_slot + role * kPair);
+    else if (i == 1) dma16(lat_src + dma_r0 * lat_step + 16, dma_slot + role * kPair + kPlane);
+    else if (i == 2) dma16(lat_src + dma_r1 * lat_step, dma_slot + (4 + role) * kPair);
+    else if (i == 3) dma16(lat_src + dma_r1 * lat_step + 16, dma_slot + (4 + role) * kPair + kPlane);
+    else if (i == 4) dma16(rope_src + ((role >> 1) ? dma_r1 : dma_r0) * rope_step, dma_slot + kLatBytes + role * 1024);
+    else if (scale_op) {
+      if (sc_elem < kTK * nblk) dma4(sc_src + dma_rs * sc_step, dma_slot + kLatBytes + kRopeBytes + 256 * role);
+    } else if (tr_op) {
+      dma4(sc_src + dma_rs * sc_step, dma_slot + kLatBytes + kRopeBytes + kScaleT + 256 * (role - nblk / 2));
+    }
+  };
+  auto issue_tile = [&](int tau) {
+    dma_prepare(tau);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) dma_part(i);
+  };
+  // wait until at most `tiles` of the most recently issued tiles are still in flight
+  auto wait_outstanding = [&](int tiles) {
+    const int per = (scale_op || tr_op) ? 6 : 5;
+    switch (min(tiles, 5) * per) {
+      case 30: asm volatile("s_waitcnt vmcnt(30)" ::: "memory"); break;
+      case 25: asm volatile("s_waitcnt vmcnt(25)" ::: "memory"); break;
+      case 24: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+      case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+      case 18: asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); break;
+      case 15: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
+      case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+  };
+
+  // ---- value side state: o[dvb][hb] = O^T[32 channels x 32 heads] ----
+  f32x16 o[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) o[i][hb][j] = 0.0f;
+  const int pvar = (role * nblk) >> 2;                         // scale block of channels 128c..
+  int pv_off[4];                                               // transposing-read offsets per 32-channel block
+  {
+    // lanes t = 0..15 of a group read 8 bytes each from eight consecutive keys' 16-byte pieces (128
+    // contiguous bytes); half selects the plane, kq2 the upper eight keys of the step
+    const int t = lane & 15, half = (lane >> 4) & 1, kq2 = lane >> 5;
+    const int r = 8 * kq2 + (t >> 1);                          // key within the 16-key step
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) pv_off[dvb] = role * kPair + half * kPlane + (dvb * 16 + r) * 16 + 8 * (t & 1);
+  }
+  // V^T fragments of one 16-key step (four 32-channel blocks), raw
+  auto load_v = [&](int tau, int kstep, i32x2 (&vr)[4]) {
+    const unsigned char* vslot = smem + (tau % kRing) * kSlotBytes + kstep * (4 * kPair);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb)
+      vr[dvb] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(vslot + pv_off[dvb]));
+  };
+  i32x2 v0[4];                                    // first step of the tile about to be consumed (read ahead of the barrier)
+  // value product of tile tv; `next`: tile tv+1 exists (it has landed: the producers are reading it)
+  auto consume = [&](int tv, bool next, bool dma) {
+    const int vpar = tv & 1;
+    if (dma) dma_prepare(tv + kAhead);
+    const unsigned char* pfrag = smem + kPOff + vpar * kPBytes + lane * 16;
+    bf16x8 pb[2][2];
+#pragma unroll
+    for (int kstep = 0; kstep < 2; ++kstep)
+#pragma unroll
+      for (int hb = 0; hb < 2; ++hb) pb[kstep][hb] = *reinterpret_cast<const bf16x8*>(pfrag + (kstep * 2 + hb) * 1024);
+    // V's scales of this wavefront's channel block for the lane's eight keys of each step
+    float4 vs[2][2];
+    if (has_scale) {
+      const float* tr = reinterpret_cast<const float*>(smem + (tv % kRing) * kSlotBytes + kLatBytes + kRopeBytes + (nblk > 1 ? kScaleT : 0)) +
+                        pvar * kTK + 8 * (lane >> 5);
+#pragma unroll
+      for (int kstep = 0; kstep < 2; ++kstep) {
+        vs[kstep][0] = *reinterpret_cast<const float4*>(tr + 16 * kstep);
+        vs[kstep][1] = *reinterpret_cast<const float4*>(tr + 16 * kstep + 4);
+      }
+    }
+    const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
+    i32x2 v1[4];
+    load_v(tv, 1, v1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (__builtin_amdgcn_readfirstlane(fl.x | fl.y | fl.z | fl.w) != 0) {      // producers moved a reference: rescale (rare)
+#pragma unroll
+      for (int hb = 0; hb < 2; ++hb) {
+        const int hd = lane & 31;
+        const int fl_p = hb == 0 ? ((hd >> 4) ? fl.y : fl.x) : ((hd >> 4) ? fl.w : fl.z);
+        const float fsc = fl_p ? facbuf[(vpar * 4 + 2 * hb + (hd >> 4)) * 16 + (hd & 15)] : 1.0f;
+#pragma unroll
+        for (int dvb = 0; dvb < 4; ++dvb)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) o[dvb][hb][j] *= fsc;
+      }
+    }
+    if (has_scale) {
+      // P times V's block scale (fp32 product, rounded to bf16 again): V itself is converted unscaled
+#pragma unroll
+      for (int kstep = 0; kstep < 2; ++kstep) {
+        const float sc[8] = {vs[kstep][0].x, vs[kstep][0].y, vs[kstep][0].z, vs[kstep][0].w,
+                             vs[kstep][1].x, vs[kstep][1].y, vs[kstep][1].z, vs[kstep][1].w};
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+          const uint4 w = __builtin_bit_cast(uint4, pb[kstep][hb]);
+          const unsigned in[4] = {w.x, w.y, w.z, w.w};
+          unsigned outw[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            outw[i] = pack_bf16(__uint_as_float(in[i] << 16) * sc[2 * i], __uint_as_float(in[i] & 0xffff0000u) * sc[2 * i + 1]);
+          pb[kstep][hb] = __builtin_bit_cast(bf16x8, make_uint4(outw[0], outw[1], outw[2], outw[3]));
+        }
+      }
+    }
+    bf16x8 a[4];
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) a[dvb] = cvt8((unsigned)v0[dvb][0], (unsigned)v0[dvb][1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+      mfma_o(o[dvb][0], a[dvb], pb[0][0]);
+      mfma_o(o[dvb][1], a[dvb], pb[0][1]);
+      if (dma) dma_part(dvb);
+    }
+    if (next) load_v(tv + 1, 0, v0);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) a[dvb] = cvt8((unsigned)v1[dvb][0], (unsigned)v1[dvb][1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dvb = 0; dvb < 4; ++dvb) {
+      mfma_o(o[dvb][0], a[dvb], pb[1][0]);
+      mfma_o(o[dvb][1], a[dvb], pb[1][1]);
+      if (dma && dvb < 2) dma_part(4 + dvb);
+    }
+  };
+
+  // ---- pipeline ----
+  // only the first tile is requested ahead of the first barrier (issuing blocks while the load
+  // unit's queue is full, and the producers cannot start before this wavefront gets there)
+  if (n_tiles > 0) issue_tile(0);
+  wait_outstanding(0);                            // tile 0 has landed
+  __syncthreads();                                // [X]
+#pragma unroll
+  for (int tau = 1; tau < kAhead; ++tau)
+    if (tau < n_tiles) issue_tile(tau);
+  if (n_tiles > 0) load_v(0, 0, v0);
+  wait_outstanding(max(min(kAhead, n_tiles) - 3, 0));   // tile 2 has landed
+  for (int t = 0; t < n_tiles; ++t) {
+    __syncthreads();                              // [B_t]
+    const bool more = t + kAhead < n_tiles;
+    consume(t, t + 1 < n_tiles, more);            // (tile t+4 goes into the slot of tile t-1)
+    // tile t+3 must have landed before the next barrier; the tile issued after it may stay in flight
+    wait_outstanding(max(min(t + kAhead, n_tiles - 1) - (t + 3), 0));
+  }
+  __syncthreads();                                // [E] statistics are visible; the ring is free
+
+  // ---- epilogue ----
+  const int hd = lane & 31, gq2 = lane >> 5;
+  const bool direct = p.num_splits == 1;
+  float* xbuf = reinterpret_cast<float*>(smem) + role * 32 * kXPitch;     // private to this wavefront
+#pragma unroll
+  for (int hb = 0; hb < 2; ++hb) {
+    const float m_all = stats[((2 * hb + (hd >> 4)) * 16 + (hd & 15)) * 2];
+    const float l_all = stats[((2 * hb + (hd >> 4)) * 16 + (hd & 15)) * 2 + 1];
+    const int h_local = 32 * hb + hd;
+    if (!direct) {
+      // key split: the unnormalised accumulators leave exactly as the lanes hold them (rounded to
+      // bf16: the values are relative to the split's own maximum, so their range is that of the
+      // output times the split's probability mass)
+      unsigned short* blk = (unsigned short*)p.workspace + part_block * (size_t)(2 * kPartFloats) +
+                            ((size_t)((role * 2 + hb) * 16) * 64 + lane) * 4;
+#pragma unroll
+      for (int dvb = 0; dvb < 4; ++dvb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x16& acc = o[dvb][hb];
+          *reinterpret_cast<uint2*>(blk + (size_t)(dvb * 4 + j) * 256) =
+              make_uint2(pack_bf16(acc[4 * j], acc[4 * j + 1]), pack_bf16(acc[4 * j + 2], acc[4 * j + 3]));
+        }
+      }
+      if (role == 0 && lane < 32) {
+        float* ml = (float*)((unsigned short*)p.workspace + part_blocks_total * (size_t)(2 * kPartFloats)) + (part_block * kHeadsWg + h_local) * 2;
+        ml[0] = m_all;
+        ml[1] = l_all;
+      }
+      continue;
+    }
     float out_scale = 1.0f, lse_val = 0.0f;
-    if (direct) {
+    {
       float m_fin = m_all, l_fin = l_all;
       if (p.sinks && h_local < heads_here) {
         const float sk = p.sinks[head0 + h_local] * kLog2e;
@@ -667,35 +790,12 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
         out_scale = 0.0f;
       }
     }
-    if (!direct) {
-      // key split: the unnormalised accumulators leave exactly as the lanes hold them (1 KiB per
-      // store instruction); the combine kernel knows the layout and does the transposition
-      // (bf16: the values are relative to the split's own maximum, so their range is that of
-      // the output times the split's probability mass; the rounding is 2^-9 relative)
-      unsigned short* blk = (unsigned short*)p.workspace + part_block * (size_t)(HG * kPartFloats) +
-                            ((size_t)((wave * HG + hg) * 16) * 64 + lane) * 4;
-#pragma unroll
-      for (int dvb = 0; dvb < 4; ++dvb) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const f32x16& acc = o[4 * dvb + hg];
-          *reinterpret_cast<uint2*>(blk + (size_t)(dvb * 4 + j) * 256) =
-              make_uint2(pack_bf16(acc[4 * j], acc[4 * j + 1]), pack_bf16(acc[4 * j + 2], acc[4 * j + 3]));
-        }
-      }
-      if (wave == 0 && lane < 32) {
-        float* ml = (float*)((unsigned short*)p.workspace + part_blocks_total * (size_t)(HG * kPartFloats)) + (part_block * (32 * HG) + h_local) * 2;
-        ml[0] = m_all;
-        ml[1] = l_all;
-      }
-      continue;
-    }
     // transpose through LDS: lane (head hd, gq2) holds channels 32dvb + 8j + 4gq2 + (0..3) in o[.][4j..4j+3]
 #pragma unroll
     for (int dvb = 0; dvb < 4; ++dvb) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const f32x16& acc = o[4 * dvb + hg];
+        const f32x16& acc = o[dvb][hb];
         const float4 v = make_float4(acc[4 * j] * out_scale, acc[4 * j + 1] * out_scale, acc[4 * j + 2] * out_scale,
                                      acc[4 * j + 3] * out_scale);
         *reinterpret_cast<float4*>(xbuf + hd * kXPitch + 32 * dvb + 8 * j + 4 * gq2) = v;
@@ -706,10 +806,10 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
 #pragma unroll 4
     for (int it = 0; it < 16; ++it) {
       const int row = 2 * it + gq2;
-      const int hl = 32 * hg + row;
+      const int hl = 32 * hb + row;
       if (hl >= heads_here) continue;
       const float4 v = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + hd * 4);
-      const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + 128 * wave + hd * 4;
+      const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + 128 * role + hd * 4;
       if (p.out_dtype == CPPMEGA_MI355_F32) {
         *reinterpret_cast<float4*>((float*)p.out + off) = v;
       } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
@@ -721,18 +821,18 @@ __global__ __launch_bounds__(256, 1) void sparse_mla_latent_kernel(const MlaPara
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (wave == 0 && lane < 32 && h_local < heads_here && p.lse) p.lse[q_index * p.H + head0 + h_local] = lse_val;
+    if (role == 0 && lane < 32 && h_local < heads_here && p.lse) p.lse[q_index * p.H + head0 + h_local] = lse_val;
   }
 }
 
 // Merges the key splits written by sparse_mla_latent_kernel.  A partial block holds, per
-// (wavefront w = 128 value channels, head group hg), 16 rows of 64 lanes x float4 exactly as the
+// (consumer w = 128 value channels, 32-head block hg), 16 rows of 64 lanes x float4 exactly as the
 // accumulator registers held them: row 4*dvb + j, lane (head hd = lane%32, half = lane/32), element e
 // is channel 128w + 32dvb + 8j + 4half + e of head 32hg + hd.  One workgroup per (query, KV group,
 // head chunk, w, hg): coalesced 1 KiB row reads, weights per head, transposition through LDS,
 // coalesced output rows.
-template <int HG>
 __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const MlaParams p) {
+  constexpr int HG = kHeadsWg / 32;
   __shared__ float x[32][kXPitch];
   const int tid = (int)threadIdx.x, lane = tid & 63, r4 = tid >> 6;
   const int chunks = (p.heads_per_group + 32 * HG - 1) / (32 * HG);
@@ -852,38 +952,17 @@ bool sparse_mla_latent_supported(const MlaParams& p) {
   if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
   if (p.kv_scale && ((uintptr_t)p.kv_scale & 3)) return false;
   if ((unsigned long long)p.B * p.Skv * p.G >= 0x7fffffffull) return false;   // cache rows are counted in 32 bits
+  if (p.topk > 16 * kMaxKeys) return false;       // the combine step merges at most 16 key splits
   return true;
 }
 
-// heads per workgroup (in units of 32) and the key-split factor
-static int latent_splits(const MlaParams& p, int hg, long long* wgs) {
-  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+void sparse_mla_latent_plan(MlaParams& p) {
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
   const long long base = (long long)p.B * p.S * p.G * chunks;
   int splits = 1;
   while (base * splits < 256 && p.topk / (splits * 2) >= 4 * kTK && splits < 16) splits *= 2;
-  while ((p.topk + splits - 1) / splits > kMaxKeys) splits *= 2;
-  *wgs = base * splits;
-  return splits;
-}
-
-void sparse_mla_latent_plan(MlaParams& p) {
-  // 128 heads per workgroup reuse every gathered row the most; 64 only when that is what it takes
-  // to cover the device (few queries, short key lists)
-  int hg = p.heads_per_group > 64 ? 4 : 2;
-  long long wgs4 = 0, wgs2 = 0;
-  if (hg == 4) {
-    latent_splits(p, 4, &wgs4);
-    latent_splits(p, 2, &wgs2);
-    if (wgs4 < 256 && wgs2 > wgs4) hg = 2;
-  }
-  if (const char* env = getenv("CPPMEGA_MI355_MLA_HEADS_PER_WG")) {
-    const int v = atoi(env);
-    if (v == 64) hg = 2;
-    if (v == 128) hg = 4;
-  }
-  p.heads_per_wg = 32 * hg;
-  long long wgs = 0;
-  const int splits = latent_splits(p, hg, &wgs);
+  while ((p.topk + splits - 1) / splits > kMaxKeys && splits < 16) splits *= 2;
+  p.heads_per_wg = kHeadsWg;
   const int tiles = (p.topk + kTK - 1) / kTK;
   const int tiles_per_split = (tiles + splits - 1) / splits;
   p.num_splits = splits;
@@ -891,54 +970,36 @@ void sparse_mla_latent_plan(MlaParams& p) {
 }
 
 int sparse_mla_latent_launch(const MlaParams& p, hipStream_t stream) {
-  const int hg = p.heads_per_wg / 32;
-  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
   const long long wgs = (long long)p.B * p.S * p.G * p.num_splits * chunks;
-  if (wgs > 0x7fffffffll || p.keys_per_split > kMaxKeys) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse MLA: launch too large");
-  const dim3 grid((unsigned)wgs), block(256);
+  if (wgs > 0x7fffffffll || p.keys_per_split > kMaxKeys || p.num_splits > 16)
+    return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse MLA: launch too large");
+  const dim3 grid((unsigned)wgs), block(512);
   const int nblk = p.kv_scale_kind == CPPMEGA_MI355_SCALE_F32_BLOCK ? kLat / p.kv_scale_block : 1;
-#define CM_LAUNCH_LATENT(HG_, NB_)                                                                                      \
-  do {                                                                                                                  \
-    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<HG_, NB_>,                                    \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, Geo<HG_>::kSmem));                      \
-    hipLaunchKernelGGL((sparse_mla_latent_kernel<HG_, NB_>), grid, block, Geo<HG_>::kSmem, stream, p);                   \
+#define CM_LAUNCH_PC(NB_)                                                                                          \
+  do {                                                                                                             \
+    CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_latent_kernel<NB_>,                                 \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmem));                           \
+    hipLaunchKernelGGL((sparse_mla_latent_kernel<NB_>), grid, block, kSmem, stream, p);                          \
   } while (0)
-  if (hg == 4) {
-    if (nblk == 4) CM_LAUNCH_LATENT(4, 4);
-    else if (nblk == 2) CM_LAUNCH_LATENT(4, 2);
-    else CM_LAUNCH_LATENT(4, 1);
-  } else {
-    if (nblk == 4) CM_LAUNCH_LATENT(2, 4);
-    else if (nblk == 2) CM_LAUNCH_LATENT(2, 2);
-    else CM_LAUNCH_LATENT(2, 1);
-  }
-#undef CM_LAUNCH_LATENT
+  if (nblk == 4) CM_LAUNCH_PC(4);
+  else if (nblk == 2) CM_LAUNCH_PC(2);
+  else CM_LAUNCH_PC(1);
+#undef CM_LAUNCH_PC
   CM_HIP_CHECK(hipGetLastError());
   if (p.num_splits > 1) {
-    const dim3 cgrid((unsigned)((size_t)p.B * p.S * p.G * chunks), (unsigned)(4 * hg));
-    if (hg == 4) hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
+    const dim3 cgrid((unsigned)((size_t)p.B * p.S * p.G * chunks), (unsigned)(4 * (kHeadsWg / 32)));
+    hipLaunchKernelGGL(sparse_mla_latent_combine_kernel, cgrid, dim3(256), 0, stream, p);
+    CM_HIP_CHECK(hipGetLastError());
   }
-  CM_HIP_CHECK(hipGetLastError());
-  return 0;
-}
-
-// the combine step alone (partials in the layout of hg 32-head groups per workgroup)
-int sparse_mla_latent_combine_launch(const MlaParams& p, int hg, hipStream_t stream) {
-  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
-  const dim3 cgrid((unsigned)((size_t)p.B * p.S * p.G * chunks), (unsigned)(4 * hg));
-  if (hg == 4) hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL(sparse_mla_latent_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
-  CM_HIP_CHECK(hipGetLastError());
   return 0;
 }
 
 size_t sparse_mla_latent_workspace_bytes(const MlaParams& p) {
   if (p.num_splits <= 1) return 0;
-  const int hg = p.heads_per_wg / 32;
-  const int chunks = (p.heads_per_group + 32 * hg - 1) / (32 * hg);
+  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
   const size_t blocks = (size_t)p.B * p.S * p.G * chunks * p.num_splits;
-  return blocks * ((size_t)hg * kPartFloats * sizeof(unsigned short) + 32 * hg * 2 * sizeof(float));
+  return blocks * ((size_t)2 * kPartFloats * sizeof(unsigned short) + kHeadsWg * 2 * sizeof(float));
 }
 
 }  // namespace cm

@@ -28,8 +28,6 @@
 //           read (ds_read_b64_tr_b16); P^T goes from the S^T accumulators to
 //           the B operand with one v_permlane16_swap, never through memory.
 
-#include <cstdlib>
-
 #include "sparse_mla_common.h"
 #include "mfma_util.h"
 
@@ -576,10 +574,6 @@ bool sparse_mla_mfma_supported(const MlaParams& p) {
 // Chooses the key-split factor: enough workgroups to cover the 256 CUs, at least 64 keys per wavefront.
 void sparse_mla_mfma_plan(MlaParams& p) {
   p.heads_per_wg = 0;
-  if (sparse_mla_latent_pc_supported(p) && !getenv("CPPMEGA_MI355_MLA_OLD")) {
-    sparse_mla_latent_pc_plan(p);
-    return;
-  }
   if (sparse_mla_latent_supported(p)) {
     sparse_mla_latent_plan(p);
     return;
@@ -595,14 +589,12 @@ void sparse_mla_mfma_plan(MlaParams& p) {
 }
 
 size_t sparse_mla_mfma_workspace_bytes(const MlaParams& p) {
-  if (p.heads_per_wg == 65) return sparse_mla_latent_pc_workspace_bytes(p);
   if (p.heads_per_wg != 0) return sparse_mla_latent_workspace_bytes(p);
   if (p.num_splits <= 1) return 0;
   return (size_t)p.B * p.S * p.H * p.num_splits * (kLat + 2) * sizeof(float);
 }
 
 int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
-  if (p.heads_per_wg == 65) return sparse_mla_latent_pc_launch(p, stream);
   if (p.heads_per_wg != 0) return sparse_mla_latent_launch(p, stream);
   const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
   const dim3 grid((unsigned)((size_t)p.B * p.S * p.G * groups_per_kv), (unsigned)p.num_splits), block(kWaves * 64);

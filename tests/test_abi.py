@@ -126,3 +126,44 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
     with pytest.raises(_lib.NativeLibraryError, match="no fallback"):
         _lib.load()
+
+
+def _latent_mla_args(**over):
+    """The decode layout (bf16 q, e4m3 latent + fp32/128 scales + bf16 rope), no buffers attached."""
+    a = _lib.SparseMlaArgs()
+    a.struct_size = C.sizeof(a)
+    a.kernel = _lib.MLA_KERNEL_AUTO
+    a.q_dtype, a.q_scale_kind = _lib.BF16, _lib.SCALE_NONE
+    a.kv_dtype, a.kv_scale_kind, a.kv_scale_block = _lib.E4M3, _lib.SCALE_F32_BLOCK, 128
+    a.rope_dtype, a.rope_dim = _lib.BF16, 64
+    a.index_dtype, a.out_dtype = _lib.I32, _lib.BF16
+    a.batch, a.seq_q, a.heads, a.kv_groups, a.seq_kv, a.topk = 32, 1, 128, 1, 65536, 2048
+    a.d_qk, a.d_v, a.sm_scale = 576, 512, 576 ** -0.5
+    for k, v in over.items():
+        setattr(a, k, v)
+    return a
+
+
+def test_kernel_choice_and_workspace_for_the_latent_cache_layout():
+    """Host-side plan of the shared-tile kernel (no GPU work): which kernel AUTO picks and what
+    workspace the key splits need.  Key lists longer than 16 splits of 2048 keys are left to the
+    scalar kernel (the combine step merges at most 16 splits)."""
+    lib = _lib.load()
+    need = C.c_size_t(0)
+    a = _latent_mla_args()
+    assert lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a)) == _lib.MLA_KERNEL_MFMA
+    assert lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == 0
+    # 32 queries x 2 head chunks x 4 key splits, each 64 heads x 512 channels bf16 + (max, sum) per head
+    assert need.value == 32 * 2 * 4 * (64 * 512 * 2 + 64 * 2 * 4)
+    a = _latent_mla_args(batch=1, seq_q=8192, seq_kv=8192)            # prefill: enough queries, no key splits
+    assert lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == 0 and need.value == 0
+    # longer lists go to the 32-head tile kernel, whose split count stops at 16 and whose partials are
+    # fp32 rows [B S, H, splits, 512 + 2]
+    a = _latent_mla_args(batch=1, topk=40000, seq_kv=65536)
+    assert lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a)) == _lib.MLA_KERNEL_MFMA
+    assert lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == 0
+    assert need.value == 128 * 16 * (512 + 2) * 4
+    a = _latent_mla_args(batch=1, topk=32768)                            # exactly 16 splits of 2048 keys
+    assert lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a)) == _lib.MLA_KERNEL_MFMA
+    assert lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == 0
+    assert need.value == 2 * 16 * (64 * 512 * 2 + 64 * 2 * 4)

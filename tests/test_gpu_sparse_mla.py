@@ -176,6 +176,8 @@ MFMA_CASES = [
     (1, 2, 48, 1, 256, 100, False, None, True),        # head count not a multiple of 32
     (4, 1, 128, 1, 4096, 2048, True, None, False),     # decode shape at reduced batch: key splits + combine
     (2, 1, 128, 1, 4096, 2048, False, None, True),     # key splits with sinks and general scales
+    (1, 1, 128, 1, 36000, 34000, True, None, False),   # more keys than 16 splits of the shared-tile kernel hold
+    (1, 3, 96, 1, 700, 300, False, 100, False),        # a second head chunk of 32 heads only
 ]
 
 
