@@ -53,13 +53,24 @@ def quantize_block_pow2(x: torch.Tensor, block: int = 128):
     return codes.reshape(shp).contiguous(), scale.contiguous()
 
 
-def make_latent_cache(gen, B, Skv, device):
+def quantize_block_amax(x: torch.Tensor, block: int = 128):
+    """x [..., K] fp32 -> (e4m3 bytes, fp32 scale [..., K/block]), scale = amax/448: the general fp32 block
+    scale of the FP8 producers (cppmega_v4/nn/moe_fp8.py:36-58), not a power of two."""
+    shp = x.shape
+    xb = x.reshape(*shp[:-1], shp[-1] // block, block)
+    amax = xb.abs().amax(dim=-1)
+    scale = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax))
+    codes = (xb / scale[..., None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    return codes.reshape(shp).contiguous(), scale.contiguous()
+
+
+def make_latent_cache(gen, B, Skv, device, pow2: bool = True):
     codes = torch.empty((B, Skv, 1, 512), dtype=torch.uint8, device=device)
     scale = torch.empty((B, Skv, 1, 4), dtype=torch.float32, device=device)
     rope = torch.empty((B, Skv, 1, 64), dtype=torch.bfloat16, device=device)
     for b in range(B):
         lat = torch.randn((Skv, 1, 512), generator=gen, device=device, dtype=torch.float32)
-        c, s = quantize_block_pow2(lat)
+        c, s = quantize_block_pow2(lat) if pow2 else quantize_block_amax(lat)
         codes[b], scale[b] = c, s
         rope[b] = torch.randn((Skv, 1, 64), generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16)
     return codes, scale, rope
@@ -106,13 +117,13 @@ def timed_graph(step_fns, steps: int, warmup: int):
 
 # --------------------------------------------------------------------------- workloads
 
-def bench_decode(args, device):
+def bench_decode(args, device, pow2: bool = False):
     from cppmega_mlx_amd import ops
     from cppmega_mlx_amd.nn._tilelang import sparse_mla_blockscaled_path_c as bs
 
     B, H, Skv, topk, d_qk, d_v = 32, 128, 65536, 2048, 576, 512
     gen = torch.Generator(device=device).manual_seed(1234)
-    codes, scale, rope = make_latent_cache(gen, B, Skv, device)
+    codes, scale, rope = make_latent_cache(gen, B, Skv, device, pow2=pow2)
     n_sets = 3
     qs = [torch.randn((B, 1, H, d_qk), generator=gen, device=device).to(torch.bfloat16) for _ in range(n_sets)]
     idxs = [uniform_indices(gen, B, 1, Skv, topk, device) for _ in range(n_sets)]
@@ -132,7 +143,8 @@ def bench_decode(args, device):
     bytes_alg = B * topk * 656 + B * H * d_qk * 2 + B * H * d_v * 2 + B * topk * 4 + B * H * 4
     per_step = secs / steps
     res = {
-        "workload": "sparse_mla_decode B=32 S_q=1 H=128 topk=2048 Skv=65536 latent e4m3[512]+fp32/128 +bf16 rope[64]",
+        "workload": "sparse_mla_decode B=32 S_q=1 H=128 topk=2048 Skv=65536 latent e4m3[512]+fp32/128 +bf16 rope[64], "
+                    + ("power-of-two block scales" if pow2 else "general fp32 block scales (amax/448)"),
         "kernel": kernel,
         "ms_per_step": per_step * 1e3,
         "host_ms_per_step": host_secs / steps * 1e3,
@@ -145,36 +157,71 @@ def bench_decode(args, device):
     return res, sample
 
 
-def cpu_baseline_decode(sample, budget_s: float = 15.0):
-    """Oracle on the first few sequences of the decode batch (compacted to their gathered rows)."""
-    from oracle import fp8, sparse_mla as om
+def host_description(threads: int) -> str:
+    model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for ln in fh:
+                if ln.startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return f"{model}, {threads} torch threads of {os.cpu_count()} logical CPUs"
+
+
+def repeat_timed(fn, min_seconds: float = 8.0, max_reps: int = 1000):
+    """Repeats fn() until min_seconds of host time have gone by (one untimed call first); returns
+    (seconds per call, calls)."""
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds or reps >= max_reps:
+            return dt / reps, reps
+
+
+def host_threads() -> int:
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    return torch.get_num_threads()
+
+
+def cpu_baseline_decode(sample, budget_s: float = 10.0):
+    """The reference's CPU fallback (gather -> fp32 matmul -> mask -> softmax -> matmul, restated in
+    float32 torch on all host cores) timed on the first sequences of the decode batch; the GPU
+    result of the same sequences is checked against the float64 oracle."""
+    from oracle import sparse_mla as om, torch_cpu
 
     q, codes, scale, rope, idx, out, lse, sm_scale = sample
     H, topk = q.shape[2], idx.shape[-1]
-    done, t_total, errs = 0, 0.0, []
-    threads = os.cpu_count() or 1
-    torch.set_num_threads(threads)
-    for b in range(q.shape[0]):
+    errs = []
+    threads = host_threads()
+    nseq = q.shape[0]
+    rows_all = np.empty((nseq, topk, 1, 576), dtype=np.float32)
+    for b in range(nseq):
         ids = idx[b, 0, 0].long()
-        rows = om.dequant_block_latent(codes[b, ids, 0].cpu().numpy(), scale[b, ids, 0].cpu().numpy(),
-                                       rope[b, ids, 0].float().cpu().numpy())[None, :, None, :]
-        qb = q[b:b + 1].float().cpu().numpy()
-        ar = np.arange(topk, dtype=np.int64)[None, None, None, :]
-        t0 = time.perf_counter()
-        want, _ = om.sparse_mla_oracle(qb, rows, ar, sm_scale=sm_scale, d_v=512)
-        t_total += time.perf_counter() - t0
+        rows_all[b] = om.dequant_block_latent(codes[b, ids, 0].cpu().numpy(), scale[b, ids, 0].cpu().numpy(),
+                                              rope[b, ids, 0].float().cpu().numpy())[:, None, :]
+    q_t = q.float().cpu()
+    rows_t = torch.from_numpy(rows_all)
+    ar = np.arange(topk, dtype=np.int64)[None, None, None, :]
+    ar_t = torch.from_numpy(np.broadcast_to(ar, (nseq, 1, 1, topk)).copy())
+    per_pass, reps = repeat_timed(lambda: torch_cpu.sparse_mla_fallback(q_t, rows_t, ar_t, sm_scale=sm_scale, d_v=512), budget_s)
+    for b in range(2):
+        want, _ = om.sparse_mla_oracle(q_t[b:b + 1].numpy(), rows_all[b:b + 1], ar, sm_scale=sm_scale, d_v=512)
         got = out[b:b + 1].float().cpu().numpy()
         errs.append(float(np.abs(got - want).max() / np.abs(want).max()))
-        done += 1
-        if t_total > budget_s:
-            break
-    flops = 2.0 * done * H * topk * (576 + 512)
+    flops = 2.0 * nseq * H * topk * (576 + 512)
     return {
-        "value": flops / t_total / 1e12,
+        "value": flops / per_pass / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"NumPy float64 oracle on {done} of 32 sequences (H=128, topk=2048 gathered rows), {t_total:.2f} s",
+        "sample": f"float32 torch restatement of the reference fallback on all {nseq} sequences (H=128, topk=2048, "
+                  f"rows already gathered), {reps} passes of {per_pass:.3f} s; {host_description(threads)}",
     }, max(errs)
 
 
@@ -240,18 +287,21 @@ def bench_vecmat_fp8x(args, device):
     }
 
 
-def cpu_baseline_vecmat(sample, rows: int = 1024):
-    from oracle import vecmat as ov
+def cpu_baseline_vecmat(sample, rows: int = 7168):
+    from oracle import fp8, torch_cpu, vecmat as ov
 
     x, w, s, out = sample
-    wn, sn, xn = w[:rows].cpu().numpy(), s[:rows].cpu().numpy(), x.float().cpu().numpy()
-    t0 = time.perf_counter()
-    want = ov.fused_fp8_gemm_oracle(wn, sn, xn)
-    dt = time.perf_counter() - t0
-    err = float(np.abs(out[:, :rows].float().cpu().numpy() - want).max() / np.abs(want).max())
+    threads = host_threads()
+    wf = torch.from_numpy(fp8.e4m3_decode(w[:rows].cpu().numpy()))
+    sn, xn = s[:rows].cpu(), x.float().cpu()
+    dt, reps = repeat_timed(lambda: torch_cpu.fused_fp8_gemm_fallback(wf, sn, xn), 8.0)
+    check = 256
+    want = ov.fused_fp8_gemm_oracle(w[:check].cpu().numpy(), s[:check].cpu().numpy(), xn.numpy())
+    err = float(np.abs(out[:, :check].float().cpu().numpy() - want).max() / np.abs(want).max())
     nbytes = rows * w.shape[1] * (1 + 4 / 128)
-    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": os.cpu_count() or 1, "kind": "port",
-            "sample": f"NumPy float64 dequant+matmul on the first {rows} of 7168 weight rows, {dt:.2f} s"}, err
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"float32 torch dequantise + matmul (the reference's fallback) on {rows} of 7168 weight rows, "
+                      f"byte decode not timed, {reps} passes of {dt:.3f} s; {host_description(threads)}"}, err
 
 
 def bench_topk(args, device):
@@ -290,18 +340,20 @@ def bench_topk(args, device):
     return res, (scores[0], ends, outs[0], k)
 
 
-def cpu_baseline_topk(sample, rows: int = 512):
-    from oracle import topk as ot
+def cpu_baseline_topk(sample, rows: int = 4096):
+    from oracle import topk as ot, torch_cpu
 
     scores, ends, out, k = sample
-    sn, en = scores[:rows].cpu().numpy(), ends[:rows].cpu().numpy()
-    t0 = time.perf_counter()
-    want = ot.topk_selector_oracle(sn, k, ends=en)
-    dt = time.perf_counter() - t0
-    exact = bool(np.array_equal(out[:rows].cpu().numpy(), want))
+    threads = host_threads()
+    st, et = scores[:rows].cpu(), ends[:rows].cpu()
+    dt, reps = repeat_timed(lambda: torch_cpu.topk_fallback(st, k, ends=et), 8.0)
+    check = 256
+    want = ot.topk_selector_oracle(st[:check].numpy(), k, ends=et[:check].numpy())
+    exact = bool(np.array_equal(out[:check].cpu().numpy(), want))
     nbytes = rows * (scores.shape[1] * 4 + k * 4)
-    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"NumPy stable-argsort oracle on the first {rows} of 4096 rows, {dt:.2f} s"}, exact
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"float32 torch stable-sort selection (the reference's argsort fallback) on {rows} of 4096 rows, "
+                      f"{reps} passes of {dt:.3f} s; {host_description(threads)}"}, exact
 
 
 def bench_prefill(args, device):
@@ -424,13 +476,18 @@ def main() -> int:
         "config": {},
     }
     if "decode" in parts:
-        res, sample = bench_decode(args, device)
+        res_pow2, sample = bench_decode(args, device, pow2=True)
+        del sample
+        torch.cuda.empty_cache()
+        res, sample = bench_decode(args, device, pow2=False)
         line["value"] = res["tflops"]
         line["ms_per_step"] = res["ms_per_step"]
         line["config"] = {"workload": res["workload"], "kernel": res["kernel"],
                           "flops_per_step": res["flops_per_step"],
                           "algorithmic_bytes_per_step": res["algorithmic_bytes_per_step"],
-                          "host_ms_per_step": res["host_ms_per_step"], "hbm_gbs": res["hbm_gbs"]}
+                          "host_ms_per_step": res["host_ms_per_step"], "hbm_gbs": res["hbm_gbs"],
+                          "power_of_two_block_scales": {"ms_per_step": res_pow2["ms_per_step"], "tflops": res_pow2["tflops"],
+                                                        "frac": res_pow2["tflops"] / MFMA_BF16_PEAK_TFLOPS}}
         line["roofline"] = {"bound": "mfma", "achieved": res["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                             "frac": res["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic("sparse_mla_decode")}
         if not args.no_cpu_baseline:
