@@ -126,7 +126,15 @@ class SparseMlaArgs(C.Structure):
         ("reserved", C.c_int32),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
+        ("sm_scale_dev", C.c_void_p),
+        ("has_sinks_dev", C.c_void_p),
+        ("seq_kv_pitch", C.c_int32),
+        ("reserved2", C.c_int32),
     ]
+
+
+# struct_size of the first ABI of SparseMlaArgs (through workspace_bytes): still accepted by the library
+SPARSE_MLA_ARGS_V1_SIZE = SparseMlaArgs.sm_scale_dev.offset
 
 
 class VecmatArgs(C.Structure):
@@ -345,8 +353,28 @@ def ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
-def require_device_tensor(t: torch.Tensor, name: str, ref: torch.Tensor | None = None) -> None:
-    """Inputs must be dense device tensors; the boundary never copies or casts."""
+def batch_pitch(t: torch.Tensor) -> int | None:
+    """Rows of dim 1 between two batches of ``t`` when everything but the batch stride is dense
+    (a ``cache[:, :n]`` view of a dense buffer), else None."""
+    if t.ndim < 2:
+        return None
+    inner = 1
+    for size, stride in zip(reversed(t.shape[1:]), reversed(t.stride()[1:])):
+        if size != 1 and stride != inner:
+            return None
+        inner *= size
+    row = inner // max(t.shape[1], 1) if t.shape[1] else 0
+    if t.shape[0] <= 1 or t.shape[1] == 0:
+        return t.shape[1]
+    if row == 0 or t.stride(0) % row != 0 or t.stride(0) < inner:
+        return None
+    return t.stride(0) // row
+
+
+def require_device_tensor(t: torch.Tensor, name: str, ref: torch.Tensor | None = None, *,
+                          allow_batch_pitch: bool = False) -> None:
+    """Inputs must be dense device tensors; the boundary never copies or casts.  With
+    ``allow_batch_pitch`` the batch stride alone may exceed the dense one."""
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor; got {type(t).__name__}")
     if not t.is_cuda:
@@ -354,7 +382,9 @@ def require_device_tensor(t: torch.Tensor, name: str, ref: torch.Tensor | None =
             ERR_UNSUPPORTED,
             f"{name} lives on {t.device}; the MI355X kernels take device tensors only and there is no CPU path",
         )
-    if not t.is_contiguous():
+    if allow_batch_pitch and batch_pitch(t) is not None:
+        pass
+    elif not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous (the boundary does not copy); got strides {t.stride()}")
     if ref is not None and t.device != ref.device:
         raise ValueError(f"{name} is on {t.device} but other operands are on {ref.device}")

@@ -83,6 +83,23 @@ static int build_mla_params(const cppmega_mi355_sparse_mla_args_t& a, MlaParams&
   p.B = a.batch; p.S = a.seq_q; p.H = a.heads; p.G = a.kv_groups; p.Skv = a.seq_kv; p.topk = a.topk;
   p.d_qk = a.d_qk; p.d_kv = d_kv; p.d_v = a.d_v; p.heads_per_group = a.heads / a.kv_groups;
   p.num_splits = 1; p.keys_per_split = a.topk; p.sm_scale = a.sm_scale;
+  p.sm_scale_dev = a.sm_scale_dev; p.has_sinks_dev = a.has_sinks_dev;
+  if (a.seq_kv_pitch != 0 && a.seq_kv_pitch < a.seq_kv)
+    return fail(CPPMEGA_MI355_ERR_SHAPE, "sparse_mla: seq_kv_pitch %d is below seq_kv %d", a.seq_kv_pitch, a.seq_kv);
+  p.Skv_pitch = a.seq_kv_pitch != 0 ? a.seq_kv_pitch : a.seq_kv;
+  return 0;
+}
+
+// Copies the caller's sparse-MLA struct into the current layout; a caller built against the first
+// ABI (struct_size ends at workspace_bytes) gets zeros for the fields appended since.
+static int widen_mla_args(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size, cppmega_mi355_sparse_mla_args_t& a) {
+  if (!args) return fail(CPPMEGA_MI355_ERR_NULL, "args is NULL");
+  const size_t have = args_size < (size_t)args->struct_size ? args_size : (size_t)args->struct_size;
+  if (have < CPPMEGA_MI355_SPARSE_MLA_ARGS_V1_SIZE)
+    return fail(CPPMEGA_MI355_ERR_STRUCT_SIZE, "args struct is %zu/%u bytes, need %zu", args_size, args->struct_size,
+                (size_t)CPPMEGA_MI355_SPARSE_MLA_ARGS_V1_SIZE);
+  memset(&a, 0, sizeof(a));
+  memcpy(&a, args, have < sizeof(a) ? have : sizeof(a));
   return 0;
 }
 
@@ -157,23 +174,25 @@ int cppmega_mi355_topk_select(const cppmega_mi355_topk_args_t* args, size_t args
 }
 
 int cppmega_mi355_sparse_mla_select_kernel(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size) {
-  if (!args) return -fail(CPPMEGA_MI355_ERR_NULL, "args is NULL");
-  if (args_size < sizeof(*args) || args->struct_size < sizeof(*args))
-    return -fail(CPPMEGA_MI355_ERR_STRUCT_SIZE, "args struct too small");
-  MlaParams p;
-  const int rc = build_mla_params(*args, p, false);
+  cppmega_mi355_sparse_mla_args_t a;
+  int rc = widen_mla_args(args, args_size, a);
   if (rc) return -rc;
-  return pick_mla_kernel(*args, p);
+  MlaParams p;
+  rc = build_mla_params(a, p, false);
+  if (rc) return -rc;
+  return pick_mla_kernel(a, p);
 }
 
 int cppmega_mi355_sparse_mla_workspace_bytes(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size,
                                              size_t* bytes) {
-  CM_CHECK_ARGS(args, args_size, cppmega_mi355_sparse_mla_args_t);
+  cppmega_mi355_sparse_mla_args_t a;
+  int rc = widen_mla_args(args, args_size, a);
+  if (rc) return rc;
   if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "bytes is NULL");
   MlaParams p;
-  int rc = build_mla_params(*args, p, false);
+  rc = build_mla_params(a, p, false);
   if (rc) return rc;
-  const int kern = pick_mla_kernel(*args, p);
+  const int kern = pick_mla_kernel(a, p);
   if (kern < 0) return -kern;
   *bytes = 0;
   if (kern == CPPMEGA_MI355_MLA_KERNEL_MFMA) {
@@ -184,18 +203,20 @@ int cppmega_mi355_sparse_mla_workspace_bytes(const cppmega_mi355_sparse_mla_args
 }
 
 int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size, void* stream) {
-  CM_CHECK_ARGS(args, args_size, cppmega_mi355_sparse_mla_args_t);
-  MlaParams p;
-  int rc = build_mla_params(*args, p, true);
+  cppmega_mi355_sparse_mla_args_t a;
+  int rc = widen_mla_args(args, args_size, a);
   if (rc) return rc;
-  const int kern = pick_mla_kernel(*args, p);
+  MlaParams p;
+  rc = build_mla_params(a, p, true);
+  if (rc) return rc;
+  const int kern = pick_mla_kernel(a, p);
   if (kern < 0) return -kern;
   if (kern == CPPMEGA_MI355_MLA_KERNEL_MFMA) {
     sparse_mla_mfma_plan(p);
     const size_t need = sparse_mla_mfma_workspace_bytes(p);
-    if (need > 0 && (!args->workspace || args->workspace_bytes < need))
+    if (need > 0 && (!a.workspace || a.workspace_bytes < need))
       return fail(CPPMEGA_MI355_ERR_WORKSPACE, "sparse_mla: workspace of %zu bytes needed, %zu given", need,
-                  args->workspace ? args->workspace_bytes : (size_t)0);
+                  a.workspace ? a.workspace_bytes : (size_t)0);
     return sparse_mla_mfma_launch(p, (hipStream_t)stream);
   }
   return sparse_mla_scalar_launch(p, (hipStream_t)stream);
@@ -203,10 +224,12 @@ int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, si
 
 int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size, float* scores,
                                     void* stream) {
-  CM_CHECK_ARGS(args, args_size, cppmega_mi355_sparse_mla_args_t);
+  cppmega_mi355_sparse_mla_args_t a;
+  int rc = widen_mla_args(args, args_size, a);
+  if (rc) return rc;
   if (!scores) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla_scores: scores is NULL");
   MlaParams p;
-  const int rc = build_mla_params(*args, p, true, false);
+  rc = build_mla_params(a, p, true, false);
   if (rc) return rc;
   p.scores = scores;
   return sparse_mla_scores_launch(p, (hipStream_t)stream);

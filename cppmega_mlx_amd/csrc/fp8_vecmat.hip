@@ -19,7 +19,6 @@
 //    output row, scalar byte loads.
 
 #include <type_traits>
-#include <cstdlib>
 
 #include "common.h"
 
@@ -703,10 +702,6 @@ static int device_cus() {
 // round over the compute units (ties: the earlier candidate).
 static int stream_rows(int n, int m) {
   const int cus = device_cus();
-  if (const char* e = getenv("CPPMEGA_MI355_VECMAT_ROWS")) {
-    const int v = atoi(e);
-    if (v >= kStreamU && v <= kStreamMaxRows && v % kStreamU == 0) return v;
-  }
   if (n < 16 * cus) {
     const int r = (n / cus) & ~(kStreamU - 1);
     return r < kStreamU ? kStreamU : r;
@@ -729,10 +724,6 @@ static int stream_rows(int n, int m) {
 // in the preference order below.
 static void stream_split(int k, int* w_out, int* ch_out) {
   const int chunks = (k + kChunk - 1) / kChunk;
-  if (const char* e = getenv("CPPMEGA_MI355_VECMAT_WAVES")) {
-    const int w = atoi(e);
-    if (w >= 1 && w <= 8 && (chunks + w - 1) / w <= 4) { *w_out = w; *ch_out = (chunks + w - 1) / w; return; }
-  }
   if (chunks < 4) { *w_out = chunks; *ch_out = 1; return; }
   const int pref[5] = {4, 8, 7, 6, 5};
   int best_w = 8, best_ch = 4, best_waste = 1 << 30;

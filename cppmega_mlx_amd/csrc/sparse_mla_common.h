@@ -28,7 +28,16 @@ struct MlaParams {
   int keys_per_split;
   int heads_per_wg;     // 0: 32-head tile kernel; 64: shared-tile latent kernel (sparse_mla_latent.hip)
   float sm_scale;
+  const float* sm_scale_dev;     // device copy of the softmax scale; read in place of sm_scale when set
+  const int* has_sinks_dev;      // device flag; sinks are ignored when it is set and holds 0
+  int Skv_pitch;                 // key rows between two batches of the cache buffers (>= Skv)
 };
+
+// softmax scale and sink switch as the kernels read them (uniform loads)
+__device__ __forceinline__ float mla_sm_scale(const MlaParams& p) { return p.sm_scale_dev ? *p.sm_scale_dev : p.sm_scale; }
+__device__ __forceinline__ bool mla_has_sinks(const MlaParams& p) {
+  return p.sinks != nullptr && (p.has_sinks_dev == nullptr || *p.has_sinks_dev != 0);
+}
 
 __device__ __forceinline__ long long load_index(const MlaParams& p, size_t i) {
   return p.index_dtype == CPPMEGA_MI355_I64 ? ((const long long*)p.indices)[i]

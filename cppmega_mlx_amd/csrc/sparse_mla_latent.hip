@@ -239,6 +239,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   // the first key tile.
   constexpr int kRounds = kMaxKeys / 512;
   const bool wide = p.index_dtype == CPPMEGA_MI355_I64;
+  const float sm_scale = mla_sm_scale(p);        // (a uniform load when the scale lives in device memory)
   int idx_lo[kRounds], idx_hi[kRounds];
   {
     const int* words = (const int*)p.indices;
@@ -268,7 +269,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
         if (ok) mine = i;
         // a tile is the 32 consecutive entries of half a wavefront; the masked-key path also serves a
         // non-positive softmax scale (the plain path takes maxima before scaling)
-        const unsigned long long okm = __ballot(ok && p.sm_scale > 0.0f);
+        const unsigned long long okm = __ballot(ok && sm_scale > 0.0f);
         if ((lane & 31) == 0 && i < list_tiles * kTK) tvalid[i / kTK] = (unsigned)(okm >> (lane & 32)) == 0xffffffffu;
       }
     }
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     for (int blk = 0; blk < 4; ++blk) qexp |= split_q32(qraw[blk], qh[blk], ql[blk]) << (8 * blk);
     float m_run = -INFINITY;                      // base-2 running reference of head n
     float l_run = 0.0f;                           // this lane's share of its denominator
-    const float qk_scale = p.sm_scale * kLog2e;
+    const float qk_scale = sm_scale * kLog2e;
 
     // K operands of a tile -> registers: per sub-tile four 32-byte block fragments, two rope
     // fragments and the scales of this lane's key row (they give the operand exponents).  They are
@@ -554,7 +555,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   const bool scale_op = has_scale && 64 * role < kTK * nblk;
   const bool tr_op = has_scale && nblk > 1 && !scale_op && 64 * (role - nblk / 2) < kTK * nblk;
   const int tr_elem = 64 * (role - nblk / 2) + lane;          // (block, row) = (tr_elem / 32, tr_elem % 32)
-  const size_t group_row0 = ((size_t)b * p.Skv) * p.G + g;     // cache row of key 0; key k is G rows further per step
+  const size_t group_row0 = ((size_t)b * p.Skv_pitch) * p.G + g;     // cache row of key 0; key k is G rows further per step
   const int sc_elem = 64 * role + lane;
   const int sc_row = min(sc_elem / nblk, kTK - 1);
   const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + 128 * role + 32 * (lane >> 4);
@@ -775,7 +776,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     float out_scale = 1.0f, lse_val = 0.0f;
     {
       float m_fin = m_all, l_fin = l_all;
-      if (p.sinks && h_local < heads_here) {
+      if (mla_has_sinks(p) && h_local < heads_here) {
         const float sk = p.sinks[head0 + h_local] * kLog2e;
         const float m2 = fmaxf(m_fin, sk);
         const float keep = (m_fin == -INFINITY) ? 0.0f : exp2f(m_fin - m2);
@@ -865,7 +866,7 @@ __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const Ml
     m_all = fmaxf(m_all, ms[s]);
   }
   float m_fin = m_all, l_fin = 0.0f;
-  if (p.sinks && h_local < heads_here) {
+  if (mla_has_sinks(p) && h_local < heads_here) {
     const float sk = p.sinks[head0 + h_local] * kLog2e;
     m_fin = fmaxf(m_all, sk);
     l_fin = exp2f(sk - m_fin);
@@ -951,7 +952,7 @@ bool sparse_mla_latent_supported(const MlaParams& p) {
   if (p.topk < 1 || (size_t)p.B * p.S == 0) return false;
   if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
   if (p.kv_scale && ((uintptr_t)p.kv_scale & 3)) return false;
-  if ((unsigned long long)p.B * p.Skv * p.G >= 0x7fffffffull) return false;   // cache rows are counted in 32 bits
+  if ((unsigned long long)p.B * p.Skv_pitch * p.G >= 0x7fffffffull) return false;   // cache rows are counted in 32 bits
   if (p.topk > 16 * kMaxKeys) return false;       // the combine step merges at most 16 key splits
   return true;
 }

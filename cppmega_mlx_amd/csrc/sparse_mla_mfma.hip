@@ -123,7 +123,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     for (int j = 0; j < 16; ++j) o[i][j] = 0.0f;
   float m_run[2] = {-INFINITY, -INFINITY};   // base-2 running reference of heads (lane%16) and 16+(lane%16)
   float l_run[2] = {0.0f, 0.0f};             // this lane's share of the denominators
-  const float qk_scale = p.sm_scale * kLog2e;
+  const float qk_scale = mla_sm_scale(p) * kLog2e;
 
   // ---- staging ---------------------------------------------------------------------
   // The gathered rows travel HBM -> LDS by the load unit itself (no registers are held
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       rows[it] = upper ? rb : ra;
     }
     const int rope_r0 = __shfl(keyv, lane >> 3, 64), rope_r1 = __shfl(keyv, 8 + (lane >> 3), 64);
-    const size_t row_base = (size_t)b * p.Skv;
+    const size_t row_base = (size_t)b * p.Skv_pitch;
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
       if (rows[it] >= 0) {
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
 #pragma unroll 1
     for (int r = 0; r < kTile; ++r) {
       const int row = __shfl(keyv, r, 64);
-      const size_t krow = row >= 0 ? ((size_t)b * p.Skv + (size_t)row) * p.G + g : 0;
+      const size_t krow = row >= 0 ? ((size_t)b * p.Skv_pitch + (size_t)row) * p.G + g : 0;
       const unsigned short* src = (const unsigned short*)p.kv + krow * (size_t)p.d_kv;
       for (int c = lane; c < kDqk / 8; c += 64) {
         uint4 v = make_uint4(0, 0, 0, 0);
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   const bool direct = p.num_splits == 1;
   if (direct) {
     float m_fin = m_all, l_fin = l_all;
-    if (p.sinks && hd < heads_here) {
+    if (mla_has_sinks(p) && hd < heads_here) {
       const float sk = p.sinks[head0 + hd] * kLog2e;
       const float m2 = fmaxf(m_fin, sk);
       const float keep = (m_fin == -INFINITY) ? 0.0f : exp2f(m_fin - m2);
@@ -513,7 +513,7 @@ __global__ __launch_bounds__(256) void sparse_mla_combine_kernel(const MlaParams
   for (int s = 0; s < p.num_splits; ++s) m_all = fmaxf(m_all, ml[2 * s]);
   float m_fin = m_all;
   float sink_term = 0.0f;
-  if (p.sinks) {
+  if (mla_has_sinks(p)) {
     const float sk = p.sinks[h] * kLog2e;
     m_fin = fmaxf(m_all, sk);
     sink_term = exp2f(sk - m_fin);

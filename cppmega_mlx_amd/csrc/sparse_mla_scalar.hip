@@ -77,7 +77,8 @@ __global__ __launch_bounds__(64) void sparse_mla_scalar_kernel(const MlaParams p
                        ? p.d_kv : p.kv_scale_block;
   const int nkblk = (p.d_kv + kblk - 1) / kblk;
 
-  const bool has_sink = p.sinks != nullptr;
+  const bool has_sink = mla_has_sinks(p);
+  const float sm_scale = mla_sm_scale(p);
   float m = has_sink ? p.sinks[h] : -INFINITY;
   float l = has_sink ? 1.0f : 0.0f;
   float acc[DVI];
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(64) void sparse_mla_scalar_kernel(const MlaParams p
     const bool valid = key >= 0 && key < p.Skv;
     float score = -INFINITY;
     if (valid) {
-      const size_t krow = ((size_t)b * p.Skv + (size_t)key) * p.G + g;
+      const size_t krow = ((size_t)b * p.Skv_pitch + (size_t)key) * p.G + g;
       float dot = 0.0f;
       for (int kb = 0; kb < nkblk; ++kb) {
         const int d0 = kb * kblk, d1 = min(d0 + kblk, p.d_kv);
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(64) void sparse_mla_scalar_kernel(const MlaParams p
         for (int d = 0; d < p.rope_dim; ++d)
           dot = fmaf(qf[p.d_kv + d], load_as(p.rope, roff + d, p.rope_dtype), dot);
       }
-      score = dot * p.sm_scale;
+      score = dot * sm_scale;
     }
     const float tmax = wave_max(score);
     const float m_new = fmaxf(m, tmax);
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(64) void sparse_mla_scalar_kernel(const MlaParams p
       const int key_j = it[jx];
       if (key_j < 0) continue;             // uniform
       const float pw = pt[jx];
-      const size_t krow = ((size_t)b * p.Skv + (size_t)key_j) * p.G + g;
+      const size_t krow = ((size_t)b * p.Skv_pitch + (size_t)key_j) * p.G + g;
 #pragma unroll
       for (int i = 0; i < DVI; ++i) {
         const int dv = lane + 64 * i;
@@ -168,11 +169,12 @@ __global__ __launch_bounds__(64) void sparse_mla_scores_kernel(const MlaParams p
   const int kblk = (p.kv_scale_kind == CPPMEGA_MI355_SCALE_NONE || p.kv_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN)
                        ? p.d_kv : p.kv_scale_block;
   const int nkblk = (p.d_kv + kblk - 1) / kblk;
+  const float sm_scale = mla_sm_scale(p);
   for (int jj = lane; jj < p.topk; jj += 64) {
     const long long key = load_index(p, idx_base + jj);
     float score = -3.4028234663852886e38f;
     if (key >= 0 && key < p.Skv) {
-      const size_t krow = ((size_t)b * p.Skv + (size_t)key) * p.G + g;
+      const size_t krow = ((size_t)b * p.Skv_pitch + (size_t)key) * p.G + g;
       float dot = 0.0f;
       for (int kb = 0; kb < nkblk; ++kb) {
         const int d0 = kb * kblk, d1 = min(d0 + kblk, p.d_kv);
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(64) void sparse_mla_scores_kernel(const MlaParams p
         for (int d = 0; d < p.rope_dim; ++d)
           dot = fmaf(qf[p.d_kv + d], load_as(p.rope, roff + d, p.rope_dtype), dot);
       }
-      score = dot * p.sm_scale;
+      score = dot * sm_scale;
     }
     p.scores[bsh * p.topk + jj] = score;
   }

@@ -33,7 +33,6 @@
 // real number can reach (0x7f9..0x7ff, 0xff9..0xfff); those bins are cleared
 // before the scan instead of testing every element.
 
-#include <cstdlib>
 
 #include "common.h"
 
@@ -623,13 +622,7 @@ int launch_kernel(K kernel, const TopkParams& p, int threads, size_t smem, hipSt
   return 0;
 }
 
-static int wide_threads() {
-  if (const char* e = getenv("CPPMEGA_MI355_TOPK_THREADS")) {
-    const int v = atoi(e);
-    if (v == 256 || v == 512 || v == 1024) return v;
-  }
-  return 512;
-}
+static int wide_threads() { return 512; }
 
 template <typename ScoreT>
 int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* smem_out) {

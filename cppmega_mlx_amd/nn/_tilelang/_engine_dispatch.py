@@ -106,14 +106,13 @@ def _launch_mla(q_kind: int, kv_kind: int, block: int):
         nblk = K // block if block else 1
         qs = bufs["q_scale"].view(B, S, H, nblk) if block else bufs["q_scale"].view(B, S, H)
         ks = bufs["kv_scale"].view(B, Skv, G, nblk) if block else bufs["kv_scale"].view(B, Skv, G)
-        sinks = bufs.get("sinks")
-        has = bufs.get("has_sinks")
-        if has is not None and int(has.item()) == 0:
-            sinks = None
+        # sm_scale_buf and has_sinks stay device buffers the kernel reads on the stream, as in the
+        # reference: no host read-back, so the launch can be captured into a HIP graph
         ops.sparse_mla_forward(
-            q, kv, idx, sm_scale=float(bufs["sm_scale_buf"].item()), d_v=dv,
+            q, kv, idx, sm_scale=bufs["sm_scale_buf"], d_v=dv,
             out=bufs["out"].view(B, S, H, dv), lse=bufs["lse"].view(B, S, H),
-            q_spec=ops.QuantSpec(q_kind, qs, block), kv_spec=ops.QuantSpec(kv_kind, ks, block), sinks=sinks)
+            q_spec=ops.QuantSpec(q_kind, qs, block), kv_spec=ops.QuantSpec(kv_kind, ks, block),
+            sinks=bufs.get("sinks"), has_sinks=bufs.get("has_sinks"))
     return run
 
 

@@ -77,7 +77,7 @@ def sparse_mla_fwd_path_c_direct(
     d_v: int | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """Owner-output forward.  ``sm_scale_buf`` is the reference's 1-element
-    float32 scalar buffer; its value is read on the host (one ``.item()``)."""
+    float32 scalar buffer; it stays on the device and the kernel reads it on the stream."""
     status = sparse_mla_path_c_status()
     if not status.available:
         raise SparseMLAPathCDirectError(status.reason)
@@ -87,7 +87,7 @@ def sparse_mla_fwd_path_c_direct(
         raise ValueError("sm_scale_buf must be a 1-element float32 tensor")
     _validate_owner_outputs(q, out, lse, shapes)
     try:
-        _float_carrier_forward(q, kv, indices, sm_scale=float(sm_scale_buf.item()), d_v=shapes.d_v,
+        _float_carrier_forward(q, kv, indices, sm_scale=sm_scale_buf, d_v=shapes.d_v,
                                return_lse=True, kernel="auto", out=out, lse=lse)
     except (_lib.NativeCallError, _lib.NativeLibraryError) as exc:
         raise SparseMLAPathCDirectError(f"sparse-MLA forward dispatch failed: {type(exc).__name__}: {exc}") from exc

@@ -87,7 +87,7 @@ def _float_carrier_forward(
     kv: torch.Tensor,
     indices: torch.Tensor,
     *,
-    sm_scale: float | None,
+    sm_scale: float | torch.Tensor | None,
     d_v: int | None,
     return_lse: bool,
     kernel: str,
@@ -97,7 +97,10 @@ def _float_carrier_forward(
 ):
     shapes = _resolve_shapes(q, kv, indices, d_v=d_v)
     _check_carriers(q, kv, indices)
-    scale = shapes.qk_dim ** -0.5 if sm_scale is None else float(sm_scale)
+    if isinstance(sm_scale, torch.Tensor):                # a device float32[1], read by the kernel on the stream
+        scale = sm_scale
+    else:
+        scale = shapes.qk_dim ** -0.5 if sm_scale is None else float(sm_scale)
     if out is None:
         out = torch.empty((shapes.batch, shapes.seq_len, shapes.heads, shapes.d_v),
                           dtype=out_dtype or q.dtype, device=q.device)

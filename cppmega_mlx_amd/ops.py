@@ -112,7 +112,16 @@ class QuantSpec:
 _KERNELS = {"auto": _lib.MLA_KERNEL_AUTO, "scalar": _lib.MLA_KERNEL_SCALAR, "mfma": _lib.MLA_KERNEL_MFMA}
 
 
-def _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel):
+def _cache_pitch(kv, kv_scale, kv_rope) -> int:
+    """Key rows between two batches of the cache buffers: one value for kv, its scales and its rope."""
+    pitches = {name: _lib.batch_pitch(t) for name, t in (("kv", kv), ("kv_scale", kv_scale), ("kv_rope", kv_rope))
+               if t is not None and t.ndim >= 2 and t.shape[:2] == kv.shape[:2]}
+    if len(set(pitches.values())) > 1 or None in pitches.values():
+        raise ValueError(f"kv, kv_scale and kv_rope must share one batch pitch; got {pitches}")
+    return int(pitches["kv"])
+
+
+def _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel, has_sinks=None):
     B, S, H, d_qk = q.shape
     _, Skv, G, d_kv = kv.shape
     rope_dim = 0 if kv_rope is None else kv_rope.shape[-1]
@@ -134,7 +143,20 @@ def _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sink
     a.index_dtype = _dtype_or_raise(indices, "indices", (_lib.I32, _lib.I64))
     a.batch, a.seq_q, a.heads, a.kv_groups, a.seq_kv, a.topk = B, S, H, G, Skv, indices.shape[-1]
     a.d_qk, a.d_v = d_qk, int(d_v)
-    a.sm_scale = float(sm_scale)
+    if isinstance(sm_scale, torch.Tensor):
+        _lib.require_device_tensor(sm_scale, "sm_scale", q)
+        if sm_scale.dtype != torch.float32 or sm_scale.numel() != 1:
+            raise ValueError(f"a device sm_scale must be one float32; got {sm_scale.dtype} {tuple(sm_scale.shape)}")
+        a.sm_scale, a.sm_scale_dev = 0.0, sm_scale.data_ptr()
+    else:
+        a.sm_scale = float(sm_scale)
+    if has_sinks is not None:
+        _lib.require_device_tensor(has_sinks, "has_sinks", q)
+        if has_sinks.dtype != torch.int32 or has_sinks.numel() != 1:
+            raise ValueError(f"has_sinks must be one int32; got {has_sinks.dtype} {tuple(has_sinks.shape)}")
+        a.has_sinks_dev = has_sinks.data_ptr()
+    pitch = _cache_pitch(kv, kv_spec.scale, kv_rope)
+    a.seq_kv_pitch = 0 if pitch == Skv else pitch
     a.sinks = _lib.ptr(sinks)
     a.out = _lib.ptr(out)
     a.lse = _lib.ptr(lse)
@@ -147,7 +169,7 @@ def sparse_mla_forward(
     kv: torch.Tensor,
     indices: torch.Tensor,
     *,
-    sm_scale: float,
+    sm_scale: float | torch.Tensor,
     d_v: int,
     out: torch.Tensor,
     lse: torch.Tensor | None = None,
@@ -155,10 +177,17 @@ def sparse_mla_forward(
     kv_spec: QuantSpec | None = None,
     kv_rope: torch.Tensor | None = None,
     sinks: torch.Tensor | None = None,
+    has_sinks: torch.Tensor | None = None,
     kernel: str = "auto",
     workspace: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
-    """Sparse MLA forward into caller-owned ``out`` [B,S,H,d_v] (and ``lse`` [B,S,H])."""
+    """Sparse MLA forward into caller-owned ``out`` [B,S,H,d_v] (and ``lse`` [B,S,H]).
+
+    ``sm_scale`` is a Python float or a device float32[1] the kernels read on the stream (the
+    reference's ``sm_scale_buf``); ``has_sinks`` is an optional device int32[1] that switches
+    ``sinks`` off when it holds 0.  ``kv`` (with its scales and rope) may be a ``cache[:, :n]``
+    view of a dense buffer: only the first ``n`` rows of every batch are attendable.
+    """
     q_spec = q_spec or QuantSpec()
     kv_spec = kv_spec or QuantSpec()
     if kernel not in _KERNELS:
@@ -167,7 +196,8 @@ def sparse_mla_forward(
              ("sinks", sinks), ("q_scale", q_spec.scale), ("kv_scale", kv_spec.scale)]
     for name, t in named:
         if t is not None:
-            _lib.require_device_tensor(t, name, q if name != "q" else None)
+            _lib.require_device_tensor(t, name, q if name != "q" else None,
+                                       allow_batch_pitch=name in ("kv", "kv_rope", "kv_scale"))
     if q.ndim != 4 or kv.ndim != 4 or indices.ndim != 4:
         raise ValueError("sparse_mla: q, kv and indices must be rank 4")
     B, S, H, _ = q.shape
@@ -177,7 +207,7 @@ def sparse_mla_forward(
         raise ValueError(f"lse must be float32 with shape {(B, S, H)}; got {lse.dtype} {tuple(lse.shape)}")
     if sinks is not None and (tuple(sinks.shape) != (H,) or sinks.dtype != torch.float32):
         raise ValueError(f"sinks must be float32 with shape ({H},), got {sinks.dtype} {tuple(sinks.shape)}")
-    a = _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel)
+    a = _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel, has_sinks)
     lib = _lib.load()
     need = C.c_size_t(0)
     _lib.check(lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)), "sparse_mla")

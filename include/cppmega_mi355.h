@@ -180,7 +180,25 @@ typedef struct cppmega_mi355_sparse_mla_args {
 
   void* workspace;            /* split-KV partials; see *_workspace_bytes      */
   size_t workspace_bytes;
+
+  /* Fields below were added after the first ABI; a caller whose struct_size
+   * ends at workspace_bytes gets zeros for them. */
+  const float* sm_scale_dev;  /* device float32[1] or NULL.  When set the kernels
+                               * read the softmax scale from it on the stream
+                               * (the reference's `sm_scale_buf` parameter) and
+                               * `sm_scale` above is ignored.                   */
+  const int32_t* has_sinks_dev; /* device int32[1] or NULL.  When set and the
+                               * value is 0, `sinks` is ignored (the `has_sinks`
+                               * buffer of sparse_mla_fp8_path_c.py:1821-1835).  */
+  int32_t seq_kv_pitch;       /* key rows between two batches of kv / kv_scale /
+                               * kv_rope; 0 = seq_kv.  Lets a cache buffer of
+                               * capacity `pitch` be attended over its first
+                               * seq_kv rows (entries >= seq_kv are skipped).   */
+  int32_t reserved2;
 } cppmega_mi355_sparse_mla_args_t;
+
+/* struct_size of the first ABI of the struct above (through workspace_bytes). */
+#define CPPMEGA_MI355_SPARSE_MLA_ARGS_V1_SIZE (offsetof(cppmega_mi355_sparse_mla_args_t, sm_scale_dev))
 
 /* Bytes of workspace cppmega_mi355_sparse_mla_fwd needs for these shapes with
  * the kernel it would pick (0 when none).  Only the shape / dtype / kernel

@@ -35,30 +35,67 @@ def test_status_probe_reports_abi_and_arch():
     assert st["device_count"] >= 0
 
 
+STRUCTS = {
+    "cppmega_mi355_status_t": _lib.StatusStruct,
+    "cppmega_mi355_topk_args_t": _lib.TopkArgs,
+    "cppmega_mi355_sparse_mla_args_t": _lib.SparseMlaArgs,
+    "cppmega_mi355_vecmat_args_t": _lib.VecmatArgs,
+    "cppmega_mi355_quantize_args_t": _lib.QuantizeArgs,
+    "cppmega_mi355_cache_append_args_t": _lib.CacheAppendArgs,
+    "cppmega_mi355_causal_indices_args_t": _lib.CausalIndicesArgs,
+    "cppmega_mi355_mask_indices_args_t": _lib.MaskIndicesArgs,
+}
+
+
+def _header_struct_fields() -> dict[str, list[str]]:
+    """Field names, in order, of every ``typedef struct ... {...} name_t;`` in the header."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    found = {}
+    for body, name in re.findall(r"typedef\s+struct\s+\w+\s*\{(.*?)\}\s*(\w+)\s*;", text, flags=re.S):
+        names = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            for part in decl.split(","):
+                names.append(re.search(r"(\w+)\s*(\[[^\]]*\])?\s*$", part.strip()).group(1))
+        found[name] = names
+    return found
+
+
+def test_every_header_struct_has_a_ctypes_mirror_with_the_same_fields():
+    header = _header_struct_fields()
+    assert set(header) == set(STRUCTS)
+    for ctype, struct in STRUCTS.items():
+        assert [n for n, _ in struct._fields_] == header[ctype], ctype
+
+
 @pytest.mark.skipif(shutil.which("gcc") is None, reason="gcc not available")
 def test_struct_layouts_match_the_header(tmp_path):
-    fields = {
-        "cppmega_mi355_topk_args_t": (_lib.TopkArgs, ["scores", "row_stride", "k", "starts", "indices", "neg_inf_is_masked"]),
-        "cppmega_mi355_sparse_mla_args_t": (_lib.SparseMlaArgs, ["q", "kv_dtype", "kv", "kv_rope", "indices", "batch", "d_qk", "sm_scale", "sinks", "out", "lse", "out_dtype", "workspace", "workspace_bytes"]),
-        "cppmega_mi355_vecmat_args_t": (_lib.VecmatArgs, ["x", "scale_w", "scale_w_kind", "k", "out", "workspace_bytes"]),
-        "cppmega_mi355_status_t": (_lib.StatusStruct, ["abi_version", "built_for", "message"]),
-    }
+    """Size of every struct and offset of every field, as a C compiler lays the header out."""
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void){"]
-    for ctype, (_, names) in fields.items():
+    for ctype, struct in STRUCTS.items():
         lines.append(f'printf("{ctype} size %zu\\n", sizeof({ctype}));')
-        for n in names:
+        for n, _ in struct._fields_:
             lines.append(f'printf("{ctype} {n} %zu\\n", offsetof({ctype}, {n}));')
+    lines.append('printf("v1 size %zu\\n", (size_t)CPPMEGA_MI355_SPARSE_MLA_ARGS_V1_SIZE);')
     lines.append("return 0;}")
     src = tmp_path / "layout.c"
     src.write_text("\n".join(lines))
     exe = tmp_path / "layout"
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", str(src), "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    checked = 0
     for line in out.strip().splitlines():
         ctype, name, value = line.split()
-        struct = fields[ctype][0]
+        if ctype == "v1":
+            assert _lib.SparseMlaArgs.sm_scale_dev.offset == int(value) == _lib.SPARSE_MLA_ARGS_V1_SIZE
+            continue
+        struct = STRUCTS[ctype]
         got = C.sizeof(struct) if name == "size" else getattr(struct, name).offset
         assert got == int(value), f"{ctype}.{name}: ctypes {got} != C {value}"
+        checked += 1
+    assert checked == sum(len(s._fields_) + 1 for s in STRUCTS.values())
 
 
 def test_null_and_short_struct_are_rejected_with_the_bridge_codes():
@@ -73,6 +110,24 @@ def test_null_and_short_struct_are_rejected_with_the_bridge_codes():
     assert lib.cppmega_mi355_fp8_vecmat(None, 0, None) == _lib.ERR_NULL
     assert lib.cppmega_mi355_sparse_mla_fwd(None, 0, None) == _lib.ERR_NULL
     assert b"NULL" in lib.cppmega_mi355_error_string(_lib.ERR_NULL)
+
+
+def test_first_abi_sparse_mla_struct_is_still_accepted():
+    """A caller built before sm_scale_dev / has_sinks_dev / seq_kv_pitch were appended passes the
+    shorter struct_size; anything shorter than that is rejected."""
+    lib = _lib.load()
+    a = _latent_mla_args()
+    want = lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a))
+    assert want == _lib.MLA_KERNEL_MFMA
+    a.seq_kv_pitch = 7                                   # below seq_kv: a shape error when it is read...
+    assert lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a)) == -_lib.ERR_SHAPE
+    a.struct_size = _lib.SPARSE_MLA_ARGS_V1_SIZE         # ...and not read at all from a first-ABI caller
+    assert lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), _lib.SPARSE_MLA_ARGS_V1_SIZE) == want
+    need = C.c_size_t(0)
+    assert lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == _lib.OK
+    a.struct_size = _lib.SPARSE_MLA_ARGS_V1_SIZE - 8
+    assert lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == _lib.ERR_STRUCT_SIZE
+    assert lib.cppmega_mi355_sparse_mla_select_kernel(C.byref(a), C.sizeof(a)) == -_lib.ERR_STRUCT_SIZE
 
 
 def test_contract_violations_return_shape_and_dtype_codes_without_a_gpu():

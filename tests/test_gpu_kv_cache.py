@@ -205,11 +205,14 @@ def test_append_argument_errors(device):
         ops.kv_cache_append(x.cpu(), kv_cache=kv, scale_cache=sc, position=0)
 
 
-def test_appended_cache_feeds_the_decode_kernel(device):
+@pytest.mark.parametrize("H", [128, 32])
+def test_appended_cache_feeds_the_decode_kernel(device, H):
     """Producer and consumer together: rows appended through the fused producer, a causal
-    window from the index producer, attention over the cache against the oracle."""
+    window from the index producer, attention over the views the cache returns (batch stride =
+    capacity) against the oracle; then the same after a trim, where list entries that point at
+    trimmed rows must be skipped."""
     rng = np.random.default_rng(9)
-    B, T, H = 2, 200, 128
+    B, T = 2, 200
     lat_t, lat_f = bf16_pair(rng.standard_normal((B, T, 1, 512)), device)
     rope_t, rope_f = bf16_pair(rng.standard_normal((B, T, 1, 64)), device)
     cfg = SparseFP8KVCacheConfig(num_layers=1, batch_size=B, num_kv_heads=1, head_dim=512, max_seq_len=256, rope_dim=64,
@@ -218,18 +221,41 @@ def test_appended_cache_feeds_the_decode_kernel(device):
     cache.append_latent(0, lat_t[:, :150].contiguous(), rope_t[:, :150].contiguous())
     for s in range(150, T):                                                          # then token by token
         kv, sc, rp = cache.append_latent(0, lat_t[:, s:s + 1].contiguous(), rope_t[:, s:s + 1].contiguous())
+    assert not kv.is_contiguous() and kv.stride(0) == 256 * 512
     codes, scale = okv.quantize_block128(lat_f, pow2=True)
     rows = om.dequant_block_latent(codes, scale, rope_f, 128)
     q, qf = bf16_pair(rng.standard_normal((B, 1, H, 576)), device)
     idx = causal_sparse_indices(B, 1, 1, 96, query_offset=T - 1, key_length=T, device=device)
-    want_out, want_lse = om.sparse_mla_oracle(qf, rows, idx.cpu().numpy().astype(np.int64), sm_scale=576 ** -0.5, d_v=512)
+    idx_np = idx.cpu().numpy().astype(np.int64)
+    sinks = rng.standard_normal(H).astype(np.float32)
+    sm = torch.tensor([576 ** -0.5], dtype=torch.float32, device=device)              # read on the device
+    has = torch.ones(1, dtype=torch.int32, device=device)
     out = torch.zeros((B, 1, H, 512), dtype=torch.bfloat16, device=device)
     lse = torch.zeros((B, 1, H), dtype=torch.float32, device=device)
-    # the cache views are strided by the capacity; the kernel takes the full buffers and Skv = capacity
+
+    def attend(kv, sc, rp):
+        ops.sparse_mla_forward(q, kv, idx, sm_scale=sm, d_v=512, out=out, lse=lse, sinks=to_dev(sinks, device), has_sinks=has,
+                               kv_spec=ops.QuantSpec(_lib.SCALE_F32_BLOCK, sc, 128), kv_rope=rp)
+        torch.cuda.synchronize()
+        return out.float().cpu().numpy(), lse.cpu().numpy()
+
+    for flag in (1, 0):
+        has.fill_(flag)
+        got_out, got_lse = attend(kv, sc, rp)
+        want_out, want_lse = om.sparse_mla_oracle(qf, rows, idx_np, sm_scale=576 ** -0.5, d_v=512, sinks=sinks if flag else None)
+        err, ref = error_report(got_out, want_out)
+        assert err <= 2e-2 * ref
+        assert np.abs(got_lse - want_lse).max() <= 5e-3
+    # trimmed rows stay in the buffer; the shorter views make them unattendable
+    assert cache.trim(30) == 30
     layer = cache.sparse_fp8_layers[0]
-    ops.sparse_mla_forward(q, layer.kv, idx, sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse,
-                           kv_spec=ops.QuantSpec(_lib.SCALE_F32_BLOCK, layer.scale, 128), kv_rope=layer.rope)
-    torch.cuda.synchronize()
-    err, ref = error_report(out.float().cpu().numpy(), want_out)
+    n = cache.position()
+    got_out, got_lse = attend(layer.kv[:, :n], layer.scale[:, :n], layer.rope[:, :n])
+    want_out, want_lse = om.sparse_mla_oracle(qf, rows[:, :n], idx_np, sm_scale=576 ** -0.5, d_v=512)
+    err, ref = error_report(got_out, want_out)
     assert err <= 2e-2 * ref
-    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 5e-3
+    assert np.abs(got_lse - want_lse).max() <= 5e-3
+    with pytest.raises(ValueError, match="batch pitch"):
+        ops.sparse_mla_forward(q, layer.kv[:, :n], idx, sm_scale=sm, d_v=512, out=out, lse=lse,
+                               kv_spec=ops.QuantSpec(_lib.SCALE_F32_BLOCK, layer.scale[:, :n].contiguous(), 128),
+                               kv_rope=layer.rope[:, :n])

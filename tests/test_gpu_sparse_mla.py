@@ -217,12 +217,14 @@ def test_mfma_kernel_matches_scalar_kernel_bf16_cache(device):
         _assert_close(out, lse, want_out, want_lse, lse_tol=LSE_TOL if kernel == "scalar" else LSE_TOL_MFMA)
 
 
-def test_decode_full_config_sampled_batches(device):
+@pytest.mark.parametrize("pow2", [True, False], ids=["pow2_scales", "general_scales"])
+def test_decode_full_config_sampled_batches(device, pow2):
     """B=32, S_q=1, H=128, topk=2048 over a 65536-token FP8 cache (the headline
-    workload): every batch runs on the GPU, two of them are checked against the
-    oracle, and the rest through properties: permuting a query's selected keys
-    leaves its output unchanged (to accumulation order), and appending masked
-    (-1) slots changes nothing."""
+    workload) with power-of-two and with general amax/448 block scales: every batch
+    runs on the GPU, five of them are checked against the oracle, and the rest
+    through properties: permuting a query's selected keys leaves its output
+    unchanged (to accumulation order), and appending masked (-1) slots changes
+    nothing."""
     from cppmega_mlx_amd import _lib
     B, H, Skv, topk = 32, 128, 65536, 2048
     gen = torch.Generator(device=device).manual_seed(5)
@@ -231,7 +233,9 @@ def test_decode_full_config_sampled_batches(device):
     rope = torch.empty((B, Skv, 1, 64), dtype=torch.bfloat16, device=device)
     for b in range(B):
         lat = torch.randn((Skv, 1, 4, 128), generator=gen, device=device)
-        sc = torch.exp2(torch.ceil(torch.log2(lat.abs().amax(dim=-1) / 448.0)))
+        sc = lat.abs().amax(dim=-1) / 448.0
+        if pow2:
+            sc = torch.exp2(torch.ceil(torch.log2(sc)))
         codes[b] = (lat / sc[..., None]).to(torch.float8_e4m3fn).view(torch.uint8).reshape(Skv, 1, 512)
         scale[b] = sc
         rope[b] = torch.randn((Skv, 1, 64), generator=gen, device=device).to(torch.bfloat16)
@@ -249,7 +253,7 @@ def test_decode_full_config_sampled_batches(device):
 
     got_out, got_lse = run(idx)
     assert ops.sparse_mla_selected_kernel(q, codes, idx, d_v=512, kv_spec=spec, kv_rope=rope) == "mfma"
-    for b in (0, 31):
+    for b in (0, 7, 13, 22, 31):
         sel = idx[b, 0, 0].cpu().numpy().astype(np.int64)
         rows = om.dequant_block_latent(codes[b, sel].cpu().numpy(), scale[b, sel].cpu().numpy(),
                                        rope[b, sel].float().cpu().numpy(), 128)[None]
