@@ -15,6 +15,7 @@ from typing import Any
 import torch
 
 ABI_VERSION = 1
+NOALLOC_SCRATCH_BYTES = 20 << 20      # CPPMEGA_MI355_NOALLOC_SCRATCH_BYTES
 LIB_NAME = "libcppmega_mi355.so"
 LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
 
@@ -39,6 +40,7 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_topk_select",
     "cppmega_mi355_sparse_mla_workspace_bytes",
     "cppmega_mi355_sparse_mla_fwd",
+    "cppmega_mi355_sparse_mla_fwd_noalloc",
     "cppmega_mi355_sparse_mla_select_kernel",
     "cppmega_mi355_sparse_mla_scores",
     "cppmega_mi355_fp8_vecmat_workspace_bytes",
@@ -268,7 +270,7 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_last_error.restype = C.c_char_p
         lib.cppmega_mi355_topk_select.argtypes = [C.POINTER(TopkArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_topk_select.restype = C.c_int
-        for name in ("cppmega_mi355_sparse_mla_fwd",):
+        for name in ("cppmega_mi355_sparse_mla_fwd", "cppmega_mi355_sparse_mla_fwd_noalloc"):
             getattr(lib, name).argtypes = [C.POINTER(SparseMlaArgs), C.c_size_t, C.c_void_p]
             getattr(lib, name).restype = C.c_int
         lib.cppmega_mi355_sparse_mla_workspace_bytes.argtypes = [

@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "sparse_mla_common.h"
 
 namespace cm {
@@ -111,6 +113,32 @@ static int pick_mla_kernel(const cppmega_mi355_sparse_mla_args_t& a, const MlaPa
               : -fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla: the MFMA kernel does not cover this shape/dtype");
   if (a.kernel != CPPMEGA_MI355_MLA_KERNEL_AUTO) return -fail(CPPMEGA_MI355_ERR_SHAPE, "sparse_mla: unknown kernel %d", a.kernel);
   return ok ? CPPMEGA_MI355_MLA_KERNEL_MFMA : CPPMEGA_MI355_MLA_KERNEL_SCALAR;
+}
+
+// ---- scratch of the entry point that allocates nothing ------------------------------------
+// The array is part of the code object, so every GPU that loads the library holds its own copy at
+// its own address until the process ends.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress; the address the kernels get is the one looked up per device below.
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[CPPMEGA_MI355_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];          // device address of `scratch`, per device; NULL = not looked up yet
+static std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch` (looked up once per device).
+static int scratch_of_current_device(void** out) {
+  int dev = -1;
+  CM_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "device ordinal %d is outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    CM_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr || ((uintptr_t)ptr & 255)) return fail(CPPMEGA_MI355_ERR_LAUNCH, "static scratch resolved to %p", ptr);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
 }
 
 }  // namespace cm
@@ -220,6 +248,32 @@ int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, si
     return sparse_mla_mfma_launch(p, (hipStream_t)stream);
   }
   return sparse_mla_scalar_launch(p, (hipStream_t)stream);
+}
+
+int cppmega_mi355_sparse_mla_fwd_noalloc(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size, void* stream) {
+  cppmega_mi355_sparse_mla_args_t a;
+  int rc = widen_mla_args(args, args_size, a);
+  if (rc) return rc;
+  MlaParams p;
+  rc = build_mla_params(a, p, true);
+  if (rc) return rc;
+  const int kern = pick_mla_kernel(a, p);
+  if (kern < 0) return -kern;
+  if (kern != CPPMEGA_MI355_MLA_KERNEL_MFMA) return sparse_mla_scalar_launch(p, (hipStream_t)stream);
+  sparse_mla_mfma_plan(p);
+  const size_t need = sparse_mla_mfma_workspace_bytes(p);
+  if (need > (size_t)CPPMEGA_MI355_NOALLOC_SCRATCH_BYTES)
+    return fail(CPPMEGA_MI355_ERR_WORKSPACE,
+                "sparse_mla_fwd_noalloc: these shapes need %zu bytes of scratch, the static array holds %zu; "
+                "use cppmega_mi355_sparse_mla_fwd with a caller workspace", need, (size_t)CPPMEGA_MI355_NOALLOC_SCRATCH_BYTES);
+  p.workspace = nullptr;
+  if (need > 0) {
+    void* ptr = nullptr;
+    rc = scratch_of_current_device(&ptr);
+    if (rc) return rc;
+    p.workspace = ptr;
+  }
+  return sparse_mla_mfma_launch(p, (hipStream_t)stream);
 }
 
 int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size, float* scores,

@@ -180,8 +180,13 @@ def sparse_mla_forward(
     has_sinks: torch.Tensor | None = None,
     kernel: str = "auto",
     workspace: torch.Tensor | None = None,
+    no_alloc: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Sparse MLA forward into caller-owned ``out`` [B,S,H,d_v] (and ``lse`` [B,S,H]).
+
+    ``no_alloc`` takes the entry point whose split-KV partials live in the library's fixed
+    per-GPU array (``_lib.NOALLOC_SCRATCH_BYTES``): no workspace tensor, nothing allocated;
+    shapes that need more raise, and calls overlapping on one GPU must be ordered.
 
     ``sm_scale`` is a Python float or a device float32[1] the kernels read on the stream (the
     reference's ``sm_scale_buf``); ``has_sinks`` is an optional device int32[1] that switches
@@ -209,9 +214,14 @@ def sparse_mla_forward(
         raise ValueError(f"sinks must be float32 with shape ({H},), got {sinks.dtype} {tuple(sinks.shape)}")
     a = _fill_mla_args(q, q_spec, kv, kv_spec, kv_rope, indices, sm_scale, d_v, sinks, out, lse, kernel, has_sinks)
     lib = _lib.load()
+    stream = _lib.current_stream(q.device)
+    if no_alloc:
+        with torch.cuda.device(q.device):
+            rc = lib.cppmega_mi355_sparse_mla_fwd_noalloc(C.byref(a), C.sizeof(a), stream)
+        _lib.check(rc, "sparse_mla_fwd_noalloc")
+        return out, lse
     need = C.c_size_t(0)
     _lib.check(lib.cppmega_mi355_sparse_mla_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)), "sparse_mla")
-    stream = _lib.current_stream(q.device)
     if need.value:
         if workspace is None:
             workspace = _workspace(q.device, need.value, stream)

@@ -209,6 +209,22 @@ int cppmega_mi355_sparse_mla_workspace_bytes(const cppmega_mi355_sparse_mla_args
 int cppmega_mi355_sparse_mla_fwd(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size,
                                  void* stream);
 
+/* cppmega_mi355_sparse_mla_fwd for callers that cannot allocate device memory or
+ * carry a workspace around (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments, kernels and results as cppmega_mi355_sparse_mla_fwd, but the
+ * split-KV partials go to a fixed array of CPPMEGA_MI355_NOALLOC_SCRATCH_BYTES that
+ * is part of the library image on every GPU the library runs on; `workspace` and
+ * `workspace_bytes` of args are ignored, and the call allocates nothing.  A request
+ * whose *_workspace_bytes exceeds the array fails with CPPMEGA_MI355_ERR_WORKSPACE
+ * before anything is launched.  All calls on one GPU share that GPU's array, whose
+ * contents are undefined between calls (nothing in it has to start at zero): two
+ * calls that overlap in time on one GPU, on different streams, race; calls on one
+ * stream, or otherwise ordered, do not. */
+#define CPPMEGA_MI355_NOALLOC_SCRATCH_BYTES (20u << 20)
+int cppmega_mi355_sparse_mla_fwd_noalloc(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size,
+                                         void* stream);
+
 /* Which kernel AUTO resolves to for these shapes (CPPMEGA_MI355_MLA_KERNEL_*),
  * or a negative status code. */
 int cppmega_mi355_sparse_mla_select_kernel(const cppmega_mi355_sparse_mla_args_t* args,
