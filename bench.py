@@ -426,6 +426,18 @@ def bench_next_rows(args, device):
     mask = (torch.arange(K, device=device)[None, :] <= torch.arange(S, device=device)[:, None]).contiguous()
     hbm("mask_indices", lambda: ops.mask_sparse_indices(mask[None, None], out, topk=2048), mask.numel() + out.numel() * 4,
         "sparse_indices_from_attention_mask: bool mask [8192, 8192] -> int32 [1,8192,1,2048]")
+    # indexer scores -> top-k: prefill (causal bounds, no mask read) and one decode step
+    for tag, B, Sq, Skv in (("indexer_prefill", 1, 8192, 8192), ("indexer_decode", 32, 1, 65536)):
+        H, D, topk = 64, 128, 2048
+        q = torch.randn((B, Sq, H, D), generator=gen, device=device).to(torch.bfloat16)
+        kk = torch.randn((B, Skv, D), generator=gen, device=device).to(torch.bfloat16)
+        w = (torch.randn((B, Sq, H), generator=gen, device=device) * H ** -0.5).to(torch.bfloat16)
+        ends = (torch.arange(1, Sq + 1, device=device, dtype=torch.int32) + (Skv - Sq)).repeat(B).contiguous()
+        idx = torch.empty((B, Sq, topk), dtype=torch.int32, device=device)
+        nbytes = (q.numel() + kk.numel() + w.numel()) * 2 + ends.numel() * 4 + idx.numel() * 4
+        hbm(tag, lambda q=q, kk=kk, w=w, ends=ends, idx=idx: ops.indexer_topk(q, kk, w, sm_scale=D ** -0.5, topk=topk, out=idx, ends=ends),
+            nbytes, f"indexer_topk q bf16[{B},{Sq},{H},{D}] k bf16[{B},{Skv},{D}] -> int32[{B},{Sq},{topk}] "
+                    f"(scores stay in a {ops.indexer_topk_workspace_bytes(q, kk, w, topk=topk) >> 20} MiB chunk buffer)")
     return res
 
 

@@ -38,6 +38,8 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_error_string",
     "cppmega_mi355_last_error",
     "cppmega_mi355_topk_select",
+    "cppmega_mi355_indexer_topk_workspace_bytes",
+    "cppmega_mi355_indexer_topk",
     "cppmega_mi355_sparse_mla_workspace_bytes",
     "cppmega_mi355_sparse_mla_fwd",
     "cppmega_mi355_sparse_mla_fwd_noalloc",
@@ -90,6 +92,35 @@ class TopkArgs(C.Structure):
         ("indices", C.c_void_p),
         ("neg_inf_is_masked", C.c_int32),
         ("reserved", C.c_int32),
+    ]
+
+
+class IndexerArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("q_dtype", C.c_int32),
+        ("q", C.c_void_p),
+        ("weights", C.c_void_p),
+        ("k", C.c_void_p),
+        ("mask", C.c_void_p),
+        ("w_dtype", C.c_int32),
+        ("k_dtype", C.c_int32),
+        ("mask_dtype", C.c_int32),
+        ("order", C.c_int32),
+        ("starts", C.c_void_p),
+        ("ends", C.c_void_p),
+        ("batch", C.c_int32),
+        ("seq_q", C.c_int32),
+        ("heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("seq_kv", C.c_int32),
+        ("topk", C.c_int32),
+        ("sm_scale", C.c_float),
+        ("chunk_rows", C.c_int32),
+        ("indices", C.c_void_p),
+        ("scores_out", C.c_void_p),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
     ]
 
 
@@ -270,6 +301,10 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_last_error.restype = C.c_char_p
         lib.cppmega_mi355_topk_select.argtypes = [C.POINTER(TopkArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_topk_select.restype = C.c_int
+        lib.cppmega_mi355_indexer_topk.argtypes = [C.POINTER(IndexerArgs), C.c_size_t, C.c_void_p]
+        lib.cppmega_mi355_indexer_topk.restype = C.c_int
+        lib.cppmega_mi355_indexer_topk_workspace_bytes.argtypes = [C.POINTER(IndexerArgs), C.c_size_t, C.POINTER(C.c_size_t)]
+        lib.cppmega_mi355_indexer_topk_workspace_bytes.restype = C.c_int
         for name in ("cppmega_mi355_sparse_mla_fwd", "cppmega_mi355_sparse_mla_fwd_noalloc"):
             getattr(lib, name).argtypes = [C.POINTER(SparseMlaArgs), C.c_size_t, C.c_void_p]
             getattr(lib, name).restype = C.c_int

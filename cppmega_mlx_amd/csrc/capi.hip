@@ -35,6 +35,8 @@ int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stre
 int kv_cache_append_launch(const cppmega_mi355_cache_append_args_t& a, hipStream_t stream);
 int causal_indices_launch(const cppmega_mi355_causal_indices_args_t& a, hipStream_t stream);
 int mask_indices_launch(const cppmega_mi355_mask_indices_args_t& a, hipStream_t stream);
+int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t stream);
+int indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t& a, size_t* bytes);
 
 static bool is_float_carrier(int dt) {
   return dt == CPPMEGA_MI355_F32 || dt == CPPMEGA_MI355_F16 || dt == CPPMEGA_MI355_BF16;
@@ -199,6 +201,17 @@ int cppmega_mi355_status(cppmega_mi355_status_t* out, size_t out_size) {
 int cppmega_mi355_topk_select(const cppmega_mi355_topk_args_t* args, size_t args_size, void* stream) {
   CM_CHECK_ARGS(args, args_size, cppmega_mi355_topk_args_t);
   return topk_select_launch(*args, (hipStream_t)stream);
+}
+
+int cppmega_mi355_indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t* args, size_t args_size, size_t* bytes) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_indexer_args_t);
+  if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "bytes is NULL");
+  return indexer_topk_workspace_bytes(*args, bytes);
+}
+
+int cppmega_mi355_indexer_topk(const cppmega_mi355_indexer_args_t* args, size_t args_size, void* stream) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_indexer_args_t);
+  return indexer_topk_launch(*args, (hipStream_t)stream);
 }
 
 int cppmega_mi355_sparse_mla_select_kernel(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size) {

@@ -97,6 +97,94 @@ def topk_select(
 
 
 # ---------------------------------------------------------------------------
+# indexer scores -> top-k
+# ---------------------------------------------------------------------------
+def _fill_indexer_args(q, k, weights, sm_scale, topk, out, mask, starts, ends, order, scores_out, chunk_rows):
+    if q.ndim != 4 or k.ndim != 3 or weights.ndim != 3:
+        raise ValueError("indexer expects q [B,Sq,H,D], k [B,Skv,D], weights [B,Sq,H]")
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    if tuple(weights.shape) != (B, Sq, H) or k.shape[0] != B or k.shape[2] != D:
+        raise ValueError(f"indexer shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, weights {tuple(weights.shape)}")
+    if order not in ("index", "value"):
+        raise ValueError(f"unknown order {order!r}")
+    a = _lib.IndexerArgs()
+    a.struct_size = C.sizeof(a)
+    a.q_dtype = _dtype_or_raise(q, "q", (_lib.F32, _lib.BF16))
+    a.w_dtype = _dtype_or_raise(weights, "weights", (_lib.F32, _lib.BF16))
+    a.k_dtype = _dtype_or_raise(k, "k", (_lib.F32, _lib.BF16))
+    a.q, a.weights, a.k = q.data_ptr(), weights.data_ptr(), k.data_ptr()
+    if mask is not None:
+        if tuple(mask.shape) != (B, Sq, Skv):
+            raise ValueError(f"mask must have shape {(B, Sq, Skv)}; got {tuple(mask.shape)}")
+        a.mask, a.mask_dtype = mask.data_ptr(), _dtype_or_raise(mask, "mask", (_lib.F32, _lib.F16, _lib.BF16))
+    for name, bound in (("starts", starts), ("ends", ends)):
+        if bound is not None and (bound.numel() != B * Sq or bound.dtype != torch.int32):
+            raise ValueError(f"{name} must be int32 with {B * Sq} entries; got {bound.dtype} {tuple(bound.shape)}")
+    a.starts, a.ends = _lib.ptr(starts), _lib.ptr(ends)
+    a.order = _lib.TOPK_ORDER_VALUE if order == "value" else _lib.TOPK_ORDER_INDEX
+    a.batch, a.seq_q, a.heads, a.head_dim, a.seq_kv, a.topk = B, Sq, H, D, Skv, int(topk)
+    a.sm_scale = float(sm_scale)
+    a.chunk_rows = int(chunk_rows)
+    if out is not None:
+        if out.dtype != torch.int32 or tuple(out.shape) != (B, Sq, int(topk)):
+            raise ValueError(f"out must be int32 with shape {(B, Sq, int(topk))}; got {out.dtype} {tuple(out.shape)}")
+        a.indices = out.data_ptr()
+    if scores_out is not None:
+        if scores_out.dtype != torch.float32 or tuple(scores_out.shape) != (B, Sq, Skv):
+            raise ValueError(f"scores_out must be float32 with shape {(B, Sq, Skv)}")
+        a.scores_out = scores_out.data_ptr()
+    return a
+
+
+def indexer_topk_workspace_bytes(q, k, weights, *, topk: int, chunk_rows: int = 0) -> int:
+    a = _fill_indexer_args(q, k, weights, 1.0, topk, None, None, None, None, "index", None, chunk_rows)
+    need = C.c_size_t(0)
+    _lib.check(_lib.load().cppmega_mi355_indexer_topk_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)), "indexer_topk")
+    return int(need.value)
+
+
+def indexer_topk(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    weights: torch.Tensor,
+    *,
+    sm_scale: float,
+    topk: int,
+    out: torch.Tensor,
+    mask: torch.Tensor | None = None,
+    starts: torch.Tensor | None = None,
+    ends: torch.Tensor | None = None,
+    order: str = "index",
+    scores_out: torch.Tensor | None = None,
+    workspace: torch.Tensor | None = None,
+    chunk_rows: int = 0,
+) -> torch.Tensor:
+    """indices[b,s,:] = top-k over t of sm_scale * sum_h weights[b,s,h] * (q[b,s,h,:] . k[b,t,:]) (+ mask),
+    into caller-owned int32 ``out`` [B,Sq,topk].  ``scores_out`` (float32 [B,Sq,Skv]) keeps every score."""
+    for name, t in (("q", q), ("k", k), ("weights", weights), ("out", out), ("mask", mask), ("starts", starts),
+                    ("ends", ends), ("scores_out", scores_out)):
+        if t is not None:
+            _lib.require_device_tensor(t, name, q if name != "q" else None)
+    a = _fill_indexer_args(q, k, weights, sm_scale, topk, out, mask, starts, ends, order, scores_out, chunk_rows)
+    lib = _lib.load()
+    stream = _lib.current_stream(q.device)
+    need = C.c_size_t(0)
+    _lib.check(lib.cppmega_mi355_indexer_topk_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)), "indexer_topk")
+    if need.value:
+        if workspace is None:
+            workspace = _workspace(q.device, need.value, stream)
+        else:
+            _lib.require_device_tensor(workspace, "workspace", q)
+        a.workspace = workspace.data_ptr()
+        a.workspace_bytes = workspace.numel() * workspace.element_size()
+    with torch.cuda.device(q.device):
+        rc = lib.cppmega_mi355_indexer_topk(C.byref(a), C.sizeof(a), stream)
+    _lib.check(rc, "indexer_topk")
+    return out
+
+
+# ---------------------------------------------------------------------------
 # sparse MLA
 # ---------------------------------------------------------------------------
 

@@ -114,6 +114,56 @@ typedef struct cppmega_mi355_topk_args {
 
 int cppmega_mi355_topk_select(const cppmega_mi355_topk_args_t* args, size_t args_size, void* stream);
 
+/* ---- indexer scores -> top-k -------------------------------------------------
+ * The score and selection tail of the reference's LightningIndexer.__call__
+ * (cppmega_v4/nn/lightning_indexer.py:132-145; the FP8 variant has the same
+ * lines, cppmega_v4/nn/lightning_indexer_fp8.py:145-157):
+ *   scores[b,s,t]  = sm_scale * sum_h weights[b,s,h] * sum_d q[b,s,h,d] * k[b,t,d]
+ *                    (+ mask[b,s,t])
+ *   indices[b,s,:] = the topk largest of scores[b,s,:]
+ *   q        [B, Sq, H, D]   float32 or bfloat16 (D <= 256)
+ *   weights  [B, Sq, H]      float32 or bfloat16 (the caller has applied H^-1/2)
+ *   k        [B, Skv, D]     float32 or bfloat16
+ *   mask     [B, Sq, Skv]    additive, float32/float16/bfloat16, or NULL
+ *   starts, ends  [B*Sq] int32 or NULL: selectable window per query row, as in
+ *            cppmega_mi355_topk_select (a causal bound costs no mask read)
+ *   indices  [B, Sq, topk] int32.  Selection rule of cppmega_mi355_topk_select:
+ *            value descending, ties toward the lower index; a slot beyond the
+ *            selectable entries of a row holds -1 (with a mask, an entry whose
+ *            score is -inf is not selectable; the reference's argpartition picks
+ *            arbitrary masked positions there).
+ * The [B,Sq,Skv] score matrix is not kept: rows are scored and selected a chunk at
+ * a time through `workspace` (*_workspace_bytes; 256 MiB of scores per pass by
+ * default, `chunk_rows` overrides the rows per pass; the head-summed queries of a
+ * pass live there too).  When `scores_out` is set every score is written there
+ * instead (float32 [B,Sq,Skv], 16-byte aligned) in one pass and the selection
+ * reads exactly those values; the workspace then only holds the summed queries. */
+typedef struct cppmega_mi355_indexer_args {
+  uint32_t struct_size;
+  int32_t q_dtype;
+  const void* q;
+  const void* weights;
+  const void* k;
+  const void* mask;
+  int32_t w_dtype;
+  int32_t k_dtype;
+  int32_t mask_dtype;
+  int32_t order;              /* CPPMEGA_MI355_TOPK_ORDER_*                    */
+  const int32_t* starts;
+  const int32_t* ends;
+  int32_t batch, seq_q, heads, head_dim, seq_kv, topk;
+  float sm_scale;
+  int32_t chunk_rows;         /* 0 = the library's choice                      */
+  int32_t* indices;
+  float* scores_out;
+  void* workspace;
+  size_t workspace_bytes;
+} cppmega_mi355_indexer_args_t;
+
+int cppmega_mi355_indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t* args, size_t args_size,
+                                               size_t* bytes);
+int cppmega_mi355_indexer_topk(const cppmega_mi355_indexer_args_t* args, size_t args_size, void* stream);
+
 /* ---- sparse MLA forward ----------------------------------------------------
  * One entry point for the three prepared-buffer kernels of the reference and
  * the float-carrier one:

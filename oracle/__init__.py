@@ -30,6 +30,9 @@ Pinning status (what fixes each function besides its own formula):
   formulation, ``torch.softmax`` / ``torch.logsumexp`` closed forms and the
   invariants the reference tests pin (all-invalid row -> zeros, duplicated
   index = doubled weight, permutation invariance).
+* ``indexer.indexer_scores_oracle`` / ``indexer_topk_oracle`` -- pinned against an
+  explicit four-loop evaluation, the head-sum-first identity, ``np.argpartition``'s
+  set on distinct scores and the reference's rope known answers.
 * ``vecmat.*``                   -- pinned against float64 ``W_deq @ x`` with
   torch's independent e4m3 decoder.
 """

@@ -38,6 +38,7 @@ def test_status_probe_reports_abi_and_arch():
 STRUCTS = {
     "cppmega_mi355_status_t": _lib.StatusStruct,
     "cppmega_mi355_topk_args_t": _lib.TopkArgs,
+    "cppmega_mi355_indexer_args_t": _lib.IndexerArgs,
     "cppmega_mi355_sparse_mla_args_t": _lib.SparseMlaArgs,
     "cppmega_mi355_vecmat_args_t": _lib.VecmatArgs,
     "cppmega_mi355_quantize_args_t": _lib.QuantizeArgs,
