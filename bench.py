@@ -438,6 +438,14 @@ def bench_next_rows(args, device):
         hbm(tag, lambda q=q, kk=kk, w=w, ends=ends, idx=idx: ops.indexer_topk(q, kk, w, sm_scale=D ** -0.5, topk=topk, out=idx, ends=ends),
             nbytes, f"indexer_topk q bf16[{B},{Sq},{H},{D}] k bf16[{B},{Skv},{D}] -> int32[{B},{Sq},{topk}] "
                     f"(scores stay in a {ops.indexer_topk_workspace_bytes(q, kk, w, topk=topk) >> 20} MiB chunk buffer)")
+    # the per-head projections either side of the decode attention call (bf16 weights, 32 sequences)
+    B, H, D_k, D_kv, D_v = 32, 128, 128, 512, 128
+    for tag, K, N in (("absorb_query", D_k, D_kv), ("unabsorb_output", D_kv, D_v)):
+        x = torch.randn((B, H, K), generator=gen, device=device).to(torch.bfloat16)
+        w = (torch.randn((H, N, K), generator=gen, device=device) * K ** -0.5).to(torch.bfloat16)
+        y = torch.empty((B, H, N), dtype=torch.bfloat16, device=device)
+        hbm(tag, lambda x=x, w=w, y=y: ops.head_gemm(x, w, out=y), (x.numel() + w.numel() + y.numel()) * 2,
+            f"head_gemm x bf16[{B},{H},{K}] . W bf16[{H},{N},{K}] -> bf16[{B},{H},{N}]")
     return res
 
 

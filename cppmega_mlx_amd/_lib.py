@@ -48,6 +48,8 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_fp8_vecmat_workspace_bytes",
     "cppmega_mi355_fp8_vecmat",
     "cppmega_mi355_fp8_quantize",
+    "cppmega_mi355_head_gemm",
+    "cppmega_mi355_dequant_block_fp8",
     "cppmega_mi355_kv_cache_append",
     "cppmega_mi355_causal_sparse_indices",
     "cppmega_mi355_mask_sparse_indices",
@@ -121,6 +123,38 @@ class IndexerArgs(C.Structure):
         ("scores_out", C.c_void_p),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class HeadGemmArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("x_dtype", C.c_int32),
+        ("x", C.c_void_p),
+        ("w", C.c_void_p),
+        ("y", C.c_void_p),
+        ("w_dtype", C.c_int32),
+        ("y_dtype", C.c_int32),
+        ("m", C.c_int32),
+        ("groups", C.c_int32),
+        ("n", C.c_int32),
+        ("k", C.c_int32),
+        ("x_row_pitch", C.c_int64),
+        ("x_group_pitch", C.c_int64),
+        ("y_row_pitch", C.c_int64),
+        ("y_group_pitch", C.c_int64),
+    ]
+
+
+class DequantBlockArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("out_dtype", C.c_int32),
+        ("weight", C.c_void_p),
+        ("scale_inv", C.c_void_p),
+        ("out", C.c_void_p),
+        ("rows", C.c_int32),
+        ("cols", C.c_int32),
     ]
 
 
@@ -319,6 +353,10 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_fp8_vecmat.restype = C.c_int
         lib.cppmega_mi355_fp8_quantize.argtypes = [C.POINTER(QuantizeArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_fp8_quantize.restype = C.c_int
+        lib.cppmega_mi355_head_gemm.argtypes = [C.POINTER(HeadGemmArgs), C.c_size_t, C.c_void_p]
+        lib.cppmega_mi355_head_gemm.restype = C.c_int
+        lib.cppmega_mi355_dequant_block_fp8.argtypes = [C.POINTER(DequantBlockArgs), C.c_size_t, C.c_void_p]
+        lib.cppmega_mi355_dequant_block_fp8.restype = C.c_int
         for fn, struct in ((lib.cppmega_mi355_kv_cache_append, CacheAppendArgs),
                            (lib.cppmega_mi355_causal_sparse_indices, CausalIndicesArgs),
                            (lib.cppmega_mi355_mask_sparse_indices, MaskIndicesArgs)):

@@ -185,6 +185,68 @@ def indexer_topk(
 
 
 # ---------------------------------------------------------------------------
+# per-head projections (absorbed MLA decode) and block-128 FP8 weight dequantisation
+# ---------------------------------------------------------------------------
+def head_gemm(x: torch.Tensor, w: torch.Tensor, *, out: torch.Tensor) -> torch.Tensor:
+    """out[m, g, n] = sum_k x[m, g, k] * w[g, n, k] into caller-owned ``out``.
+
+    ``x`` [M, G, K] and ``out`` [M, G, N] may be views with their own row and group strides (the
+    last axis contiguous); ``w`` [G, N, K] is dense.  float32 / bfloat16 operands, fp32 accumulation."""
+    for name, t in (("x", x), ("w", w), ("out", out)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch.Tensor")
+        if not t.is_cuda:
+            raise _lib.NativeCallError(_lib.ERR_UNSUPPORTED, f"{name} lives on {t.device}; there is no CPU path")
+    if x.ndim != 3 or w.ndim != 3 or out.ndim != 3:
+        raise ValueError("head_gemm expects x [M,G,K], w [G,N,K], out [M,G,N]")
+    M, G, K = x.shape
+    N = w.shape[1]
+    if tuple(w.shape) != (G, N, K) or tuple(out.shape) != (M, G, N):
+        raise ValueError(f"head_gemm shape mismatch: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    if not w.is_contiguous():
+        raise ValueError("head_gemm: w must be dense [G, N, K] (the contraction index contiguous)")
+    for name, t in (("x", x), ("out", out)):
+        if t.shape[-1] > 1 and t.stride(-1) != 1:
+            raise ValueError(f"head_gemm: the last axis of {name} must be contiguous; got strides {t.stride()}")
+    a = _lib.HeadGemmArgs()
+    a.struct_size = C.sizeof(a)
+    a.x_dtype = _dtype_or_raise(x, "x", (_lib.F32, _lib.BF16))
+    a.w_dtype = _dtype_or_raise(w, "w", (_lib.F32, _lib.BF16))
+    a.y_dtype = _dtype_or_raise(out, "out", (_lib.F32, _lib.F16, _lib.BF16))
+    a.x, a.w, a.y = x.data_ptr(), w.data_ptr(), out.data_ptr()
+    a.m, a.groups, a.n, a.k = M, G, N, K
+    a.x_row_pitch, a.x_group_pitch = x.stride(0), x.stride(1)
+    a.y_row_pitch, a.y_group_pitch = out.stride(0), out.stride(1)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().cppmega_mi355_head_gemm(C.byref(a), C.sizeof(a), _lib.current_stream(x.device))
+    _lib.check(rc, "head_gemm")
+    return out
+
+
+def dequant_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, *, out: torch.Tensor) -> torch.Tensor:
+    """out[r, c] = dec(weight[r, c]) * scale_inv[r // 128, c // 128] (e4m3 bytes, float32 scales)."""
+    for name, t in (("weight", weight), ("scale_inv", scale_inv), ("out", out)):
+        _lib.require_device_tensor(t, name, weight if name != "weight" else None)
+    if weight.ndim != 2 or weight.dtype != torch.uint8:
+        raise TypeError(f"weight must be 2D uint8 (fp8 storage); got {weight.dtype} {tuple(weight.shape)}")
+    m, n = weight.shape
+    want = ((m + 127) // 128, (n + 127) // 128)
+    if tuple(scale_inv.shape) != want or scale_inv.dtype != torch.float32:
+        raise ValueError(f"scale_inv must be float32 with shape {want}; got {scale_inv.dtype} {tuple(scale_inv.shape)}")
+    if tuple(out.shape) != (m, n):
+        raise ValueError(f"out must have shape {(m, n)}; got {tuple(out.shape)}")
+    a = _lib.DequantBlockArgs()
+    a.struct_size = C.sizeof(a)
+    a.out_dtype = _dtype_or_raise(out, "out", (_lib.F32, _lib.F16, _lib.BF16))
+    a.weight, a.scale_inv, a.out = weight.data_ptr(), scale_inv.data_ptr(), out.data_ptr()
+    a.rows, a.cols = m, n
+    with torch.cuda.device(weight.device):
+        rc = _lib.load().cppmega_mi355_dequant_block_fp8(C.byref(a), C.sizeof(a), _lib.current_stream(weight.device))
+    _lib.check(rc, "dequant_block_fp8")
+    return out
+
+
+# ---------------------------------------------------------------------------
 # sparse MLA
 # ---------------------------------------------------------------------------
 

@@ -329,6 +329,53 @@ int cppmega_mi355_fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t* 
 
 int cppmega_mi355_fp8_vecmat(const cppmega_mi355_vecmat_args_t* args, size_t args_size, void* stream);
 
+/* ---- per-head projections of the absorbed MLA decode ----------------------------
+ * Y[m, g, n] = sum_k X[m, g, k] * W[g, n, k]: one skinny matrix product per group g.
+ * Replaces the two einsums that bracket the attention call in the reference's
+ * absorbed_mla_decode (cppmega_v4/nn/mla_absorb.py:116-134):
+ *   "bthk,hkv->bthv"  q_abs = q . W_UK^T[h]:   m = b*t rows, g = h, k = D_k, n = D_kv,
+ *                     W[h][v][k] = w_uk[h][v][k] (the layout absorb_weights :39-77 is given)
+ *   "bthv,hvm->btm"   out = sum_h v_abs . (W_UV W_O)[h]: one group, k = H*D_kv,
+ *                     W[0][m][h*D_kv + v] = w_uv_w_o[h][v][m]
+ * and serves the per-head un-absorb o[b,t,h,:] . W_UV[h] (g = h, k = D_kv, n = D_v).
+ *   x   [M, G, K] float32 or bfloat16; row pitch x_row_pitch, group pitch x_group_pitch
+ *       (elements), k contiguous
+ *   w   [G, N, K] float32 or bfloat16, dense: the contraction index is contiguous
+ *   y   [M, G, N] float32 / float16 / bfloat16 with its own row and group pitch, so a
+ *       result can land inside wider rows (q_abs inside [.., D_kv + rope] query rows)
+ * fp32 accumulation; float32 operands enter the matrix cores as bf16 hi + lo pairs
+ * (16 significand bits). */
+typedef struct cppmega_mi355_head_gemm_args {
+  uint32_t struct_size;
+  int32_t x_dtype;
+  const void* x;
+  const void* w;
+  void* y;
+  int32_t w_dtype;
+  int32_t y_dtype;
+  int32_t m, groups, n, k;
+  int64_t x_row_pitch, x_group_pitch;
+  int64_t y_row_pitch, y_group_pitch;
+} cppmega_mi355_head_gemm_args_t;
+
+int cppmega_mi355_head_gemm(const cppmega_mi355_head_gemm_args_t* args, size_t args_size, void* stream);
+
+/* dequant_block_fp8 (cppmega_v4/nn/_external/_mlx_lm_fp8_dequant_vendored.py:24-46), the
+ * tensor step of sanitize_fp8_weights (:50-71): out[r, c] = dec(weight[r, c]) *
+ * scale_inv[r / 128, c / 128], weight e4m3 bytes [rows, cols], scale_inv float32
+ * [ceil(rows/128), ceil(cols/128)], out [rows, cols] bfloat16 (float16 / float32 also
+ * accepted).  The bytes 0x7F / 0xFF decode to NaN. */
+typedef struct cppmega_mi355_dequant_block_args {
+  uint32_t struct_size;
+  int32_t out_dtype;
+  const void* weight;
+  const float* scale_inv;
+  void* out;
+  int32_t rows, cols;
+} cppmega_mi355_dequant_block_args_t;
+
+int cppmega_mi355_dequant_block_fp8(const cppmega_mi355_dequant_block_args_t* args, size_t args_size, void* stream);
+
 /* ---- FP8 producers ------------------------------------------------------------
  * The quantisers that write the prepared buffers of the attention entry points, and the
  * matching dequantiser:
