@@ -337,6 +337,18 @@ def bench_topk(args, device):
         "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic("topk_selector")},
     }
+    # the decode-time shape: one row per sequence over the whole cache, two-stage selection
+    from cppmega_mlx_amd import ops
+    wide = [torch.randn((32, 65536), generator=gen, device=device) for _ in range(n_sets)]
+    wide_out = torch.empty((32, k), dtype=torch.int32, device=device)
+    for name, two_stage in (("decode_shape", True), ("decode_shape_one_workgroup_per_row", False)):
+        secs, _ = timed_graph([lambda i=i: ops.topk_select(wide[i], k, out=wide_out, two_stage=two_stage) for i in range(n_sets)],
+                              steps, args.warmup)
+        nbytes = 32 * 65536 * 4 + 32 * k * 4
+        res[name] = {"workload": "topk_selector scores fp32[32,65536] -> int32[32,2048]", "us_per_launch": secs / steps * 1e6,
+                     "algorithmic_bytes": nbytes,
+                     "roofline": {"bound": "hbm", "achieved": nbytes / (secs / steps) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": nbytes / (secs / steps) / 1e9 / HBM_PEAK_GBS, "traffic": None}}
     return res, (scores[0], ends, outs[0], k)
 
 

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_error_string",
     "cppmega_mi355_last_error",
     "cppmega_mi355_topk_select",
+    "cppmega_mi355_topk_workspace_bytes",
     "cppmega_mi355_indexer_topk_workspace_bytes",
     "cppmega_mi355_indexer_topk",
     "cppmega_mi355_sparse_mla_workspace_bytes",
@@ -94,7 +95,12 @@ class TopkArgs(C.Structure):
         ("indices", C.c_void_p),
         ("neg_inf_is_masked", C.c_int32),
         ("reserved", C.c_int32),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
     ]
+
+
+TOPK_ARGS_V1_SIZE = TopkArgs.workspace.offset
 
 
 class IndexerArgs(C.Structure):
@@ -335,6 +341,8 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_last_error.restype = C.c_char_p
         lib.cppmega_mi355_topk_select.argtypes = [C.POINTER(TopkArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_topk_select.restype = C.c_int
+        lib.cppmega_mi355_topk_workspace_bytes.argtypes = [C.POINTER(TopkArgs), C.c_size_t, C.POINTER(C.c_size_t)]
+        lib.cppmega_mi355_topk_workspace_bytes.restype = C.c_int
         lib.cppmega_mi355_indexer_topk.argtypes = [C.POINTER(IndexerArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_indexer_topk.restype = C.c_int
         lib.cppmega_mi355_indexer_topk_workspace_bytes.argtypes = [C.POINTER(IndexerArgs), C.c_size_t, C.POINTER(C.c_size_t)]

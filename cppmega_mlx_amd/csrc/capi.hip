@@ -29,6 +29,7 @@ int fail(int code, const char* fmt, ...) {
 }
 
 int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream);
+int topk_workspace_bytes(const cppmega_mi355_topk_args_t& a, size_t* bytes);
 int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream);
 int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes);
 int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stream);
@@ -200,9 +201,31 @@ int cppmega_mi355_status(cppmega_mi355_status_t* out, size_t out_size) {
   return CPPMEGA_MI355_OK;
 }
 
+// Copies the caller's top-k struct into the current layout (zeros for fields appended after the first ABI).
+static int widen_topk_args(const cppmega_mi355_topk_args_t* args, size_t args_size, cppmega_mi355_topk_args_t& a) {
+  if (!args) return fail(CPPMEGA_MI355_ERR_NULL, "args is NULL");
+  const size_t have = args_size < (size_t)args->struct_size ? args_size : (size_t)args->struct_size;
+  if (have < CPPMEGA_MI355_TOPK_ARGS_V1_SIZE)
+    return fail(CPPMEGA_MI355_ERR_STRUCT_SIZE, "args struct is %zu/%u bytes, need %zu", args_size, args->struct_size,
+                (size_t)CPPMEGA_MI355_TOPK_ARGS_V1_SIZE);
+  memset(&a, 0, sizeof(a));
+  memcpy(&a, args, have < sizeof(a) ? have : sizeof(a));
+  return 0;
+}
+
 int cppmega_mi355_topk_select(const cppmega_mi355_topk_args_t* args, size_t args_size, void* stream) {
-  CM_CHECK_ARGS(args, args_size, cppmega_mi355_topk_args_t);
-  return topk_select_launch(*args, (hipStream_t)stream);
+  cppmega_mi355_topk_args_t a;
+  const int rc = widen_topk_args(args, args_size, a);
+  if (rc) return rc;
+  return topk_select_launch(a, (hipStream_t)stream);
+}
+
+int cppmega_mi355_topk_workspace_bytes(const cppmega_mi355_topk_args_t* args, size_t args_size, size_t* bytes) {
+  cppmega_mi355_topk_args_t a;
+  const int rc = widen_topk_args(args, args_size, a);
+  if (rc) return rc;
+  if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "bytes is NULL");
+  return topk_workspace_bytes(a, bytes);
 }
 
 int cppmega_mi355_indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t* args, size_t args_size, size_t* bytes) {

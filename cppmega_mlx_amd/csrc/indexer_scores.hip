@@ -37,6 +37,7 @@
 namespace cm {
 
 int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream);
+int topk_workspace_bytes(const cppmega_mi355_topk_args_t& a, size_t* bytes);
 
 namespace {
 
@@ -294,6 +295,7 @@ struct Plan {
   int batches_per_pass;  // batches per pass (when whole batches fit), else 1
   size_t score_bytes;    // bytes of the score chunk
   size_t qw_bytes;       // bytes of the head-summed queries of one pass (bf16 hi + lo planes)
+  size_t topk_bytes;     // candidate buffers of the selector's two-stage path (wide rows)
 };
 
 constexpr size_t kChunkBytes = (size_t)256 << 20;
@@ -318,7 +320,12 @@ Plan make_plan(const cppmega_mi355_indexer_args_t& a) {
   }
   const size_t rows = (size_t)pl.rows_per_pass * (size_t)pl.batches_per_pass;
   pl.score_bytes = a.scores_out ? 0 : ((rows * row_bytes + 255) & ~(size_t)255);
-  pl.qw_bytes = rows * (size_t)((a.head_dim + 31) & ~31) * 2 * 2;
+  pl.qw_bytes = (rows * (size_t)((a.head_dim + 31) & ~31) * 2 * 2 + 255) & ~(size_t)255;
+  cppmega_mi355_topk_args_t t;
+  memset(&t, 0, sizeof(t));
+  t.rows = (int)rows; t.width = a.seq_kv; t.row_stride = a.seq_kv; t.k = a.topk;
+  pl.topk_bytes = 0;
+  if (a.topk >= 1 && a.topk <= a.seq_kv) (void)topk_workspace_bytes(t, &pl.topk_bytes);
   return pl;
 }
 
@@ -348,7 +355,7 @@ int indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t& a, size_t* 
   const int rc = validate(a, false);
   if (rc) return rc;
   const Plan pl = make_plan(a);
-  *bytes = pl.score_bytes + pl.qw_bytes;
+  *bytes = pl.score_bytes + pl.qw_bytes + pl.topk_bytes;
   return 0;
 }
 
@@ -368,7 +375,7 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
   if (rc) return rc;
   if ((size_t)a.batch * a.seq_q == 0) return 0;
   const Plan pl = make_plan(a);
-  const size_t need = pl.score_bytes + pl.qw_bytes;
+  const size_t need = pl.score_bytes + pl.qw_bytes + pl.topk_bytes;
   if (!a.workspace || a.workspace_bytes < need)
     return fail(CPPMEGA_MI355_ERR_WORKSPACE, "indexer: workspace of %zu bytes needed, %zu given", need,
                 a.workspace ? a.workspace_bytes : (size_t)0);
@@ -422,6 +429,10 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
       t.ends = a.ends ? a.ends + row0 : nullptr;
       t.indices = a.indices + row0 * (size_t)a.topk;
       t.neg_inf_is_masked = a.mask ? 1 : 0;
+      if (pl.topk_bytes) {
+        t.workspace = (char*)a.workspace + pl.score_bytes + pl.qw_bytes;
+        t.workspace_bytes = pl.topk_bytes;
+      }
       rc = topk_select_launch(t, stream);
       if (rc) return rc;
     }

@@ -49,6 +49,15 @@ struct TopkParams {
   int* out;
   int rows, width, k, order, neg_inf_masked;
   int sort_len;  // power of two >= k, used by the value-descending order
+  // Rows too wide for one workgroup's fast path are selected in two stages (tile kernel only):
+  // stage 1 launches one workgroup per (row, segment of seg_width columns) and writes the
+  // segment's k best as candidates (value, column) in ascending column order; stage 2 selects
+  // among a row's segs * k candidates and translates positions through index_map.
+  int segs;             // > 1: stage 1; blockIdx.x = row * segs + segment, width = columns of the whole row
+  int seg_width;
+  float* cand_val;      // stage 1 out: [rows, segs, k] (NaN = no candidate)
+  int* cand_idx;        // stage 1 out: [rows, segs, k] (-1 = no candidate)
+  const int* index_map; // stage 2 in: [rows, width] column of each candidate position
 };
 
 struct Half {};   // tag types: 16-bit storage
@@ -217,7 +226,9 @@ constexpr int kTileThreads = 256;
 constexpr int kTileScratch = kHistBins + 64;            // words: histogram + scan scratch
 __host__ __device__ constexpr int tile_pad(int E) { return E == 4 ? 0 : 4; }
 
-template <typename ScoreT, int E, int VEC, int THREADS = kTileThreads>
+// MODE 0: a row per workgroup.  MODE 1: stage 1 of a wide row (a segment per workgroup, candidates
+// out).  MODE 2: stage 2 (a row of candidates per workgroup, positions translated through index_map).
+template <typename ScoreT, int E, int VEC, int THREADS = kTileThreads, int MODE = 0>
 __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) {
   constexpr int ITEMS = E / VEC;                        // loads per thread
   constexpr int CHUNK = THREADS * VEC;                  // columns covered by one load per thread
@@ -228,13 +239,15 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
   typedef typename Storage<ScoreT>::type St;
 
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int row = (int)blockIdx.x;
-  const int T = p.width;
-  int start = p.starts ? p.starts[row] : 0;
-  int end = p.ends ? p.ends[row] : T;
+  constexpr bool stage1 = MODE == 1;
+  const int row = stage1 ? (int)blockIdx.x / p.segs : (int)blockIdx.x;
+  const int base = stage1 ? ((int)blockIdx.x % p.segs) * p.seg_width : 0;   // first column of this workgroup's share
+  const int T = stage1 ? min(p.seg_width, p.width - base) : p.width;
+  int start = (p.starts ? p.starts[row] : 0) - base;
+  int end = (p.ends ? p.ends[row] : p.width) - base;
   start = min(max(start, 0), T);
   end = min(max(end, 0), T);
-  const St* src = reinterpret_cast<const St*>(p.scores) + (long long)row * p.row_stride;
+  const St* src = reinterpret_cast<const St*>(p.scores) + (long long)row * p.row_stride + base;
   int* out_row = p.out + (long long)row * p.k;
   const float kNaN = __uint_as_float(0x7fc00000u);
   const float kNegInf = __uint_as_float(0xff800000u);
@@ -392,9 +405,21 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
   }
   if (!sorted) {
     __syncthreads();
-    for (unsigned i = tid; i < k; i += THREADS) out_row[i] = (i < n_sel) ? stage[i] : -1;
+    if (stage1) {                                        // candidates: (value, column of the whole row), ascending column
+      const long long at = (long long)blockIdx.x * p.k;
+      for (unsigned i = tid; i < k; i += THREADS) {
+        const bool have = i < n_sel;
+        const int c = have ? stage[i] : 0;
+        p.cand_idx[at + i] = have ? base + c : -1;
+        p.cand_val[at + i] = have ? ScoreLoad<ScoreT>::one(src + c) + 0.0f : kNaN;
+      }
+      return;
+    }
+    const int* map = MODE == 2 ? p.index_map + (long long)row * p.width : nullptr;
+    for (unsigned i = tid; i < k; i += THREADS) out_row[i] = (i < n_sel) ? (MODE == 2 ? map[stage[i]] : stage[i]) : -1;
     return;
   }
+  const int* map = MODE == 2 ? p.index_map + (long long)row * p.width : nullptr;
   const unsigned P = (unsigned)p.sort_len;
   for (unsigned i = n_sel + tid; i < P; i += THREADS) pairs[i] = 0ull;   // sorts last
   __syncthreads();
@@ -411,8 +436,10 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
       __syncthreads();
     }
   }
-  for (unsigned i = tid; i < k; i += THREADS)
-    out_row[i] = (i < n_sel) ? (int)(0xffffffffu - (unsigned)(pairs[i] & 0xffffffffull)) : -1;
+  for (unsigned i = tid; i < k; i += THREADS) {
+    const int pos = (int)(0xffffffffu - (unsigned)(pairs[i] & 0xffffffffull));
+    out_row[i] = (i < n_sel) ? (MODE == 2 ? map[pos] : pos) : -1;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -618,15 +645,15 @@ int launch_kernel(K kernel, const TopkParams& p, int threads, size_t smem, hipSt
   if (smem > 64 * 1024 &&
       hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
     return -2;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)p.rows), dim3((unsigned)threads), smem, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(p.rows * (p.segs > 1 ? p.segs : 1))), dim3((unsigned)threads), smem, stream, p);
   return 0;
 }
 
 static int wide_threads() { return 512; }
 
-template <typename ScoreT>
+template <typename ScoreT, int MODE = 0>
 int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* smem_out) {
-  const int T = p.width;
+  const int T = p.segs > 1 ? p.seg_width : p.width;      // columns one workgroup looks at
   const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
   const size_t out_words = sorted ? (size_t)p.sort_len * 2 : (size_t)p.k;
   if (T <= 32768) {
@@ -640,9 +667,12 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
     const size_t smem = tile_smem(E, THR);                                                \
     *smem_out = smem;                                                                     \
     if (smem > 160 * 1024) return -3;                                                     \
-    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4, THR>, p, THR, smem, stream) \
-                : launch_kernel(topk_tile_kernel<ScoreT, E, 1, THR>, p, THR, smem, stream); \
+    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4, THR, MODE>, p, THR, smem, stream) \
+                : launch_kernel(topk_tile_kernel<ScoreT, E, 1, THR, MODE>, p, THR, smem, stream); \
   } while (0)
+    if constexpr (MODE == 1) {                            // a segment is always kSegWidth columns wide
+      CM_TOPK_TILE(16, 512);
+    }
     if (T <= 1024) CM_TOPK_TILE(4, kTileThreads);
     if (T <= 2048) CM_TOPK_TILE(8, kTileThreads);
     if (T <= 4096) CM_TOPK_TILE(16, kTileThreads);
@@ -672,6 +702,27 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
 
 }  // namespace
 
+// Rows wider than 16384 columns are cut into segments of 8192 (the fastest single-workgroup
+// shape) when the caller supplies a workspace; k must fit a segment and segs * k one stage-2 row.
+constexpr int kSegWidth = 8192;
+static int topk_segments(const cppmega_mi355_topk_args_t& a) {
+  if (a.width <= 16384 || a.k > kSegWidth || a.width % 4 != 0 || a.row_stride % 4 != 0) return 1;
+  const int segs = (a.width + kSegWidth - 1) / kSegWidth;
+  if ((long long)segs * a.k > 32768 || ((long long)segs * a.k) % 4 != 0) return 1;
+  return segs;
+}
+static size_t topk_workspace_for(const cppmega_mi355_topk_args_t& a, int segs) {
+  const size_t cands = (size_t)a.rows * segs * a.k;
+  return ((cands * 4 + 255) & ~(size_t)255) + cands * 4;
+}
+
+int topk_workspace_bytes(const cppmega_mi355_topk_args_t& a, size_t* bytes) {
+  if (a.rows < 0 || a.width < 1 || a.k < 1 || a.k > a.width) return fail(CPPMEGA_MI355_ERR_SHAPE, "topk: rows=%d width=%d k=%d", a.rows, a.width, a.k);
+  const int segs = topk_segments(a);
+  *bytes = segs > 1 ? topk_workspace_for(a, segs) : 0;
+  return 0;
+}
+
 int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream) {
   if (!a.scores || !a.indices) return fail(CPPMEGA_MI355_ERR_NULL, "topk: scores/indices is NULL");
   if (a.rows < 0 || a.width < 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "topk: rows=%d width=%d", a.rows, a.width);
@@ -695,10 +746,34 @@ int topk_select_launch(const cppmega_mi355_topk_args_t& a, hipStream_t stream) {
   int sort_len = 2;
   while (sort_len < a.k) sort_len <<= 1;
   p.sort_len = sort_len;
+  p.segs = 1; p.seg_width = 0; p.cand_val = nullptr; p.cand_idx = nullptr; p.index_map = nullptr;
 
   int rc;
   size_t smem = 0;
-  if (a.score_dtype == CPPMEGA_MI355_F32) rc = launch_for_type<float>(p, vec4, stream, &smem);
+  const int segs = topk_segments(a);
+  if (segs > 1 && a.workspace) {
+    const size_t need = topk_workspace_for(a, segs);
+    if (a.workspace_bytes < need)
+      return fail(CPPMEGA_MI355_ERR_WORKSPACE, "topk: workspace of %zu bytes needed, %zu given", need, (size_t)a.workspace_bytes);
+    if ((uintptr_t)a.workspace & 15) return fail(CPPMEGA_MI355_ERR_ALIGNMENT, "topk: workspace must be 16-byte aligned");
+    const size_t cands = (size_t)a.rows * segs * a.k;
+    // stage 1: every (row, segment) keeps its k best, ascending column (so a candidate's position
+    // orders like its column and stage 2 breaks ties toward the lower column)
+    TopkParams s1 = p;
+    s1.segs = segs; s1.seg_width = kSegWidth; s1.order = CPPMEGA_MI355_TOPK_ORDER_INDEX;
+    s1.cand_val = (float*)a.workspace;
+    s1.cand_idx = (int*)((char*)a.workspace + ((cands * 4 + 255) & ~(size_t)255));
+    if (a.score_dtype == CPPMEGA_MI355_F32) rc = launch_for_type<float, 1>(s1, vec4, stream, &smem);
+    else if (a.score_dtype == CPPMEGA_MI355_F16) rc = launch_for_type<Half, 1>(s1, vec4, stream, &smem);
+    else rc = launch_for_type<BHalf, 1>(s1, vec4, stream, &smem);
+    if (rc == 0) {
+      // stage 2: the bounds and the -inf rule have been applied; what is left is a plain selection
+      TopkParams s2 = p;
+      s2.scores = s1.cand_val; s2.row_stride = (long long)segs * a.k; s2.width = segs * a.k;
+      s2.starts = nullptr; s2.ends = nullptr; s2.neg_inf_masked = 0; s2.index_map = s1.cand_idx;
+      rc = launch_for_type<float, 2>(s2, true, stream, &smem);
+    }
+  } else if (a.score_dtype == CPPMEGA_MI355_F32) rc = launch_for_type<float>(p, vec4, stream, &smem);
   else if (a.score_dtype == CPPMEGA_MI355_F16) rc = launch_for_type<Half>(p, vec4, stream, &smem);
   else rc = launch_for_type<BHalf>(p, vec4, stream, &smem);
   if (rc == -3)

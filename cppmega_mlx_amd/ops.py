@@ -59,8 +59,11 @@ def topk_select(
     ends: torch.Tensor | None = None,
     order: str = "index",
     neg_inf_is_masked: bool = False,
+    workspace: torch.Tensor | None = None,
+    two_stage: bool = True,
 ) -> torch.Tensor:
-    """Write the per-row top-k indices of ``scores`` (rows, width) into ``out`` (rows, k)."""
+    """Write the per-row top-k indices of ``scores`` (rows, width) into ``out`` (rows, k).  Rows wider
+    than 16384 columns go through a workspace in two stages unless ``two_stage`` is off."""
     _lib.require_device_tensor(scores, "scores")
     _lib.require_device_tensor(out, "out", scores)
     if scores.ndim != 2:
@@ -90,8 +93,18 @@ def topk_select(
     args.indices = out.data_ptr()
     args.neg_inf_is_masked = 1 if neg_inf_is_masked else 0
     lib = _lib.load()
+    stream = _lib.current_stream(scores.device)
+    need = C.c_size_t(0)
+    _lib.check(lib.cppmega_mi355_topk_workspace_bytes(C.byref(args), C.sizeof(args), C.byref(need)), "topk_select")
+    if need.value and two_stage:
+        if workspace is None:
+            workspace = _workspace(scores.device, need.value, stream)
+        else:
+            _lib.require_device_tensor(workspace, "workspace", scores)
+        args.workspace = workspace.data_ptr()
+        args.workspace_bytes = workspace.numel() * workspace.element_size()
     with torch.cuda.device(scores.device):
-        rc = lib.cppmega_mi355_topk_select(C.byref(args), C.sizeof(args), _lib.current_stream(scores.device))
+        rc = lib.cppmega_mi355_topk_select(C.byref(args), C.sizeof(args), stream)
     _lib.check(rc, "topk_select")
     return out
 

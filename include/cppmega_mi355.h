@@ -110,9 +110,24 @@ typedef struct cppmega_mi355_topk_args {
   int32_t* indices;           /* out [rows, k], dense                          */
   int32_t neg_inf_is_masked;  /* non-zero: an in-range -inf is unselectable    */
   int32_t reserved;
+
+  /* Appended after the first ABI (a caller whose struct_size ends at `reserved`
+   * gets NULL / 0). */
+  void* workspace;            /* optional, uninitialised: with *_workspace_bytes of it,
+                               * rows wider than 16384 columns are selected in two
+                               * stages (k best of every 8192-column segment, then k of
+                               * those), one workgroup per segment instead of one per
+                               * row; same result                               */
+  size_t workspace_bytes;
 } cppmega_mi355_topk_args_t;
 
+#define CPPMEGA_MI355_TOPK_ARGS_V1_SIZE (offsetof(cppmega_mi355_topk_args_t, workspace))
+
 int cppmega_mi355_topk_select(const cppmega_mi355_topk_args_t* args, size_t args_size, void* stream);
+
+/* Bytes of workspace that let cppmega_mi355_topk_select take the two-stage path for this
+ * shape (0 when it has none: narrow rows, k above 8192 or 32768 / segments). */
+int cppmega_mi355_topk_workspace_bytes(const cppmega_mi355_topk_args_t* args, size_t args_size, size_t* bytes);
 
 /* ---- indexer scores -> top-k -------------------------------------------------
  * The score and selection tail of the reference's LightningIndexer.__call__

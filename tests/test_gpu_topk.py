@@ -121,3 +121,37 @@ def test_public_entry_points(device):
     for backend in ("auto", "hip", "path_c", "mlx"):
         np.testing.assert_array_equal(tk.topk_selector(t, 16, backend=backend).cpu().numpy(), otopk.topk_selector_oracle(s, 16))
     assert tk.topk_selector_path_c_status().available
+
+
+@pytest.mark.parametrize("rows,width,k", [(32, 65536, 2048), (3, 40000, 4000), (2, 24576, 8192), (5, 16388, 100)])
+def test_wide_rows_two_stage_and_single_workgroup_paths_agree_with_the_oracle(device, rows, width, k):
+    """Rows wider than 16384 columns: k best of every 8192-column segment, then k of those.  Ties that
+    straddle segments, bounds that empty whole segments, -inf and NaN entries."""
+    import ctypes as C
+    from cppmega_mlx_amd import _lib, ops
+    rng = np.random.default_rng(rows + width + k)
+    s = topk_scores(rng, rows, width, tie_fraction=0.2)
+    s[0, ::5] = 1.5                                      # one value far beyond k times, in every segment
+    s[1, 100:9000] = np.nan
+    s[1, 9000:9500] = -np.inf
+    starts = rng.integers(0, width // 3, rows).astype(np.int32)
+    ends = rng.integers(width // 2, width + 1, rows).astype(np.int32)
+    starts[-1], ends[-1] = 9000, 9000 + k // 2           # fewer selectable columns than k, inside one segment
+    t = to_dev(s, device)
+    for order in ("index", "value"):
+        for bounds in (False, True):
+            st = to_dev(starts, device) if bounds else None
+            en = to_dev(ends, device) if bounds else None
+            want = otopk.topk_selector_oracle(s, k, starts=starts if bounds else None, ends=ends if bounds else None,
+                                              order=order, neg_inf_is_masked=True)
+            for two_stage in (True, False):
+                out = torch.full((rows, k), -7, dtype=torch.int32, device=device)
+                ops.topk_select(t, k, out=out, starts=st, ends=en, order=order, neg_inf_is_masked=True, two_stage=two_stage)
+                torch.cuda.synchronize()
+                np.testing.assert_array_equal(out.cpu().numpy(), want)
+    a = _lib.TopkArgs()
+    a.struct_size = C.sizeof(a)
+    a.rows, a.width, a.row_stride, a.k = rows, width, width, k
+    need = C.c_size_t(0)
+    assert _lib.load().cppmega_mi355_topk_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == _lib.OK
+    assert (need.value > 0) == (width % 4 == 0 and width > 16384)
