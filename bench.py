@@ -471,14 +471,137 @@ def measured_traffic(name):
         return None
 
 
+# --------------------------------------------------------------------------- rocprofv3 summaries
+# The three profiler runs whose CSV output `--summarise-profiles DIR` turns into profiles/*.md and
+# profiles/traffic.json.  Each is run from /tmp (`cd /tmp && export TMPDIR=/tmp`) with DIR as below.
+PROFILE_RUNS = {
+    "prof_all": "rocprofv3 --kernel-trace --stats --output-format csv -d DIR/prof_all -o all -- python3 bench.py "
+                "--only decode,vecmat,topk,copy,next --steps 20 --no-cpu-baseline",
+    "pmc_fetch": "rocprofv3 --pmc FETCH_SIZE --output-format csv -d DIR/pmc_fetch -o f -- python3 bench.py "
+                 "--only decode,vecmat,topk,copy,next --steps 3 --warmup 1 --no-cpu-baseline",
+    "pmc_write": "rocprofv3 --pmc WRITE_SIZE --output-format csv -d DIR/pmc_write -o w -- python3 bench.py "
+                 "--only decode,vecmat,topk,copy,next --steps 3 --warmup 1 --no-cpu-baseline",
+    "pmc_sq": "rocprofv3 --pmc SQ_WAVE_CYCLES SQ_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES "
+              "SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY SQ_ACTIVE_INST_LDS --output-format csv -d DIR/pmc_sq -o s -- python3 bench.py "
+              "--only decode --steps 3 --warmup 1 --no-cpu-baseline",
+}
+# summary file -> (kernel-name fragments, workload text)
+PROFILE_WORKLOADS = [
+    ("sparse_mla_decode", ("sparse_mla_latent",),
+     "decode B=32 S_q=1 H=128 topk=2048 Skv=65536 (e4m3 latent + fp32/128 scales + bf16 rope); the run times the "
+     "power-of-two-scale cache and the general-scale cache, so each row averages both"),
+    ("fp8_vecmat", ("gemv_stream_kernel<1, 4, 4, 0>",), "W e4m3[7168,16384] + fp32 scale/128, x bf16[1,16384]"),
+    ("fp8_vecmat_e4m3_activation", ("gemv_stream_kernel<1, 4, 4, 1>",),
+     "W e4m3[7168,16384] + fp32 scale per row, x e4m3[16384] + fp32 scale -> f32[7168] (the reference's own vecmat form)"),
+    ("fp8_vecmat_m4", ("gemv_stream_kernel<4",), "W e4m3[7168,16384] + fp32 scale/128, x bf16[4,16384]"),
+    ("fp8_vecmat_m16", ("skinny_mfma_kernel<1>", "skinny_reduce"),
+     "W e4m3[7168,16384] + fp32 scale/128, x bf16[16,16384] (the reduce kernel row averages the M = 16 and M = 32 calls of the run)"),
+    ("fp8_vecmat_m32", ("skinny_mfma_kernel<2>", "skinny_reduce"),
+     "W e4m3[7168,16384] + fp32 scale/128, x bf16[32,16384] (the reduce kernel row averages the M = 16 and M = 32 calls of the run)"),
+    ("topk_selector", ("topk_tile_kernel<float, 16, 4, 512, 0>",), "scores fp32[4096 rows,8192] -> int32[4096,2048]"),
+    ("topk_selector_decode_shape", ("topk_tile_kernel<float, 16, 4, 512, 1>", "topk_tile_kernel<float, 16, 4, 1024, 2>", "topk_wide_kernel"),
+     "scores fp32[32,65536] -> int32[32,2048]: the two-stage path (segment kernel, then candidate kernel) and, for "
+     "comparison, the one-workgroup-per-row kernel; the indexer's decode row runs the two-stage kernels as well"),
+    ("indexer_scores_topk", ("indexer_",),
+     "indexer_topk q bf16[B,Sq,64,128], k bf16[B,Skv,128]: prefill (1, 8192, 8192) and decode (32, 1, 65536) dispatches"),
+    ("mla_absorb_head_gemm", ("head_gemm_kernel",),
+     "head_gemm x bf16[32,128,128] . W bf16[128,512,128] and x bf16[32,128,512] . W bf16[128,128,512]"),
+    ("kv_cache_append", ("cache_append_kernel",),
+     "bf16 latent[B,S,1,512] + rope[..,64] -> e4m3 + fp32/128 scales + bf16 rope in the cache: one dispatch of 8192 rows "
+     "(prefill chunk) and one of 32 rows (decode step) per step"),
+    ("sparse_index_producers", ("_indices_",),
+     "causal_sparse_indices(1,8192,1,2048) and sparse_indices_from_attention_mask(bool [8192,8192], topk 2048)"),
+]
+
+
+def summarise_profiles(src: str) -> int:
+    """Write profiles/*.md and profiles/traffic.json from the CSV output of PROFILE_RUNS under `src`."""
+    import collections
+    import csv
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    out_dir = os.path.join(here, "profiles")
+    os.makedirs(out_dir, exist_ok=True)
+
+    def rows(rel):
+        with open(os.path.join(src, rel)) as fh:
+            return list(csv.DictReader(fh))
+
+    stats = {r["Name"]: r for r in rows("prof_all/all_kernel_stats.csv")}
+
+    def counters(rel):
+        agg = collections.defaultdict(list)
+        for r in rows(rel):
+            agg[r["Kernel_Name"]].append(float(r["Counter_Value"]))
+        return agg
+
+    fetch, write = counters("pmc_fetch/f_counter_collection.csv"), counters("pmc_write/w_counter_collection.csv")
+    copy_kib = 262144.0                                    # the 256 MiB device copy of bench_copy, each way
+    copy_f, copy_w = max(fetch["__amd_rocclr_copyBuffer"]), max(write["__amd_rocclr_copyBuffer"])
+    scale_f, scale_w = copy_kib / copy_f, copy_kib / copy_w
+
+    def cmd(key):
+        return "`cd /tmp && export TMPDIR=/tmp && " + PROFILE_RUNS[key].replace("DIR", "$GRAFT_REPO_ROOT/gpurun_out").replace(
+            "bench.py", "$GRAFT_REPO_ROOT/bench.py") + "`"
+
+    def short(name):
+        return name.replace("(anonymous namespace)::", "")
+
+    traffic = {}
+    for fname, frags, workload in PROFILE_WORKLOADS:
+        names = [n for n in stats if "cm::" in n and any(f in n for f in frags)]
+        text = [f"# rocprofv3 summary: {fname}", "", f"Workload: {workload} (one MI355X, synthetic inputs resident in HBM).", "",
+                "## Kernel durations (`--kernel-trace --stats`)", "", "Command: " + cmd("prof_all"), "",
+                "| kernel | calls | avg us | min us | max us |", "|---|---|---|---|---|"]
+        for n in names:
+            r = stats[n]
+            text.append("| `%s` | %s | %.2f | %.2f | %.2f |" % (short(n), r["Calls"], float(r["AverageNs"]) / 1e3,
+                                                              float(r["MinNs"]) / 1e3, float(r["MaxNs"]) / 1e3))
+        text += ["", "## HBM traffic per dispatch (`--pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, KiB)", "",
+                 "Commands: " + cmd("pmc_fetch") + " and " + cmd("pmc_write") + ".", "",
+                 "Scale factors from the 256 MiB device copy in the same runs (`__amd_rocclr_copyBuffer`, 262144 KiB each way): "
+                 "FETCH_SIZE read %.1f KiB -> x%.3f, WRITE_SIZE read %.1f KiB -> x%.3f." % (copy_f, scale_f, copy_w, scale_w), "",
+                 "| kernel | FETCH_SIZE KiB | WRITE_SIZE KiB | scaled read MiB | scaled write MiB |", "|---|---|---|---|---|"]
+        total = 0.0
+        for n in names:
+            f = sum(fetch[n]) / len(fetch[n]) if fetch.get(n) else 0.0
+            w = sum(write[n]) / len(write[n]) if write.get(n) else 0.0
+            text.append("| `%s` | %.1f | %.1f | %.1f | %.1f |" % (short(n), f, w, f * scale_f / 1024, w * scale_w / 1024))
+            total += (f * scale_f + w * scale_w) * 1024
+        traffic[fname] = {"hbm_bytes_per_launch": int(total), "kernels": names}
+        if fname == "sparse_mla_decode" and os.path.exists(os.path.join(src, "pmc_sq/s_counter_collection.csv")):
+            sq = collections.defaultdict(list)
+            for r in rows("pmc_sq/s_counter_collection.csv"):
+                if "sparse_mla_latent_kernel" in r["Kernel_Name"]:
+                    sq[r["Counter_Name"]].append(float(r["Counter_Value"]))
+            text += ["", "## SQ counters of the main kernel (one `--pmc` pass, average per dispatch, summed over its wavefronts)", "",
+                     "Command: " + cmd("pmc_sq"), "", "| counter | value |", "|---|---|"]
+            avg = {k: sum(v) / len(v) for k, v in sq.items()}
+            for k in sorted(avg):
+                text.append("| %s | %.0f |" % (k, avg[k]))
+            if avg.get("SQ_WAVE_CYCLES"):
+                text += ["", "SQ_VALU_MFMA_BUSY_CYCLES / (4 x SQ_WAVE_CYCLES) = %.3f: the matrix-core busy fraction of the wavefronts' "
+                         "lifetime (wave cycles count in units of 4 clocks)." % (avg.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) / (4 * avg["SQ_WAVE_CYCLES"]))]
+        with open(os.path.join(out_dir, fname + ".md"), "w") as fh:
+            fh.write("\n".join(text) + "\n")
+    with open(os.path.join(out_dir, "traffic.json"), "w") as fh:
+        json.dump({"fetch_scale": scale_f, "write_scale": scale_w, "workloads": traffic}, fh, indent=1)
+    print(f"wrote {len(PROFILE_WORKLOADS)} summaries and traffic.json to {out_dir}")
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--summarise-profiles", metavar="DIR", default=None,
+                    help="no GPU work: turn the rocprofv3 CSVs under DIR (see PROFILE_RUNS) into profiles/*.md and profiles/traffic.json")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", type=str, default="decode,vecmat,topk,next")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
+    if args.summarise_profiles:
+        return summarise_profiles(args.summarise_profiles)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; the path shards without communication "
               "(rows / sequences / queries per GPU), so --gpus N>1 is not run here.", file=sys.stderr)
