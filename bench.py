@@ -458,6 +458,21 @@ def bench_next_rows(args, device):
         y = torch.empty((B, H, N), dtype=torch.bfloat16, device=device)
         hbm(tag, lambda x=x, w=w, y=y: ops.head_gemm(x, w, out=y), (x.numel() + w.numel() + y.numel()) * 2,
             f"head_gemm x bf16[{B},{H},{K}] . W bf16[{H},{N},{K}] -> bf16[{B},{H},{N}]")
+    # training side: float-carrier sparse-MLA backward (fp32 arithmetic; bound by the fp32 vector rate)
+    B, S, H, D, d_v, Skv, topk = 1, 1024, 16, 576, 512, 4096, 256
+    q = torch.randn((B, S, H, D), generator=gen, device=device).to(torch.bfloat16)
+    kv = torch.randn((B, Skv, 1, D), generator=gen, device=device).to(torch.bfloat16)
+    d_out = torch.randn((B, S, H, d_v), generator=gen, device=device).to(torch.bfloat16)
+    idx = torch.stack([torch.randperm(Skv, generator=gen, device=device)[:topk] for _ in range(S)]).to(torch.int32).view(B, S, 1, topk)
+    dq = torch.empty_like(q)
+    dkv = torch.empty((B, Skv, 1, D), dtype=torch.float32, device=device)
+    secs, _ = timed_graph([lambda: ops.sparse_mla_backward(q, kv, d_out, idx, sm_scale=D ** -0.5, d_v=d_v, dq=dq, dkv=dkv)], steps, args.warmup)
+    flops = 2.0 * B * S * H * topk * (3 * D + 2 * d_v)
+    res["sparse_mla_backward"] = {
+        "workload": f"sparse_mla_bwd q bf16[{B},{S},{H},{D}] kv bf16[{B},{Skv},1,{D}] topk {topk} -> dq bf16, dkv f32 (atomic adds)",
+        "us_per_launch": secs / steps * 1e6, "algorithmic_flops": flops,
+        "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 157.3, "unit": "TFLOP/s",
+                     "frac": flops / (secs / steps) / 1e12 / 157.3, "traffic": None}}
     return res
 
 

@@ -50,6 +50,7 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_fp8_vecmat",
     "cppmega_mi355_fp8_quantize",
     "cppmega_mi355_head_gemm",
+    "cppmega_mi355_sparse_mla_bwd",
     "cppmega_mi355_dequant_block_fp8",
     "cppmega_mi355_kv_cache_append",
     "cppmega_mi355_causal_sparse_indices",
@@ -129,6 +130,36 @@ class IndexerArgs(C.Structure):
         ("scores_out", C.c_void_p),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class SparseMlaBwdArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("q_dtype", C.c_int32),
+        ("q", C.c_void_p),
+        ("kv", C.c_void_p),
+        ("d_out", C.c_void_p),
+        ("indices", C.c_void_p),
+        ("kv_dtype", C.c_int32),
+        ("d_out_dtype", C.c_int32),
+        ("dq_dtype", C.c_int32),
+        ("index_dtype", C.c_int32),
+        ("batch", C.c_int32),
+        ("seq_q", C.c_int32),
+        ("heads", C.c_int32),
+        ("kv_groups", C.c_int32),
+        ("seq_kv", C.c_int32),
+        ("topk", C.c_int32),
+        ("d_qk", C.c_int32),
+        ("d_v", C.c_int32),
+        ("sm_scale", C.c_float),
+        ("clear_dkv", C.c_int32),
+        ("sm_scale_dev", C.c_void_p),
+        ("dq", C.c_void_p),
+        ("dkv", C.c_void_p),
+        ("q_scale", C.c_void_p),
+        ("kv_scale", C.c_void_p),
     ]
 
 
@@ -361,6 +392,8 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_fp8_vecmat.restype = C.c_int
         lib.cppmega_mi355_fp8_quantize.argtypes = [C.POINTER(QuantizeArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_fp8_quantize.restype = C.c_int
+        lib.cppmega_mi355_sparse_mla_bwd.argtypes = [C.POINTER(SparseMlaBwdArgs), C.c_size_t, C.c_void_p]
+        lib.cppmega_mi355_sparse_mla_bwd.restype = C.c_int
         lib.cppmega_mi355_head_gemm.argtypes = [C.POINTER(HeadGemmArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_head_gemm.restype = C.c_int
         lib.cppmega_mi355_dequant_block_fp8.argtypes = [C.POINTER(DequantBlockArgs), C.c_size_t, C.c_void_p]

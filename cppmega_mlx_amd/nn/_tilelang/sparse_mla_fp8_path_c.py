@@ -8,6 +8,9 @@ score = (sum dec*dec) * qs * ks * sm_scale, optional attention ``sinks`` ``[H]``
 (one extra logit per head in the max and the denominator, no value row),
 ``out`` float32/float16/bfloat16 (``output_dtype``), ``lse`` float32.
 
+``sparse_mla_fp8_bwd_path_c`` :3007-3080 is the backward over the same prepared
+buffers (kernel :1966-2214): float32 gradients with respect to the dequantised q and kv.
+
 A float32 ``kv_scale`` of rank 4 selects the block-128 latent layout described
 in ``sparse_mla_blockscaled_path_c`` (per-token is its one-block case), so the
 sink path is available for the latent KV cache as well.
@@ -28,6 +31,7 @@ __all__ = [
     "sparse_mla_fp8_path_c_apply",
     "sparse_mla_fp8_path_c_apply_direct",
     "sparse_mla_fp8_path_c_status",
+    "sparse_mla_fp8_bwd_path_c",
     "fp8_sparse_mla_indexed_qk_reduce_path_c",
     "fp8_sparse_mla_qk_reduce_path_c",
 ]
@@ -158,6 +162,51 @@ def sparse_mla_fp8_path_c_apply(
             f"sparse_mla_fp8_path_c_apply: kernel dispatch failed: {type(exc).__name__}: {exc}"
         ) from exc
     return (out, lse) if return_lse else out
+
+
+def sparse_mla_fp8_bwd_path_c(
+    q_fp8: torch.Tensor,
+    q_scale: torch.Tensor,
+    kv_fp8: torch.Tensor,
+    kv_scale: torch.Tensor,
+    d_out: torch.Tensor,
+    indices: torch.Tensor,
+    *,
+    sm_scale: float,
+    d_v: int | None = None,
+    force_path_c: bool = False,
+    causal: bool = False,
+    dq_buffer: torch.Tensor | None = None,
+    dkv_buffer: torch.Tensor | None = None,
+):
+    """Backward over prepared per-token FP8 buffers: ``(dq_dequant [B,S,H,K], dkv_dequant
+    [B,Skv,G,K])`` float32, written into ``dq_buffer`` / ``dkv_buffer`` when given."""
+    status = sparse_mla_fp8_path_c_status()
+    if not status.available:
+        if force_path_c:
+            raise RuntimeError(f"sparse_mla_fp8_bwd_path_c: {status.reason}")
+        return None
+    del causal  # the sparse indices define the scatter pattern; kept for call compatibility
+    plan = _prepared.plan_prepared(q_fp8, q_scale, kv_fp8, kv_scale, indices, d_v=d_v, kv_rope=None, op_name=_OP, family="fp8")
+    if plan.layout != "per_token":
+        raise ValueError("sparse_mla_fp8_bwd_path_c takes per-token float32 scales (q_scale [B,S,H], kv_scale [B,Skv,G])")
+    want = (plan.batch, plan.seq_len, plan.heads, plan.d_v)
+    if tuple(d_out.shape) != want:
+        raise ValueError(f"d_out must have shape {want}; got {tuple(d_out.shape)}")
+    _float_dtype(d_out.dtype, name="d_out dtype")
+    dq_shape = (plan.batch, plan.seq_len, plan.heads, plan.qk_dim)
+    dkv_shape = (plan.batch, plan.seq_len_kv, plan.kv_group, plan.qk_dim)
+    for name, buf, shape in (("dq_buffer", dq_buffer, dq_shape), ("dkv_buffer", dkv_buffer, dkv_shape)):
+        if buf is not None and (tuple(buf.shape) != shape or buf.dtype != torch.float32):
+            raise ValueError(f"{name} must be float32 with shape {shape}; got {buf.dtype} {tuple(buf.shape)}")
+    dq = dq_buffer if dq_buffer is not None else torch.empty(dq_shape, dtype=torch.float32, device=q_fp8.device)
+    dkv = dkv_buffer if dkv_buffer is not None else torch.empty(dkv_shape, dtype=torch.float32, device=q_fp8.device)
+    try:
+        ops.sparse_mla_backward(q_fp8, kv_fp8, d_out.contiguous(), indices, sm_scale=float(sm_scale), d_v=plan.d_v, dq=dq, dkv=dkv,
+                                clear_dkv=True, q_scale=q_scale, kv_scale=kv_scale)
+    except (_lib.NativeCallError, _lib.NativeLibraryError) as exc:
+        raise SparseMLAFp8PathCDirectError(f"FP8 sparse-MLA backward dispatch failed: {type(exc).__name__}: {exc}") from exc
+    return dq, dkv
 
 
 # invalid slots of the score-only kernels hold this finite sentinel

@@ -398,6 +398,54 @@ def sparse_mla_forward(
     return out, lse
 
 
+def sparse_mla_backward(q: torch.Tensor, kv: torch.Tensor, d_out: torch.Tensor, indices: torch.Tensor, *,
+                        sm_scale: float | torch.Tensor, d_v: int, dq: torch.Tensor, dkv: torch.Tensor,
+                        clear_dkv: bool = True, q_scale: torch.Tensor | None = None,
+                        kv_scale: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Gradients of the sparse MLA forward into caller-owned ``dq`` [B,S,H,D] (any float carrier) and
+    ``dkv`` [B,Skv,G,D] (float32, accumulated with atomic adds; cleared first unless ``clear_dkv``
+    is off).  q / kv are float carriers, or uint8 e4m3 bytes with per-token float32 scales."""
+    for name, t in (("q", q), ("kv", kv), ("d_out", d_out), ("indices", indices), ("dq", dq), ("dkv", dkv),
+                    ("q_scale", q_scale), ("kv_scale", kv_scale)):
+        if t is not None:
+            _lib.require_device_tensor(t, name, q if name != "q" else None)
+    if q.ndim != 4 or kv.ndim != 4 or indices.ndim != 4:
+        raise ValueError("sparse_mla: q, kv and indices must be rank 4")
+    B, S, H, D = q.shape
+    _, Skv, G, _ = kv.shape
+    if tuple(d_out.shape) != (B, S, H, int(d_v)):
+        raise ValueError(f"d_out must have shape {(B, S, H, int(d_v))}; got {tuple(d_out.shape)}")
+    if tuple(dq.shape) != (B, S, H, D):
+        raise ValueError(f"dq must have shape {(B, S, H, D)}; got {tuple(dq.shape)}")
+    if tuple(dkv.shape) != tuple(kv.shape) or dkv.dtype != torch.float32:
+        raise ValueError(f"dkv must be float32 with shape {tuple(kv.shape)}; got {dkv.dtype} {tuple(dkv.shape)}")
+    a = _lib.SparseMlaBwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.q_dtype = _dtype_or_raise(q, "q", (_lib.F32, _lib.F16, _lib.BF16, _lib.E4M3))
+    a.kv_dtype = _dtype_or_raise(kv, "kv", (_lib.F32, _lib.F16, _lib.BF16, _lib.E4M3))
+    a.d_out_dtype = _dtype_or_raise(d_out, "d_out", (_lib.F32, _lib.F16, _lib.BF16))
+    a.dq_dtype = _dtype_or_raise(dq, "dq", (_lib.F32, _lib.F16, _lib.BF16))
+    for name, t, scale, want in (("q", q, q_scale, (B, S, H)), ("kv", kv, kv_scale, (B, Skv, G))):
+        if t.dtype == torch.uint8 and (scale is None or tuple(scale.shape) != want or scale.dtype != torch.float32):
+            raise ValueError(f"{name}_scale must be float32 with shape {want} for e4m3 {name}")
+    a.q_scale, a.kv_scale = _lib.ptr(q_scale), _lib.ptr(kv_scale)
+    a.index_dtype = _dtype_or_raise(indices, "indices", (_lib.I32, _lib.I64))
+    a.q, a.kv, a.d_out, a.indices, a.dq, a.dkv = (t.data_ptr() for t in (q, kv, d_out, indices, dq, dkv))
+    a.batch, a.seq_q, a.heads, a.kv_groups, a.seq_kv, a.topk, a.d_qk, a.d_v = B, S, H, G, Skv, indices.shape[-1], D, int(d_v)
+    if isinstance(sm_scale, torch.Tensor):
+        _lib.require_device_tensor(sm_scale, "sm_scale", q)
+        if sm_scale.dtype != torch.float32 or sm_scale.numel() != 1:
+            raise ValueError(f"a device sm_scale must be one float32; got {sm_scale.dtype} {tuple(sm_scale.shape)}")
+        a.sm_scale_dev = sm_scale.data_ptr()
+    else:
+        a.sm_scale = float(sm_scale)
+    a.clear_dkv = 1 if clear_dkv else 0
+    with torch.cuda.device(q.device):
+        rc = _lib.load().cppmega_mi355_sparse_mla_bwd(C.byref(a), C.sizeof(a), _lib.current_stream(q.device))
+    _lib.check(rc, "sparse_mla_bwd")
+    return dq, dkv
+
+
 def sparse_mla_scores(
     q: torch.Tensor,
     kv: torch.Tensor,

@@ -304,6 +304,41 @@ int cppmega_mi355_sparse_mla_select_kernel(const cppmega_mi355_sparse_mla_args_t
 int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args, size_t args_size,
                                     float* scores, void* stream);
 
+/* ---- sparse MLA backward ---------------------------------------------------------
+ * Replaces sparse_mla_bwd_direct, called as kernel(d_out, indices, kv, q, sm_scale_buf,
+ * out=(dkv, dq)) (cppmega_mlx/nn/_tilelang/sparse_mla_path_c.py:2644-2816, 3314-3421),
+ * its per-token FP8 form fp8_sparse_mla_bwd_kernel(q_fp8, q_scale, kv_fp8, kv_scale,
+ * d_out, indices, sm_scale_buf, dq_dequant, dkv_dequant)
+ * (sparse_mla_fp8_path_c.py:1966-2214, 3007-3080), and the dkv clearing kernels in
+ * front of them (sparse_mla_path_c.py:3163-3230, sparse_mla_fp8_path_c.py:2217-2272):
+ *   dq  [B, S, H, d_qk]      gradient of q, float32 / float16 / bfloat16
+ *   dkv [B, Skv, G, d_qk]    gradient of the KV rows, float32, accumulated with atomic
+ *                            adds; cleared first when clear_dkv is non-zero
+ * for out = softmax(sm_scale * q . K_sel^T) . K_sel[:, :d_v] and the cotangent d_out
+ * [B, S, H, d_v].  q, kv: float32 / float16 / bfloat16, or e4m3 bytes with per-token
+ * float32 scales q_scale [B,S,H] / kv_scale [B,Skv,G] (gradients are then with respect
+ * to the dequantised values); d_out a float carrier; everything dense; an index < 0 or
+ * >= Skv is skipped; a row with nothing to attend to contributes zero gradients. */
+typedef struct cppmega_mi355_sparse_mla_bwd_args {
+  uint32_t struct_size;
+  int32_t q_dtype;
+  const void* q;
+  const void* kv;
+  const void* d_out;
+  const void* indices;
+  int32_t kv_dtype, d_out_dtype, dq_dtype, index_dtype;
+  int32_t batch, seq_q, heads, kv_groups, seq_kv, topk, d_qk, d_v;
+  float sm_scale;
+  int32_t clear_dkv;
+  const float* sm_scale_dev;  /* device float32[1] read in place of sm_scale, or NULL */
+  void* dq;
+  float* dkv;
+  const float* q_scale;       /* e4m3 q only */
+  const float* kv_scale;      /* e4m3 kv only */
+} cppmega_mi355_sparse_mla_bwd_args_t;
+
+int cppmega_mi355_sparse_mla_bwd(const cppmega_mi355_sparse_mla_bwd_args_t* args, size_t args_size, void* stream);
+
 /* ---- FP8 vecmat / skinny GEMM ----------------------------------------------
  * Replaces fp8_vecmat_reduce_direct, called as kernel(A, A_scale, B, B_scale, C)
  * (cppmega_mlx/nn/_tilelang/fp8_vecmat_path_c.py:737-821, 1039-1046) and the

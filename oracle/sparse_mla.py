@@ -175,3 +175,42 @@ def sparse_mla_scores_oracle(q: np.ndarray, kv: np.ndarray, indices: np.ndarray,
                 sc = (qs @ rows.T) * float(sm_scale)
                 out[b, s, g * hpg:(g + 1) * hpg] = np.where(ok[None, :], sc, INVALID_SCORE_SENTINEL).astype(np.float32)
     return out
+
+
+def sparse_mla_bwd_oracle(q, kv, indices, d_out, *, sm_scale: float | None = None, d_v: int | None = None):
+    """Float64 gradients (dq [B,S,H,D], dkv [B,Skv,G,D]) of ``sparse_mla_oracle``'s output for the
+    cotangent ``d_out`` [B,S,H,d_v]; the closed form of the reference's backward kernel
+    (cppmega_mlx/nn/_tilelang/sparse_mla_path_c.py:2700-2814): p = softmax over the valid
+    selected keys, dp_k = d_out . kv_k[:d_v], ds = p * (dp - sum p dp), dq = sm_scale * ds . K,
+    dkv[i_k] += sm_scale * ds_k * q (+ p_k * d_out on the first d_v channels).  A key index
+    < 0 or >= Skv is skipped (the forward's rule); repeated indices accumulate.
+    Pinned in tests/test_oracle_sparse_mla.py by central finite differences of the forward
+    oracle and by torch autograd through a dense masked attention."""
+    q = np.asarray(q, dtype=np.float64)
+    kv = np.asarray(kv, dtype=np.float64)
+    d_out = np.asarray(d_out, dtype=np.float64)
+    indices = np.asarray(indices)
+    B, S, H, D, Skv, G, hpg, dv, topk = resolve_shapes(q, kv, indices, d_v)
+    scale = D ** -0.5 if sm_scale is None else float(sm_scale)
+    dq = np.zeros_like(q)
+    dkv = np.zeros_like(kv)
+    for b in range(B):
+        for s in range(S):
+            for g in range(G):
+                idx = indices[b, s, g].astype(np.int64)
+                valid = (idx >= 0) & (idx < Skv)
+                if not valid.any():
+                    continue
+                sel = idx[valid]
+                rows = kv[b, sel, g, :]                                    # [n, D]
+                for h in range(g * hpg, (g + 1) * hpg):
+                    sc = rows @ q[b, s, h] * scale
+                    e = np.exp(sc - sc.max())
+                    p = e / e.sum()
+                    dp = rows[:, :dv] @ d_out[b, s, h]
+                    ds = p * (dp - np.dot(p, dp))
+                    dq[b, s, h] = scale * (ds @ rows)
+                    contrib = scale * np.outer(ds, q[b, s, h])
+                    contrib[:, :dv] += np.outer(p, d_out[b, s, h])
+                    np.add.at(dkv[b, :, g, :], sel, contrib)
+    return dq, dkv

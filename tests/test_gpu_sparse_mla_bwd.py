@@ -1,0 +1,123 @@
+"""GPU parity: the float-carrier sparse-MLA backward (through the C ABI) vs the float64 oracle.
+
+dkv is accumulated with float32 atomic adds, so results agree to rounding, not bit for bit:
+float32 carriers are held to 1e-4 of each gradient's scale, half carriers to 2e-2 for dq (one
+rounding of the result) and 1e-2 for the float32 dkv (inputs are already rounded; the oracle
+sees the same values)."""
+
+import numpy as np
+import pytest
+import torch
+
+from cppmega_mlx_amd import ops
+from cppmega_mlx_amd.nn._tilelang import sparse_mla_path_c as pc
+from oracle import sparse_mla as om
+from tests._inputs import error_report, sparse_indices, to_dev
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    dict(B=1, S=4, H=4, G=1, Skv=32, topk=8, D=64, d_v=64),
+    dict(B=2, S=5, H=8, G=2, Skv=64, topk=16, D=64, d_v=48),
+    dict(B=1, S=3, H=6, G=3, Skv=300, topk=100, D=128, d_v=32),
+    dict(B=1, S=2, H=16, G=1, Skv=256, topk=64, D=576, d_v=512),       # the tiny bf16 configuration's widths
+    dict(B=1, S=2, H=2, G=1, Skv=50, topk=37, D=20, d_v=7),
+]
+
+
+@pytest.mark.parametrize("shape", CASES, ids=lambda c: "B%dS%dH%dG%dT%dk%dD%ddv%d" % tuple(c.values()))
+@pytest.mark.parametrize("carrier", [torch.float32, torch.bfloat16, torch.float16])
+def test_backward_matches_oracle(device, shape, carrier):
+    B, S, H, G, Skv, topk, D, d_v = shape.values()
+    rng = np.random.default_rng(B * 100 + S * 10 + D)
+    qt = to_dev(rng.standard_normal((B, S, H, D)).astype(np.float32), device).to(carrier)
+    kt = to_dev(rng.standard_normal((B, Skv, G, D)).astype(np.float32), device).to(carrier)
+    dt = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(carrier)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)      # repeated keys accumulate
+    idx[rng.random(idx.shape) < 0.2] = -1
+    idx[0, 1] = -1                                                   # a query with nothing to attend to
+    idx[0, 0, 0, 0] = Skv + 5                                        # out of range: skipped
+    want_dq, want_dkv = om.sparse_mla_bwd_oracle(qt.double().cpu().numpy(), kt.double().cpu().numpy(), idx,
+                                                 dt.double().cpu().numpy(), sm_scale=D ** -0.5, d_v=d_v)
+    dq = torch.full((B, S, H, D), 9.0, dtype=carrier, device=device)
+    dkv = torch.full((B, Skv, G, D), 9.0, dtype=torch.float32, device=device)
+    got = ops.sparse_mla_backward(qt, kt, dt, to_dev(idx.astype(np.int32), device), sm_scale=D ** -0.5, d_v=d_v, dq=dq, dkv=dkv)
+    torch.cuda.synchronize()
+    assert got[0] is dq and got[1] is dkv
+    half = carrier != torch.float32
+    err, ref = error_report(dq.float().cpu().numpy(), want_dq)
+    assert err <= (2e-2 if half else 1e-4) * ref, (err, ref)
+    err, ref = error_report(dkv.cpu().numpy(), want_dkv)
+    assert err <= 1e-4 * ref, (err, ref)
+    assert (dq[0, 1] == 0).all()
+    # accumulate on top of existing contents when asked not to clear
+    ops.sparse_mla_backward(qt, kt, dt, to_dev(idx, device), sm_scale=torch.tensor([D ** -0.5], device=device), d_v=d_v, dq=dq, dkv=dkv,
+                            clear_dkv=False)
+    torch.cuda.synchronize()
+    err, ref = error_report(dkv.cpu().numpy(), 2 * want_dkv)
+    assert err <= 2e-4 * ref
+
+
+def test_public_backward_entry_points_and_autograd(device):
+    rng = np.random.default_rng(8)
+    B, S, H, G, Skv, topk, D = 2, 4, 4, 2, 48, 12, 64
+    q = to_dev(rng.standard_normal((B, S, H, D)).astype(np.float32), device)
+    kv = to_dev(rng.standard_normal((B, Skv, G, D)).astype(np.float32), device)
+    d_out = to_dev(rng.standard_normal((B, S, H, D)).astype(np.float32), device)
+    idx = sparse_indices(rng, B, S, G, Skv, topk)
+    idx[..., -2:] = -1
+    it = to_dev(idx, device)
+    want_dq, want_dkv = om.sparse_mla_bwd_oracle(q.cpu().numpy(), kv.cpu().numpy(), idx, d_out.cpu().numpy())
+    dq, dkv = pc.sparse_mla_bwd_path_c(q, kv, d_out, it)
+    torch.cuda.synchronize()
+    assert dq.dtype == torch.float32 and dkv.dtype == torch.float32
+    np.testing.assert_allclose(dq.cpu().numpy(), want_dq, atol=1e-4 * np.abs(want_dq).max())
+    np.testing.assert_allclose(dkv.cpu().numpy(), want_dkv, atol=1e-4 * np.abs(want_dkv).max())
+    qa, ka = q.clone().requires_grad_(True), kv.clone().requires_grad_(True)
+    out = pc.sparse_mla_path_c_metal_apply(qa, ka, it)
+    (out * d_out).sum().backward()
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(qa.grad.cpu().numpy(), want_dq, atol=1e-4 * np.abs(want_dq).max())
+    np.testing.assert_allclose(ka.grad.cpu().numpy(), want_dkv, atol=1e-4 * np.abs(want_dkv).max())
+    with pytest.raises(pc.SparseMLAPathCDirectError):
+        pc._sparse_mla_bwd_path_c_direct(q, kv.half(), d_out, it, sm_scale_buf=torch.tensor([0.1], device=device))
+    with pytest.raises(ValueError):
+        ops.sparse_mla_backward(q, kv, d_out, it, sm_scale=0.1, d_v=D, dq=torch.empty_like(q), dkv=torch.empty_like(kv).half())
+
+
+def test_per_token_fp8_backward_over_prepared_buffers(device):
+    """fp8_sparse_mla_bwd_kernel's contract: gradients with respect to the dequantised q and kv."""
+    from cppmega_mlx_amd.nn._tilelang import sparse_mla_fp8_path_c as f8
+    from oracle import fp8
+
+    rng = np.random.default_rng(12)
+    B, S, H, G, Skv, topk, D, d_v = 2, 5, 4, 2, 40, 16, 64, 32
+    qc, qs = fp8.quantize_per_token(rng.standard_normal((B * S * H, D)).astype(np.float32))
+    kc, ks = fp8.quantize_per_token(rng.standard_normal((B * Skv * G, D)).astype(np.float32))
+    qc, qs, kc, ks = qc.reshape(B, S, H, D), qs.reshape(B, S, H), kc.reshape(B, Skv, G, D), ks.reshape(B, Skv, G)
+    d_out = rng.standard_normal((B, S, H, d_v)).astype(np.float32)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[0, 2] = -1
+    idx[1, 0, 0, :3] = Skv + 1
+    want_dq, want_dkv = om.sparse_mla_bwd_oracle(om.dequant_per_token(qc, qs), om.dequant_per_token(kc, ks), idx, d_out,
+                                                 sm_scale=0.2, d_v=d_v)
+    args = (to_dev(qc, device), to_dev(qs, device), to_dev(kc, device), to_dev(ks, device))
+    for dtype in (torch.float32, torch.float16):
+        dq, dkv = f8.sparse_mla_fp8_bwd_path_c(*args, to_dev(d_out, device).to(dtype), to_dev(idx.astype(np.int32), device),
+                                               sm_scale=0.2, d_v=d_v)
+        torch.cuda.synchronize()
+        tol = 1e-4 if dtype == torch.float32 else 2e-3
+        for got, want in ((dq, want_dq), (dkv, want_dkv)):
+            assert got.dtype == torch.float32
+            err, ref = error_report(got.cpu().numpy(), want)
+            assert err <= tol * ref, (err, ref)
+    dq_buf = torch.zeros((B, S, H, D), dtype=torch.float32, device=device)
+    dkv_buf = torch.full((B, Skv, G, D), 3.0, dtype=torch.float32, device=device)
+    got = f8.sparse_mla_fp8_bwd_path_c(*args, to_dev(d_out, device), to_dev(idx, device), sm_scale=0.2, d_v=d_v,
+                                       dq_buffer=dq_buf, dkv_buffer=dkv_buf)
+    torch.cuda.synchronize()
+    assert got[0] is dq_buf and got[1] is dkv_buf
+    err, ref = error_report(dkv_buf.cpu().numpy(), want_dkv)
+    assert err <= 1e-4 * ref
+    with pytest.raises(ValueError):
+        f8.sparse_mla_fp8_bwd_path_c(*args, to_dev(d_out, device)[..., :8].contiguous(), to_dev(idx, device), sm_scale=0.2, d_v=d_v)

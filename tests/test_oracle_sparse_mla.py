@@ -113,3 +113,59 @@ def test_shape_validation_messages():
         om.sparse_mla_oracle(q, kv, idx, d_v=17)
     with pytest.raises(ValueError, match="not divisible by kv_group"):
         om.sparse_mla_oracle(q[:, :, :3], kv, idx)
+
+
+def _bwd_case(rng, B=1, S=2, H=4, G=2, Skv=9, topk=5, D=6, d_v=4):
+    q = rng.standard_normal((B, S, H, D))
+    kv = rng.standard_normal((B, Skv, G, D))
+    idx = rng.integers(0, Skv, (B, S, G, topk))
+    idx[0, 0, 0, 1] = idx[0, 0, 0, 0]          # a repeated key
+    idx[0, 1, 1, 2] = -1                       # a skipped slot
+    idx[0, 1, 0, 3] = Skv + 2                  # out of range: skipped as well
+    d_out = rng.standard_normal((B, S, H, d_v))
+    return q, kv, idx, d_out, d_v
+
+
+def test_backward_oracle_matches_finite_differences_of_the_forward_oracle():
+    rng = np.random.default_rng(31)
+    q, kv, idx, d_out, d_v = _bwd_case(rng)
+    dq, dkv = om.sparse_mla_bwd_oracle(q, kv, idx, d_out, sm_scale=0.37, d_v=d_v)
+
+    def loss(q_, kv_):
+        out, _ = om.sparse_mla_oracle(q_, kv_, idx, sm_scale=0.37, d_v=d_v)
+        return float((out * d_out).sum())
+
+    eps = 1e-6
+    for arr, grad in ((q, dq), (kv, dkv)):
+        num = np.zeros_like(arr)
+        it = np.nditer(arr, flags=["multi_index"])
+        for _ in it:
+            i = it.multi_index
+            hi, lo = arr.copy(), arr.copy()
+            hi[i] += eps
+            lo[i] -= eps
+            num[i] = (loss(hi, kv) - loss(lo, kv)) / (2 * eps) if arr is q else (loss(q, hi) - loss(q, lo)) / (2 * eps)
+        np.testing.assert_allclose(grad, num, atol=1e-7, rtol=1e-6)
+    # rows nobody selected get no gradient; a fully skipped query row gives none either
+    assert (dkv[0, [i for i in range(9) if i not in set(idx[idx >= 0].ravel().tolist())]] == 0).all()
+    idx2 = idx.copy(); idx2[0, 0] = -1
+    dq2, _ = om.sparse_mla_bwd_oracle(q, kv, idx2, d_out, sm_scale=0.37, d_v=d_v)
+    assert (dq2[0, 0] == 0).all()
+
+
+def test_backward_oracle_matches_torch_autograd_through_dense_attention():
+    rng = np.random.default_rng(32)
+    B, S, H, G, Skv, topk, D, d_v = 2, 3, 4, 2, 7, 4, 8, 8
+    q = rng.standard_normal((B, S, H, D)); kv = rng.standard_normal((B, Skv, G, D))
+    idx = np.stack([np.stack([np.stack([rng.choice(Skv, topk, replace=False) for _ in range(G)]) for _ in range(S)]) for _ in range(B)])
+    d_out = rng.standard_normal((B, S, H, d_v))
+    dq, dkv = om.sparse_mla_bwd_oracle(q, kv, idx, d_out, d_v=d_v)
+    qt = torch.tensor(q, requires_grad=True); kt = torch.tensor(kv, requires_grad=True)
+    mask = torch.full((B, S, G, Skv), float("-inf"), dtype=torch.float64)
+    mask.scatter_(3, torch.tensor(idx), 0.0)
+    kh = kt.repeat_interleave(H // G, dim=2)                                   # [B, Skv, H, D]
+    logits = torch.einsum("bshd,bkhd->bshk", qt, kh) * D ** -0.5 + mask.repeat_interleave(H // G, dim=2)
+    out = torch.einsum("bshk,bkhd->bshd", torch.softmax(logits, dim=-1), kh[..., :d_v])
+    (out * torch.tensor(d_out)).sum().backward()
+    np.testing.assert_allclose(dq, qt.grad.numpy(), atol=1e-12, rtol=1e-10)
+    np.testing.assert_allclose(dkv, kt.grad.numpy(), atol=1e-12, rtol=1e-10)
