@@ -473,6 +473,23 @@ def bench_next_rows(args, device):
         "us_per_launch": secs / steps * 1e6, "algorithmic_flops": flops,
         "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 157.3, "unit": "TFLOP/s",
                      "frac": flops / (secs / steps) / 1e12 / 157.3, "traffic": None}}
+
+    # DSA indexer KL loss (training side): one launch over every (batch, query position)
+    ASq = Sk = 4096; AB, AH, AD, topk = 1, 8, 64, 1024
+    qq = torch.randn((ASq, AB, AH, AD), generator=gen, device=device).to(torch.bfloat16)
+    kk = torch.randn((Sk, AB, AH, AD), generator=gen, device=device).to(torch.bfloat16)
+    isc = torch.randn((AB, ASq, Sk), generator=gen, device=device)
+    top = torch.topk(isc, topk, dim=-1).indices.to(torch.int32).contiguous()
+    loss = torch.empty((AB, ASq), dtype=torch.float32, device=device)
+    for name, lst in (("dsa_indexer_loss_dense", None), ("dsa_indexer_loss_sparse", top)):
+        secs, _ = timed_graph([lambda: ops.dsa_indexer_loss(qq, kk, isc, softmax_scale=AD ** -0.5, out=loss, topk_indices=lst)], steps, args.warmup)
+        flops = 2.0 * AB * AH * AD * (ASq * (ASq + 1) / 2)
+        res[name] = {
+            "workload": f"dsa_indexer_loss query/key bf16[{ASq},{AB},{AH},{AD}] index_scores f32[{AB},{ASq},{Sk}]"
+                        + (f" topk_indices i32[{AB},{ASq},{topk}]" if lst is not None else "") + " -> loss f32",
+            "us_per_launch": secs / steps * 1e6, "algorithmic_flops": flops,
+            "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 157.3, "unit": "TFLOP/s",
+                         "frac": flops / (secs / steps) / 1e12 / 157.3, "traffic": None}}
     return res
 
 

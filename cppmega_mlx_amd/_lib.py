@@ -50,6 +50,7 @@ EXPORTED_SYMBOLS = (
     "cppmega_mi355_fp8_vecmat",
     "cppmega_mi355_fp8_quantize",
     "cppmega_mi355_head_gemm",
+    "cppmega_mi355_dsa_indexer_loss",
     "cppmega_mi355_sparse_mla_bwd",
     "cppmega_mi355_dequant_block_fp8",
     "cppmega_mi355_kv_cache_append",
@@ -160,6 +161,27 @@ class SparseMlaBwdArgs(C.Structure):
         ("dkv", C.c_void_p),
         ("q_scale", C.c_void_p),
         ("kv_scale", C.c_void_p),
+    ]
+
+
+class DsaLossArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("in_dtype", C.c_int32),
+        ("query", C.c_void_p),
+        ("key", C.c_void_p),
+        ("index_scores", C.c_void_p),
+        ("index_mask", C.c_void_p),
+        ("loss", C.c_void_p),
+        ("seq_q", C.c_int32),
+        ("batch", C.c_int32),
+        ("heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("seq_k", C.c_int32),
+        ("softmax_scale", C.c_float),
+        ("topk_indices", C.c_void_p),
+        ("topk", C.c_int32),
+        ("index_dtype", C.c_int32),
     ]
 
 
@@ -394,6 +416,8 @@ def load() -> C.CDLL:
         lib.cppmega_mi355_fp8_quantize.restype = C.c_int
         lib.cppmega_mi355_sparse_mla_bwd.argtypes = [C.POINTER(SparseMlaBwdArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_sparse_mla_bwd.restype = C.c_int
+        lib.cppmega_mi355_dsa_indexer_loss.argtypes = [C.POINTER(DsaLossArgs), C.c_size_t, C.c_void_p]
+        lib.cppmega_mi355_dsa_indexer_loss.restype = C.c_int
         lib.cppmega_mi355_head_gemm.argtypes = [C.POINTER(HeadGemmArgs), C.c_size_t, C.c_void_p]
         lib.cppmega_mi355_head_gemm.restype = C.c_int
         lib.cppmega_mi355_dequant_block_fp8.argtypes = [C.POINTER(DequantBlockArgs), C.c_size_t, C.c_void_p]

@@ -37,6 +37,7 @@ int kv_cache_append_launch(const cppmega_mi355_cache_append_args_t& a, hipStream
 int causal_indices_launch(const cppmega_mi355_causal_indices_args_t& a, hipStream_t stream);
 int mask_indices_launch(const cppmega_mi355_mask_indices_args_t& a, hipStream_t stream);
 int sparse_mla_bwd_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStream_t stream);
+int dsa_indexer_loss_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStream_t stream);
 int head_gemm_launch(const cppmega_mi355_head_gemm_args_t& a, hipStream_t stream);
 int dequant_block_fp8_launch(const cppmega_mi355_dequant_block_args_t& a, hipStream_t stream);
 int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t stream);
@@ -331,6 +332,11 @@ int cppmega_mi355_sparse_mla_scores(const cppmega_mi355_sparse_mla_args_t* args,
 int cppmega_mi355_sparse_mla_bwd(const cppmega_mi355_sparse_mla_bwd_args_t* args, size_t args_size, void* stream) {
   CM_CHECK_ARGS(args, args_size, cppmega_mi355_sparse_mla_bwd_args_t);
   return sparse_mla_bwd_launch(*args, (hipStream_t)stream);
+}
+
+int cppmega_mi355_dsa_indexer_loss(const cppmega_mi355_dsa_loss_args_t* args, size_t args_size, void* stream) {
+  CM_CHECK_ARGS(args, args_size, cppmega_mi355_dsa_loss_args_t);
+  return dsa_indexer_loss_launch(*args, (hipStream_t)stream);
 }
 
 int cppmega_mi355_head_gemm(const cppmega_mi355_head_gemm_args_t* args, size_t args_size, void* stream) {

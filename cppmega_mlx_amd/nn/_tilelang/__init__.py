@@ -5,6 +5,7 @@ Exports the hot-path names of the reference's
 """
 
 from ._engine_dispatch import dispatch_lower, tilelang_engine_mode
+from .dsa_splitk_indexer_loss import dsa_splitk_indexer_loss_tilelang, dsa_splitk_path_c_status
 from .fp8_msl_kernels import fp8_scaled_vecmat
 from .fp8_vecmat_path_c import (
     FP8VecmatPathCDirectError,
@@ -34,6 +35,8 @@ __all__ = [
     "FP8VecmatPathCDirectError",
     "FP8VecmatPathCLegacyError",
     "dispatch_lower",
+    "dsa_splitk_indexer_loss_tilelang",
+    "dsa_splitk_path_c_status",
     "fp8_scaled_vecmat",
     "fp8_scaled_vecmat_path_c",
     "fp8_scaled_vecmat_path_c_direct",

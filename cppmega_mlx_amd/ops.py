@@ -260,6 +260,48 @@ def dequant_block_fp8(weight: torch.Tensor, scale_inv: torch.Tensor, *, out: tor
 
 
 # ---------------------------------------------------------------------------
+# DSA indexer KL loss (training side)
+# ---------------------------------------------------------------------------
+def dsa_indexer_loss(query: torch.Tensor, key: torch.Tensor, index_scores: torch.Tensor, *, softmax_scale: float,
+                     out: torch.Tensor, index_mask: torch.Tensor | None = None,
+                     topk_indices: torch.Tensor | None = None) -> torch.Tensor:
+    """Per-position KL(attention || index) into caller-owned float32 ``out`` [AB, ASq];
+    ``query`` [ASq, AB, AH, AD], ``key`` [Sk, AB, AH, AD], ``index_scores`` / ``index_mask`` float32 [AB, ASq, Sk];
+    ``topk_indices`` int32 / int64 [AB, ASq, topk] restricts both distributions to the listed keys."""
+    for name, t in (("query", query), ("key", key), ("index_scores", index_scores), ("out", out), ("index_mask", index_mask),
+                    ("topk_indices", topk_indices)):
+        if t is not None:
+            _lib.require_device_tensor(t, name, query if name != "query" else None)
+    if query.ndim != 4 or key.ndim != 4 or tuple(query.shape[1:]) != tuple(key.shape[1:]):
+        raise ValueError(f"query/key shape mismatch: query {tuple(query.shape)}, key {tuple(key.shape)}")
+    ASq, AB, AH, AD = query.shape
+    Sk = key.shape[0]
+    if key.dtype != query.dtype:
+        raise TypeError("query/key dtypes must match")
+    for name, t in (("index_scores", index_scores), ("index_mask", index_mask)):
+        if t is not None and (tuple(t.shape) != (AB, ASq, Sk) or t.dtype != torch.float32):
+            raise ValueError(f"{name} must be float32 with shape {(AB, ASq, Sk)}; got {t.dtype} {tuple(t.shape)}")
+    if tuple(out.shape) != (AB, ASq) or out.dtype != torch.float32:
+        raise ValueError(f"out must be float32 with shape {(AB, ASq)}; got {out.dtype} {tuple(out.shape)}")
+    a = _lib.DsaLossArgs()
+    a.struct_size = C.sizeof(a)
+    a.in_dtype = _dtype_or_raise(query, "query", (_lib.F32, _lib.F16, _lib.BF16))
+    a.query, a.key, a.index_scores, a.index_mask, a.loss = (query.data_ptr(), key.data_ptr(), index_scores.data_ptr(),
+                                                            _lib.ptr(index_mask), out.data_ptr())
+    a.seq_q, a.batch, a.heads, a.head_dim, a.seq_k = ASq, AB, AH, AD, Sk
+    a.softmax_scale = float(softmax_scale)
+    if topk_indices is not None:
+        if topk_indices.ndim != 3 or tuple(topk_indices.shape[:2]) != (AB, ASq):
+            raise ValueError(f"topk_indices must have shape (AB={AB}, ASq={ASq}, TOPK); got {tuple(topk_indices.shape)}")
+        a.topk_indices, a.topk = topk_indices.data_ptr(), int(topk_indices.shape[2])
+        a.index_dtype = _dtype_or_raise(topk_indices, "topk_indices", (_lib.I32, _lib.I64))
+    with torch.cuda.device(query.device):
+        rc = _lib.load().cppmega_mi355_dsa_indexer_loss(C.byref(a), C.sizeof(a), _lib.current_stream(query.device))
+    _lib.check(rc, "dsa_indexer_loss")
+    return out
+
+
+# ---------------------------------------------------------------------------
 # sparse MLA
 # ---------------------------------------------------------------------------
 

@@ -339,6 +339,37 @@ typedef struct cppmega_mi355_sparse_mla_bwd_args {
 
 int cppmega_mi355_sparse_mla_bwd(const cppmega_mi355_sparse_mla_bwd_args_t* args, size_t args_size, void* stream);
 
+/* ---- DSA indexer KL loss, per position ---------------------------------------------
+ * Replaces the two kernels behind dsa_splitk_indexer_loss_tilelang
+ * (cppmega_mlx/nn/_tilelang/dsa_splitk_indexer_loss.py: dsa_stage1 :398-656, dsa_stage2
+ * :855-1165, called at :1514-1570):
+ *   loss[b, sq] = sum_{j <= sq} p[j] * (log(p[j] + 1e-10) - log(q[j] + 1e-10))
+ *   p = head average of the causal attention softmax of softmax_scale * query . key
+ *       (+ index_mask), q = softmax over all keys of index_scores (+ index_mask)
+ *   query [ASq, AB, AH, AD], key [Sk, AB, AH, AD]: float32 / float16 / bfloat16
+ *   index_scores, index_mask [AB, ASq, Sk] float32 (index_mask NULL = no additive mask)
+ *   topk_indices [AB, ASq, topk] int32 / int64 or NULL: the sparse loss.  A key that is not
+ *       in its row's list counts as masked with -inf, which is what the reference's
+ *       scatter(-inf, topk_indices, 0) mask (:1443-1445) adds, without the [AB, ASq, Sk]
+ *       tensor; entries outside [0, Sk) select nothing; topk must be >= 1.
+ *   loss [AB, ASq] float32.  The caller takes mean(loss) * loss_coeff. */
+typedef struct cppmega_mi355_dsa_loss_args {
+  uint32_t struct_size;
+  int32_t in_dtype;
+  const void* query;
+  const void* key;
+  const float* index_scores;
+  const float* index_mask;
+  float* loss;
+  int32_t seq_q, batch, heads, head_dim, seq_k;
+  float softmax_scale;
+  const void* topk_indices;
+  int32_t topk;
+  int32_t index_dtype;
+} cppmega_mi355_dsa_loss_args_t;
+
+int cppmega_mi355_dsa_indexer_loss(const cppmega_mi355_dsa_loss_args_t* args, size_t args_size, void* stream);
+
 /* ---- FP8 vecmat / skinny GEMM ----------------------------------------------
  * Replaces fp8_vecmat_reduce_direct, called as kernel(A, A_scale, B, B_scale, C)
  * (cppmega_mlx/nn/_tilelang/fp8_vecmat_path_c.py:737-821, 1039-1046) and the

@@ -40,6 +40,7 @@ STRUCTS = {
     "cppmega_mi355_topk_args_t": _lib.TopkArgs,
     "cppmega_mi355_indexer_args_t": _lib.IndexerArgs,
     "cppmega_mi355_head_gemm_args_t": _lib.HeadGemmArgs,
+    "cppmega_mi355_dsa_loss_args_t": _lib.DsaLossArgs,
     "cppmega_mi355_sparse_mla_bwd_args_t": _lib.SparseMlaBwdArgs,
     "cppmega_mi355_dequant_block_args_t": _lib.DequantBlockArgs,
     "cppmega_mi355_sparse_mla_args_t": _lib.SparseMlaArgs,
