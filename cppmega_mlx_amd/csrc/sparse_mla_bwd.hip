@@ -165,6 +165,9 @@ bool operand_dtype(int dt) { return float_carrier(dt) || dt == CPPMEGA_MI355_E4M
 
 }  // namespace
 
+bool sparse_mla_bwd_mfma_supports(const cppmega_mi355_sparse_mla_bwd_args_t& a);                    // sparse_mla_bwd_mfma.hip
+int sparse_mla_bwd_mfma_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStream_t stream);
+
 int sparse_mla_bwd_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStream_t stream) {
   if (!a.q || !a.kv || !a.d_out || !a.indices || !a.dq || !a.dkv) return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla_bwd: a pointer is NULL");
   if (a.batch < 0 || a.seq_q < 0 || a.heads < 1 || a.kv_groups < 1 || a.seq_kv < 0 || a.topk < 0 || a.d_qk < 1)
@@ -177,8 +180,9 @@ int sparse_mla_bwd_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStrea
     return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla_bwd: e4m3 operands need their per-token scales");
   if (a.index_dtype != CPPMEGA_MI355_I32 && a.index_dtype != CPPMEGA_MI355_I64)
     return fail(CPPMEGA_MI355_ERR_DTYPE, "sparse_mla_bwd: indices must be int32 or int64");
+  const bool on_matrix_cores = sparse_mla_bwd_mfma_supports(a);      // bfloat16 q, kv and d_out
   const size_t lds = ((size_t)3 * a.topk + a.d_qk + a.d_v + 8) * sizeof(float);
-  if (lds > 160 * 1024) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: topk %d with d_qk %d needs %zu bytes of LDS (limit 160 KiB)", a.topk, a.d_qk, lds);
+  if (!on_matrix_cores && lds > 160 * 1024) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: topk %d with d_qk %d needs %zu bytes of LDS (limit 160 KiB)", a.topk, a.d_qk, lds);
   const size_t n_dkv = (size_t)a.batch * a.seq_kv * a.kv_groups * a.d_qk;
   if (a.clear_dkv && n_dkv) {
     size_t blocks = (n_dkv + kThreads * 8 - 1) / (kThreads * 8);
@@ -187,6 +191,7 @@ int sparse_mla_bwd_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStrea
   }
   const size_t lanes = (size_t)a.batch * a.seq_q * a.heads;
   if (lanes == 0) return 0;
+  if (on_matrix_cores) return sparse_mla_bwd_mfma_launch(a, stream);
   if (lanes > 0x7fffffffull) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: too many (batch, query, head) rows for one launch");
   BwdParams p;
   p.q = a.q; p.kv = a.kv; p.d_out = a.d_out; p.indices = a.indices; p.sm_scale_dev = a.sm_scale_dev; p.dq = a.dq; p.dkv = a.dkv;

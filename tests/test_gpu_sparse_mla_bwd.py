@@ -58,6 +58,49 @@ def test_backward_matches_oracle(device, shape, carrier):
     assert err <= 2e-4 * ref
 
 
+MATRIX_CORE_CASES = [
+    dict(B=1, S=3, H=16, G=1, Skv=256, topk=100, D=576, d_v=512),      # one chunk of 16 heads, a partial last tile
+    dict(B=1, S=2, H=40, G=1, Skv=300, topk=70, D=576, d_v=512),       # chunks of 32 heads, the second one with 8
+    dict(B=2, S=3, H=24, G=2, Skv=200, topk=130, D=128, d_v=64),       # 12 heads per group, three tiles
+    dict(B=1, S=4, H=64, G=1, Skv=64, topk=33, D=64, d_v=64),          # d_v == d_qk
+    dict(B=1, S=2, H=1, G=1, Skv=40, topk=5, D=96, d_v=32),            # a single head
+    dict(B=1, S=2, H=128, G=1, Skv=512, topk=256, D=576, d_v=512),     # the production head count
+]
+
+
+@pytest.mark.parametrize("shape", MATRIX_CORE_CASES, ids=lambda c: "B%dS%dH%dG%dT%dk%dD%ddv%d" % tuple(c.values()))
+@pytest.mark.parametrize("index_dtype", [np.int32, np.int64])
+def test_bfloat16_backward_on_the_matrix_cores(device, shape, index_dtype):
+    """bfloat16 q / kv / d_out take the matrix-core kernel; with float32 dq both gradients are held to
+    1e-4 of their scale (P and dS enter the second products as hi + lo bfloat16 planes)."""
+    B, S, H, G, Skv, topk, D, d_v = shape.values()
+    rng = np.random.default_rng(B * 1000 + H * 10 + topk)
+    qt = to_dev(rng.standard_normal((B, S, H, D)).astype(np.float32), device).to(torch.bfloat16)
+    kt = to_dev(rng.standard_normal((B, Skv, G, D)).astype(np.float32), device).to(torch.bfloat16)
+    dt = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(torch.bfloat16)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[rng.random(idx.shape) < 0.15] = -1
+    idx[0, 1] = -1
+    idx[0, 0, 0, 0] = Skv + 5
+    sm = 1.7 * D ** -0.5
+    want_dq, want_dkv = om.sparse_mla_bwd_oracle(qt.double().cpu().numpy(), kt.double().cpu().numpy(), idx,
+                                                 dt.double().cpu().numpy(), sm_scale=sm, d_v=d_v)
+    dq = torch.full((B, S, H, D), 9.0, dtype=torch.float32, device=device)
+    dkv = torch.full((B, Skv, G, D), 9.0, dtype=torch.float32, device=device)
+    ops.sparse_mla_backward(qt, kt, dt, to_dev(idx.astype(index_dtype), device), sm_scale=sm, d_v=d_v, dq=dq, dkv=dkv)
+    torch.cuda.synchronize()
+    for got, want in ((dq, want_dq), (dkv, want_dkv)):
+        err, ref = error_report(got.cpu().numpy(), want)
+        assert err <= 1e-4 * ref, (err, ref)
+    assert (dq[0, 1] == 0).all()
+    # bfloat16 dq: one rounding of the same values
+    dq16 = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=device)
+    ops.sparse_mla_backward(qt, kt, dt, to_dev(idx.astype(index_dtype), device), sm_scale=torch.tensor([sm], device=device), d_v=d_v,
+                            dq=dq16, dkv=dkv)
+    torch.cuda.synchronize()
+    assert torch.equal(dq16, dq.to(torch.bfloat16))
+
+
 def test_public_backward_entry_points_and_autograd(device):
     rng = np.random.default_rng(8)
     B, S, H, G, Skv, topk, D = 2, 4, 4, 2, 48, 12, 64
