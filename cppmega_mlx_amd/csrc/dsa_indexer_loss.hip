@@ -165,6 +165,9 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_kernel(const LossPa
 
 }  // namespace
 
+bool dsa_indexer_loss_mfma_supports(const cppmega_mi355_dsa_loss_args_t& a);                    // dsa_indexer_loss_mfma.hip
+int dsa_indexer_loss_mfma_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStream_t stream);
+
 int dsa_indexer_loss_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStream_t stream) {
   if (!a.query || !a.key || !a.index_scores || !a.loss) return fail(CPPMEGA_MI355_ERR_NULL, "dsa_indexer_loss: a pointer is NULL");
   if (a.seq_q < 0 || a.batch < 0 || a.heads < 0 || a.head_dim < 0 || a.seq_k < 0)
@@ -178,6 +181,7 @@ int dsa_indexer_loss_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStream_t 
     if (a.index_dtype != CPPMEGA_MI355_I32 && a.index_dtype != CPPMEGA_MI355_I64)
       return fail(CPPMEGA_MI355_ERR_DTYPE, "dsa_indexer_loss: topk_indices must be int32 or int64");
   }
+  if (dsa_indexer_loss_mfma_supports(a)) return dsa_indexer_loss_mfma_launch(a, stream);    // bfloat16 / float16 rows
   const size_t lds = ((size_t)2 * a.seq_k + a.head_dim + 8 + (a.seq_k + 31) / 32) * sizeof(float);
   if (lds > 160 * 1024) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "dsa_indexer_loss: Sk %d needs %zu bytes of LDS (limit 160 KiB)", a.seq_k, lds);
   if ((size_t)a.seq_q * a.batch > 0x7fffffffull) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "dsa_indexer_loss: too many rows for one launch");

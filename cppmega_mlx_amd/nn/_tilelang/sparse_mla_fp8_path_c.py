@@ -10,6 +10,10 @@ score = (sum dec*dec) * qs * ks * sm_scale, optional attention ``sinks`` ``[H]``
 
 ``sparse_mla_fp8_bwd_path_c`` :3007-3080 is the backward over the same prepared
 buffers (kernel :1966-2214): float32 gradients with respect to the dequantised q and kv.
+``sparse_mla_fp8_path_c_apply_prepared_float`` :3138-3252 is the differentiable owner wrapper
+(forward over the prepared buffers, gradients delivered straight through to the float q / kv
+the buffers were produced from); ``sparse_mla_fp8_path_c_apply_from_float`` :3255-3280 fails
+closed, as in the reference.
 
 A float32 ``kv_scale`` of rank 4 selects the block-128 latent layout described
 in ``sparse_mla_blockscaled_path_c`` (per-token is its one-block case), so the
@@ -32,6 +36,8 @@ __all__ = [
     "sparse_mla_fp8_path_c_apply_direct",
     "sparse_mla_fp8_path_c_status",
     "sparse_mla_fp8_bwd_path_c",
+    "sparse_mla_fp8_path_c_apply_from_float",
+    "sparse_mla_fp8_path_c_apply_prepared_float",
     "fp8_sparse_mla_indexed_qk_reduce_path_c",
     "fp8_sparse_mla_qk_reduce_path_c",
 ]
@@ -207,6 +213,65 @@ def sparse_mla_fp8_bwd_path_c(
     except (_lib.NativeCallError, _lib.NativeLibraryError) as exc:
         raise SparseMLAFp8PathCDirectError(f"FP8 sparse-MLA backward dispatch failed: {type(exc).__name__}: {exc}") from exc
     return dq, dkv
+
+
+class _PreparedFloatFunction(torch.autograd.Function):
+    """Forward over prepared FP8 buffers; the cotangent goes back to the float producers."""
+
+    @staticmethod
+    def forward(ctx, q, kv, q_fp8, q_scale, kv_fp8, kv_scale, indices, sm_scale, d_v, sinks, output_dtype):
+        out = sparse_mla_fp8_path_c_apply(q_fp8, q_scale, kv_fp8, kv_scale, indices, sm_scale=sm_scale, d_v=d_v, sinks=sinks,
+                                          force_path_c=True, output_dtype=_float_dtype(q.dtype if output_dtype is None else output_dtype,
+                                                                                       name="output_dtype"))
+        ctx.save_for_backward(q_fp8, q_scale, kv_fp8, kv_scale, indices)
+        ctx.meta = (float(sm_scale), d_v, sinks is not None, q.dtype, kv.dtype)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q_fp8, q_scale, kv_fp8, kv_scale, indices = ctx.saved_tensors
+        sm_scale, d_v, has_sinks, q_dtype, kv_dtype = ctx.meta
+        if has_sinks:
+            raise RuntimeError("sparse_mla_fp8_path_c_apply_prepared_float: sinks backward is not implemented")
+        dq, dkv = sparse_mla_fp8_bwd_path_c(q_fp8, q_scale, kv_fp8, kv_scale, d_out, indices, sm_scale=sm_scale, d_v=d_v,
+                                            force_path_c=True)
+        return (dq.to(q_dtype), dkv.to(kv_dtype)) + (None,) * 9
+
+
+def sparse_mla_fp8_path_c_apply_prepared_float(
+    q: torch.Tensor,
+    kv: torch.Tensor,
+    q_fp8: torch.Tensor,
+    q_scale: torch.Tensor,
+    kv_fp8: torch.Tensor,
+    kv_scale: torch.Tensor,
+    indices: torch.Tensor,
+    *,
+    sm_scale: float,
+    d_v: int | None = None,
+    sinks: torch.Tensor | None = None,
+    force_path_c: bool = False,
+    causal: bool = False,
+    output_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    """Differentiable owner wrapper: the forward reads only the prepared ``q_fp8 / q_scale /
+    kv_fp8 / kv_scale``; the backward kernel's gradients (with respect to the dequantised values)
+    are handed to the float ``q`` / ``kv`` they were quantised from, in their dtypes.  There is no
+    float fallback here: without the library the call raises."""
+    del force_path_c, causal
+    status = sparse_mla_fp8_path_c_status()
+    if not status.available:
+        raise RuntimeError(f"sparse_mla_fp8_path_c_apply_prepared_float: Path C forward unavailable: {status.reason}")
+    return _PreparedFloatFunction.apply(q, kv, q_fp8, q_scale, kv_fp8, kv_scale, indices, sm_scale, d_v, sinks, output_dtype)
+
+
+def sparse_mla_fp8_path_c_apply_from_float(q, kv, indices, *, sm_scale, d_v=None, sinks=None, force_path_c=False):
+    """Fail-closed hook for float q / kv callers: the FP8 ABI is prepared-buffer only."""
+    del q, kv, indices, sm_scale, d_v, sinks, force_path_c
+    raise RuntimeError(
+        "sparse_mla_fp8_path_c_apply_from_float requires prepared FP8 buffers; use "
+        "sparse_mla_fp8_path_c_apply_prepared_float with existing q_fp8/q_scale/kv_fp8/kv_scale buffers instead of "
+        "materializing them inside the Path C wrapper")
 
 
 # invalid slots of the score-only kernels hold this finite sentinel

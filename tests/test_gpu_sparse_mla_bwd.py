@@ -164,3 +164,21 @@ def test_per_token_fp8_backward_over_prepared_buffers(device):
     assert err <= 1e-4 * ref
     with pytest.raises(ValueError):
         f8.sparse_mla_fp8_bwd_path_c(*args, to_dev(d_out, device)[..., :8].contiguous(), to_dev(idx, device), sm_scale=0.2, d_v=d_v)
+    # the differentiable owner wrapper: forward over the prepared buffers, gradients to the float producers
+    qf = to_dev(om.dequant_per_token(qc, qs).astype(np.float32), device).requires_grad_(True)
+    kf = to_dev(om.dequant_per_token(kc, ks).astype(np.float32), device).to(torch.bfloat16).requires_grad_(True)
+    out = f8.sparse_mla_fp8_path_c_apply_prepared_float(qf, kf, *args, to_dev(idx.astype(np.int32), device), sm_scale=0.2, d_v=d_v)
+    assert out.dtype == torch.float32 and tuple(out.shape) == (B, S, H, d_v)
+    (out * to_dev(d_out, device)).sum().backward()
+    torch.cuda.synchronize()
+    assert qf.grad.dtype == torch.float32 and kf.grad.dtype == torch.bfloat16
+    err, ref = error_report(qf.grad.cpu().numpy(), want_dq)
+    assert err <= 1e-4 * ref
+    err, ref = error_report(kf.grad.float().cpu().numpy(), want_dkv)
+    assert err <= 1e-2 * ref                                    # one rounding to bfloat16
+    with pytest.raises(RuntimeError, match="sinks backward"):
+        o2 = f8.sparse_mla_fp8_path_c_apply_prepared_float(qf, kf, *args, to_dev(idx.astype(np.int32), device), sm_scale=0.2, d_v=d_v,
+                                                           sinks=torch.zeros(H, device=device))
+        o2.sum().backward()
+    with pytest.raises(RuntimeError, match="requires prepared FP8 buffers"):
+        f8.sparse_mla_fp8_path_c_apply_from_float(qf, kf, to_dev(idx, device), sm_scale=0.2)
