@@ -458,7 +458,7 @@ def bench_next_rows(args, device):
         y = torch.empty((B, H, N), dtype=torch.bfloat16, device=device)
         hbm(tag, lambda x=x, w=w, y=y: ops.head_gemm(x, w, out=y), (x.numel() + w.numel() + y.numel()) * 2,
             f"head_gemm x bf16[{B},{H},{K}] . W bf16[{H},{N},{K}] -> bf16[{B},{H},{N}]")
-    # training side: float-carrier sparse-MLA backward (fp32 arithmetic; bound by the fp32 vector rate)
+    # training side: sparse-MLA backward on the matrix cores (bound by the float32 atomic adds into dkv)
     B, S, H, D, d_v, Skv, topk = 1, 1024, 16, 576, 512, 4096, 256
     q = torch.randn((B, S, H, D), generator=gen, device=device).to(torch.bfloat16)
     kv = torch.randn((B, Skv, 1, D), generator=gen, device=device).to(torch.bfloat16)
@@ -471,8 +471,24 @@ def bench_next_rows(args, device):
     res["sparse_mla_backward"] = {
         "workload": f"sparse_mla_bwd q bf16[{B},{S},{H},{D}] kv bf16[{B},{Skv},1,{D}] topk {topk} -> dq bf16, dkv f32 (atomic adds)",
         "us_per_launch": secs / steps * 1e6, "algorithmic_flops": flops,
-        "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 157.3, "unit": "TFLOP/s",
-                     "frac": flops / (secs / steps) / 1e12 / 157.3, "traffic": None}}
+        "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": flops / (secs / steps) / 1e12 / 2500.0, "traffic": None},
+        "float32_atomic_adds": B * S * topk * D, "atomic_add_floor_us": B * S * topk * D / (128 * 2.4e9) * 1e6}
+
+    # the same backward over per-token FP8 operands (e4m3 code values + float32 scale per token)
+    q8 = (torch.randn((B, S, H, D), generator=gen, device=device) * 64).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    kv8 = (torch.randn((B, Skv, 1, D), generator=gen, device=device) * 64).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    qs = torch.rand((B, S, H), generator=gen, device=device) * 0.02 + 0.005
+    kvs = torch.rand((B, Skv, 1), generator=gen, device=device) * 0.02 + 0.005
+    dq32 = torch.empty((B, S, H, D), dtype=torch.float32, device=device)
+    secs, _ = timed_graph([lambda: ops.sparse_mla_backward(q8, kv8, d_out, idx, sm_scale=D ** -0.5, d_v=d_v, dq=dq32, dkv=dkv,
+                                                           q_scale=qs, kv_scale=kvs)], steps, args.warmup)
+    res["sparse_mla_backward_fp8"] = {
+        "workload": f"sparse_mla_bwd q e4m3[{B},{S},{H},{D}] + f32 scale per token, kv e4m3[{B},{Skv},1,{D}] + f32 scale per token, "
+                    f"d_out bf16, topk {topk} -> dq f32, dkv f32 (atomic adds)",
+        "us_per_launch": secs / steps * 1e6, "algorithmic_flops": flops,
+        "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": flops / (secs / steps) / 1e12 / 2500.0, "traffic": None}}
 
     # DSA indexer KL loss (training side): one launch over every (batch, query position)
     ASq = Sk = 4096; AB, AH, AD, topk = 1, 8, 64, 1024
@@ -488,8 +504,8 @@ def bench_next_rows(args, device):
             "workload": f"dsa_indexer_loss query/key bf16[{ASq},{AB},{AH},{AD}] index_scores f32[{AB},{ASq},{Sk}]"
                         + (f" topk_indices i32[{AB},{ASq},{topk}]" if lst is not None else "") + " -> loss f32",
             "us_per_launch": secs / steps * 1e6, "algorithmic_flops": flops,
-            "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 157.3, "unit": "TFLOP/s",
-                         "frac": flops / (secs / steps) / 1e12 / 157.3, "traffic": None}}
+            "roofline": {"bound": "mfma", "achieved": flops / (secs / steps) / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
+                         "frac": flops / (secs / steps) / 1e12 / 2500.0, "traffic": None}}
     return res
 
 
@@ -541,6 +557,12 @@ PROFILE_WORKLOADS = [
     ("kv_cache_append", ("cache_append_kernel",),
      "bf16 latent[B,S,1,512] + rope[..,64] -> e4m3 + fp32/128 scales + bf16 rope in the cache: one dispatch of 8192 rows "
      "(prefill chunk) and one of 32 rows (decode step) per step"),
+    ("sparse_mla_backward", ("sparse_mla_bwd", "fill_zero_kernel"),
+     "sparse_mla_bwd q bf16[1,1024,16,576], kv bf16[1,4096,1,576], d_out bf16[1,1024,16,512], topk 256 -> dq bf16, dkv f32 "
+     "(the dkv clear, then the matrix-core kernel with its float32 atomic adds)"),
+    ("dsa_indexer_loss", ("dsa_indexer_loss",),
+     "dsa_indexer_loss query / key bf16[4096,1,8,64], index_scores f32[1,4096,4096]: one dense and one sparse "
+     "(topk_indices i32[1,4096,1024]) dispatch per step"),
     ("sparse_index_producers", ("_indices_",),
      "causal_sparse_indices(1,8192,1,2048) and sparse_indices_from_attention_mask(bool [8192,8192], topk 2048)"),
 ]

@@ -1,4 +1,5 @@
-// Sparse MLA backward on the matrix cores, bfloat16 operands (gfx950).
+// Sparse MLA backward on the matrix cores: bfloat16 operands, or e4m3 q / kv with per-token
+// scales (gfx950).
 //
 // Same gradients as sparse_mla_bwd.hip (the reference's sparse_mla_bwd_direct,
 // cppmega_mlx/nn/_tilelang/sparse_mla_path_c.py:2644-2816), organised so that the heads of a KV
@@ -27,6 +28,13 @@
 // gradients agree with fp32 arithmetic on the same bfloat16 inputs to ~1e-5 of their scale; the
 // extra matrix instructions are hidden behind the atomic adds.  The atomic adds per selected row
 // drop from one per head to one per chunk of heads.
+//
+// Per-token FP8 operands (the reference's fp8_sparse_mla_bwd_kernel,
+// cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:1966-2214): the e4m3 bytes of q and of the
+// gathered rows become bfloat16 (exactly) on their way into LDS, so the products run on the raw
+// code values; the scales q_scale[b,s,h] and kv_scale[b,t,g] multiply the scores and dP afterwards,
+// and are folded into dS before the second pair of products (dS * kv_scale for dQ, dS * q_scale
+// for dKV), so the gradients are with respect to the dequantised values, as in the reference.
 
 #include "common.h"
 #include "mfma_util.h"
@@ -39,8 +47,10 @@ constexpr int kMaxBlk = 9;            // 16-channel blocks per wavefront: d_qk <
 constexpr int kPad = 8;               // bfloat16 elements of padding per LDS row
 
 struct BwdMfmaParams {
-  const unsigned short* q;      // [B, S, H, D] bf16
-  const unsigned short* kv;     // [B, Skv, G, D] bf16
+  const void* q;                // [B, S, H, D] bf16, or e4m3 bytes
+  const void* kv;               // [B, Skv, G, D] bf16, or e4m3 bytes
+  const float* q_scale;         // [B, S, H] (e4m3 only)
+  const float* kv_scale;        // [B, Skv, G] (e4m3 only)
   const unsigned short* d_out;  // [B, S, H, d_v] bf16
   const void* indices;          // [B, S, G, topk]
   const float* sm_scale_dev;
@@ -68,11 +78,20 @@ __device__ __forceinline__ bf16x8 join(const bf16x4 a, const bf16x4 b) {
   r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
   return r;
 }
+// 8 e4m3 bytes -> 8 bfloat16, exact
+__device__ __forceinline__ uint4 e4m3x8_to_bf16(const uint2 v) {
+  uint4 r;
+  r.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, false));
+  r.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, true));
+  r.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, false));
+  r.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, true));
+  return r;
+}
 __device__ __forceinline__ bf16x8 zero8() {
   return __builtin_bit_cast(bf16x8, make_uint4(0u, 0u, 0u, 0u));
 }
 
-template <int HB>
+template <int HB, bool FP8>
 __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const BwdMfmaParams p) {
   constexpr int HC = 16 * HB;            // heads per workgroup
   constexpr int KT = 64 / HB;            // keys per tile
@@ -88,10 +107,13 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
   unsigned short* Ks = dOs + HC * Dvp;                              // [KT][Dp]
   constexpr int kPlane = HC * Kp;
   unsigned short* Ps = Ks + KT * Dp;                                // [hi, lo][HC][Kp]
-  unsigned short* dSs = Ps + 2 * kPlane;                            // [hi, lo][HC][Kp]
-  float* wstat = reinterpret_cast<float*>(dSs + 2 * kPlane);        // [4 waves][16 heads][3]
+  unsigned short* dSs = Ps + 2 * kPlane;                            // [hi, lo][HC][Kp]: dS (* kv_scale of the key)
+  unsigned short* dSq = FP8 ? dSs + 2 * kPlane : dSs;               // [hi, lo][HC][Kp]: dS * q_scale of the head
+  float* wstat = reinterpret_cast<float*>(dSq + 2 * kPlane);        // [4 waves][16 heads][3]
   float* stat = wstat + 4 * 16 * 3;                                 // [HC][3]: max, 1 / sum, delta
-  int* rows = reinterpret_cast<int*>(stat + HC * 3);                // [ntiles * KT]
+  float* qsc = stat + HC * 3;                                       // [HC] q scales (e4m3 only)
+  float* ksc = qsc + HC;                                            // [KT] kv scales of the tile (e4m3 only)
+  int* rows = reinterpret_cast<int*>(ksc + KT);                     // [ntiles * KT]
 
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kg = lane >> 4;
@@ -122,9 +144,14 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
     for (int piece = tid; piece < HC * dpr; piece += kThreads) {
       const int h = (int)(((float)piece + 0.5f) * inv_dpr), c8 = piece - h * dpr;
       uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (h < nh) v = *reinterpret_cast<const uint4*>(p.q + (bs * p.H + h0 + h) * (size_t)D + c8 * 8);
+      if (h < nh) {
+        const size_t at = (bs * p.H + h0 + h) * (size_t)D + c8 * 8;
+        if (FP8) v = e4m3x8_to_bf16(*reinterpret_cast<const uint2*>(static_cast<const unsigned char*>(p.q) + at));
+        else v = *reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(p.q) + at);
+      }
       *reinterpret_cast<uint4*>(Qs + h * Dp + c8 * 8) = v;
     }
+    if (FP8 && tid < HC) qsc[tid] = tid < nh ? p.q_scale[bs * p.H + h0 + tid] : 0.0f;
     for (int piece = tid; piece < HC * (dv / 8); piece += kThreads) {
       const int h = (int)(((float)piece + 0.5f) * inv_vpr), c8 = piece - h * (dv / 8);
       uint4 v = make_uint4(0u, 0u, 0u, 0u);
@@ -135,7 +162,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
   __syncthreads();
 
   // ---- tile staging: global -> registers one tile ahead -> LDS ----------------------------
-  uint4 pre[NP];
+  uint4 pre[NP];                                      // (e4m3: the 8 bytes of a piece in .x, .y and the row's scale in .z)
   int pre_off[NP];                                    // LDS element offset of each piece, -1 = none
   {
     const float inv_dpr = 1.0f / (float)dpr;
@@ -153,7 +180,17 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
       if (pre_off[i] >= 0) {
         const int r = pre_off[i] >> 16, c8 = pre_off[i] & 0xffff;
         const int row = rows[t * KT + r];
-        if (row >= 0) pre[i] = *reinterpret_cast<const uint4*>(p.kv + (((size_t)b * p.Skv + (size_t)row) * p.G + g) * (size_t)D + c8 * 8);
+        if (row >= 0) {
+          const size_t krow = ((size_t)b * p.Skv + (size_t)row) * p.G + g;
+          if (FP8) {
+            const uint2 v = *reinterpret_cast<const uint2*>(static_cast<const unsigned char*>(p.kv) + krow * (size_t)D + c8 * 8);
+            pre[i].x = v.x;
+            pre[i].y = v.y;
+            if (c8 == 0) pre[i].z = __float_as_uint(p.kv_scale[krow]);
+          } else {
+            pre[i] = *reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(p.kv) + krow * (size_t)D + c8 * 8);
+          }
+        }
       }
     }
   };
@@ -162,7 +199,12 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
     for (int i = 0; i < NP; ++i)
       if (pre_off[i] >= 0) {
         const int r = pre_off[i] >> 16, c8 = pre_off[i] & 0xffff;
-        *reinterpret_cast<uint4*>(Ks + r * Dp + c8 * 8) = pre[i];
+        if (FP8) {
+          *reinterpret_cast<uint4*>(Ks + r * Dp + c8 * 8) = e4m3x8_to_bf16(make_uint2(pre[i].x, pre[i].y));
+          if (c8 == 0) ksc[r] = __uint_as_float(pre[i].z);
+        } else {
+          *reinterpret_cast<uint4*>(Ks + r * Dp + c8 * 8) = pre[i];
+        }
       }
   };
 
@@ -181,6 +223,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
     }
     for (int kk = dv32; kk < d32; ++kk)
       s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_b128(a_base + kk * 32), lds_b128(q_base + kk * 32), s, 0, 0, 0);
+    if (FP8) {                                        // code-value products -> products of the dequantised values
+      const f32x4 kscale = *reinterpret_cast<const f32x4*>(ksc + 16 * ks + 4 * kg);
+      const float qscale = qsc[16 * hb + l16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        s[i] *= qscale * kscale[i];
+        dp[i] *= kscale[i];
+      }
+    }
   };
   // this lane's accumulator element i is (key 16 * ks + 4 * kg + i of the tile, head 16 * hb + l16)
 
@@ -267,16 +318,28 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
         ds[i] = pv[i] * (dp[i] - st_delta) * sm_scale;
       }
       const int off = (16 * hb + l16) * Kp + 16 * ks + 4 * kg;
-      float pl[4], dl[4];
+      auto planes = [&](unsigned short* base, const float (&v)[4]) {      // hi and lo bfloat16 planes of 4 values
+        float lo[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        pl[i] = pv[i] - (float)(__bf16)pv[i];
-        dl[i] = ds[i] - (float)(__bf16)ds[i];
+        for (int i = 0; i < 4; ++i) lo[i] = v[i] - (float)(__bf16)v[i];
+        *reinterpret_cast<uint2*>(base + off) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+        *reinterpret_cast<uint2*>(base + kPlane + off) = make_uint2(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]));
+      };
+      planes(Ps, pv);
+      if (FP8) {
+        const f32x4 kscale = *reinterpret_cast<const f32x4*>(ksc + 16 * ks + 4 * kg);
+        const float qscale = qsc[16 * hb + l16];
+        float dk[4], dq_[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          dk[i] = ds[i] * kscale[i];
+          dq_[i] = ds[i] * qscale;
+        }
+        planes(dSs, dk);
+        planes(dSq, dq_);
+      } else {
+        planes(dSs, ds);
       }
-      *reinterpret_cast<uint2*>(Ps + off) = make_uint2(pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]));
-      *reinterpret_cast<uint2*>(Ps + kPlane + off) = make_uint2(pack_bf16(pl[0], pl[1]), pack_bf16(pl[2], pl[3]));
-      *reinterpret_cast<uint2*>(dSs + off) = make_uint2(pack_bf16(ds[0], ds[1]), pack_bf16(ds[2], ds[3]));
-      *reinterpret_cast<uint2*>(dSs + kPlane + off) = make_uint2(pack_bf16(dl[0], dl[1]), pack_bf16(dl[2], dl[3]));
     }
     __syncthreads();
 
@@ -311,10 +374,10 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
       for (int pl = 0; pl < 2; ++pl) {
         if (HB == 2) {
           const int o = pl * kPlane + (8 * kg + tr_row) * Kp + kb * 16 + tr_col;
-          a_ds[pl] = join(lds_tr16(dSs + o), lds_tr16(dSs + o + 4 * Kp));
+          a_ds[pl] = join(lds_tr16(dSq + o), lds_tr16(dSq + o + 4 * Kp));
           a_p[pl] = join(lds_tr16(Ps + o), lds_tr16(Ps + o + 4 * Kp));
         } else {                                      // contraction slots 0..15: dS of the 16 heads, 16..31: P
-          const unsigned short* src = (kg < 2 ? dSs : Ps) + pl * kPlane + (8 * (kg & 1) + tr_row) * Kp + kb * 16 + tr_col;
+          const unsigned short* src = (kg < 2 ? dSq : Ps) + pl * kPlane + (8 * (kg & 1) + tr_row) * Kp + kb * 16 + tr_col;
           a_ds[pl] = join(lds_tr16(src), lds_tr16(src + 4 * Kp));
           a_p[pl] = a_ds[pl];
         }
@@ -381,31 +444,36 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
 }
 
 template <int HB>
-size_t lds_bytes(int D, int dv, int ntiles) {
+size_t lds_bytes(int D, int dv, int ntiles, bool fp8) {
   constexpr int HC = 16 * HB, KT = 64 / HB;
-  return (size_t)2 * (HC * (D + kPad) + HC * (dv + kPad) + KT * (D + kPad) + 4 * HC * (KT + kPad)) + (4 * 16 * 3 + HC * 3) * 4 + (size_t)ntiles * KT * 4;
+  return (size_t)2 * (HC * (D + kPad) + HC * (dv + kPad) + KT * (D + kPad) + (fp8 ? 6 : 4) * HC * (KT + kPad)) +
+         (4 * 16 * 3 + HC * 3 + HC + KT) * 4 + (size_t)ntiles * KT * 4;
+}
+
+bool fp8_operands(const cppmega_mi355_sparse_mla_bwd_args_t& a) {
+  return a.q_dtype == CPPMEGA_MI355_E4M3 && a.kv_dtype == CPPMEGA_MI355_E4M3 && a.q_scale && a.kv_scale;
 }
 
 }  // namespace
 
 // Whether the matrix-core kernel takes this problem (else the fp32 kernel runs).
 bool sparse_mla_bwd_mfma_supports(const cppmega_mi355_sparse_mla_bwd_args_t& a) {
-  if (a.q_dtype != CPPMEGA_MI355_BF16 || a.kv_dtype != CPPMEGA_MI355_BF16 || a.d_out_dtype != CPPMEGA_MI355_BF16) return false;
+  const bool bf16 = a.q_dtype == CPPMEGA_MI355_BF16 && a.kv_dtype == CPPMEGA_MI355_BF16;
+  if ((!bf16 && !fp8_operands(a)) || a.d_out_dtype != CPPMEGA_MI355_BF16) return false;
   if (a.d_qk % 32 != 0 || a.d_v % 32 != 0 || a.d_qk > kMaxBlk * 64 || a.topk < 1) return false;
   const int hg = a.heads / a.kv_groups;
   const int kt = hg > 16 ? 32 : 64;
   const int ntiles = (a.topk + kt - 1) / kt;
-  const size_t lds = hg > 16 ? lds_bytes<2>(a.d_qk, a.d_v, ntiles) : lds_bytes<1>(a.d_qk, a.d_v, ntiles);
+  const size_t lds = hg > 16 ? lds_bytes<2>(a.d_qk, a.d_v, ntiles, !bf16) : lds_bytes<1>(a.d_qk, a.d_v, ntiles, !bf16);
   return lds <= 160 * 1024;
 }
 
 int sparse_mla_bwd_mfma_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStream_t stream) {
   const int hg = a.heads / a.kv_groups;
-  const bool wide = hg > 16;
+  const bool wide = hg > 16, fp8 = fp8_operands(a);
   const int hc = wide ? 32 : 16, kt = wide ? 32 : 64;
   BwdMfmaParams p;
-  p.q = static_cast<const unsigned short*>(a.q);
-  p.kv = static_cast<const unsigned short*>(a.kv);
+  p.q = a.q; p.kv = a.kv; p.q_scale = a.q_scale; p.kv_scale = a.kv_scale;
   p.d_out = static_cast<const unsigned short*>(a.d_out);
   p.indices = a.indices; p.sm_scale_dev = a.sm_scale_dev; p.dq = a.dq; p.dkv = a.dkv;
   p.dq_dtype = a.dq_dtype; p.index_dtype = a.index_dtype;
@@ -416,15 +484,12 @@ int sparse_mla_bwd_mfma_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hip
   const size_t grid = (size_t)a.batch * a.seq_q * a.kv_groups * p.chunks;
   if (grid == 0) return 0;
   if (grid > 0x7fffffffull) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: too many (batch, query, head chunk) workgroups for one launch");
-  const size_t lds = wide ? lds_bytes<2>(a.d_qk, a.d_v, p.ntiles) : lds_bytes<1>(a.d_qk, a.d_v, p.ntiles);
-  if (wide) {
-    if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_bwd_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(sparse_mla_bwd_mfma_kernel<2>, dim3((unsigned)grid), dim3(kThreads), lds, stream, p);
-  } else {
-    if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute((const void*)sparse_mla_bwd_mfma_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(sparse_mla_bwd_mfma_kernel<1>, dim3((unsigned)grid), dim3(kThreads), lds, stream, p);
-  }
-  CM_HIP_CHECK(hipGetLastError());
+  const size_t lds = wide ? lds_bytes<2>(a.d_qk, a.d_v, p.ntiles, fp8) : lds_bytes<1>(a.d_qk, a.d_v, p.ntiles, fp8);
+  const void* fn = wide ? (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<2, true> : (const void*)sparse_mla_bwd_mfma_kernel<2, false>)
+                        : (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<1, true> : (const void*)sparse_mla_bwd_mfma_kernel<1, false>);
+  if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  void* kargs[] = {(void*)&p};
+  CM_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(kThreads), kargs, lds, stream));
   return 0;
 }
 

@@ -101,6 +101,40 @@ def test_bfloat16_backward_on_the_matrix_cores(device, shape, index_dtype):
     assert torch.equal(dq16, dq.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("shape", [
+    dict(B=2, S=3, H=8, G=2, Skv=120, topk=70, D=64, d_v=32),
+    dict(B=1, S=2, H=48, G=1, Skv=300, topk=45, D=576, d_v=512),
+    dict(B=1, S=3, H=16, G=1, Skv=200, topk=130, D=128, d_v=128),
+], ids=lambda c: "B%dS%dH%dG%dT%dk%dD%ddv%d" % tuple(c.values()))
+def test_per_token_fp8_backward_on_the_matrix_cores(device, shape):
+    """e4m3 q / kv with per-token scales and a bfloat16 cotangent take the matrix-core kernel: the code
+    values are exact in bfloat16 and the scales are applied in fp32, so the 1e-4 bar of the fp32 kernel holds."""
+    from cppmega_mlx_amd.nn._tilelang import sparse_mla_fp8_path_c as f8
+    from oracle import fp8
+
+    B, S, H, G, Skv, topk, D, d_v = shape.values()
+    rng = np.random.default_rng(H * 100 + topk)
+    qc, qs = fp8.quantize_per_token((rng.standard_normal((B * S * H, D)) * rng.uniform(0.2, 3.0, (B * S * H, 1))).astype(np.float32))
+    kc, ks = fp8.quantize_per_token((rng.standard_normal((B * Skv * G, D)) * rng.uniform(0.2, 3.0, (B * Skv * G, 1))).astype(np.float32))
+    qc, qs, kc, ks = qc.reshape(B, S, H, D), qs.reshape(B, S, H), kc.reshape(B, Skv, G, D), ks.reshape(B, Skv, G)
+    d_out = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(torch.bfloat16)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[rng.random(idx.shape) < 0.15] = -1
+    idx[0, 1] = -1
+    idx[0, 0, 0, :2] = Skv + 1
+    sm = 0.9 * D ** -0.5
+    want_dq, want_dkv = om.sparse_mla_bwd_oracle(om.dequant_per_token(qc, qs), om.dequant_per_token(kc, ks), idx,
+                                                 d_out.double().cpu().numpy(), sm_scale=sm, d_v=d_v)
+    dq, dkv = f8.sparse_mla_fp8_bwd_path_c(to_dev(qc, device), to_dev(qs, device), to_dev(kc, device), to_dev(ks, device), d_out,
+                                           to_dev(idx.astype(np.int32), device), sm_scale=sm, d_v=d_v)
+    torch.cuda.synchronize()
+    for got, want in ((dq, want_dq), (dkv, want_dkv)):
+        assert got.dtype == torch.float32
+        err, ref = error_report(got.cpu().numpy(), want)
+        assert err <= 1e-4 * ref, (err, ref)
+    assert (dq[0, 1] == 0).all()
+
+
 def test_public_backward_entry_points_and_autograd(device):
     rng = np.random.default_rng(8)
     B, S, H, G, Skv, topk, D = 2, 4, 4, 2, 48, 12, 64
