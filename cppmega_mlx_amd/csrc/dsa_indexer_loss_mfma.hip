@@ -8,9 +8,11 @@
 //   are cut into tiles of 32 and dealt to the wavefronts round robin, so a workgroup's keys are
 //   read once per pass and the wavefronts never wait for each other inside a pass;
 //   S^T[key, query] = K_h[key, :] . Q_h[query, :]^T per head h: the key rows are the A operand and
-//   the query rows the B operand, both fetched from memory in operand order (16-byte loads, the
-//   next head's while the current one is reduced); a lane then holds 4 consecutive keys of one
-//   query per 16-key block, which is also how it reads the index scores (one 16-byte load).
+//   the query rows the B operand; the key fragments are fetched from memory in operand order
+//   (16-byte loads, the next head's while the current one is reduced), the 16 query rows sit in
+//   LDS when all their heads fit there (else they are fetched like the keys); a lane then holds
+//   4 consecutive keys of one query per 16-key block, which is also how it reads the index
+//   scores.
 //
 //   prologue  membership bits of the 16 index lists in LDS (sparse loss); max and sum of the index
 //             softmax of each row over all keys;
@@ -54,15 +56,19 @@ __device__ __forceinline__ f32x4 mfma16(const uint4 a, const uint4 b, const f32x
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-template <bool F16, int KSTEPS>
+constexpr int kQPad = 8;              // bfloat16 elements of padding per query row in LDS
+
+template <bool F16, int KSTEPS, bool Q_LDS>
 __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const LossMfmaParams p) {
   extern __shared__ __align__(16) float lds[];
   float* wstat = lds;                                     // [kWaves][AH][16][2]: running max, sum
   float* stat = wstat + kWaves * p.AH * 32;               // [AH][16][2]: max, 1 / sum
   float* idxstat = stat + p.AH * 32;                      // [16][2]: max, 1 / sum of the index softmax
   float* klred = idxstat + 32;                            // [kWaves][16]
-  unsigned* bits = reinterpret_cast<unsigned*>(klred + kWaves * 16);   // [16][words]
+  unsigned* bits = reinterpret_cast<unsigned*>(klred + kWaves * 16);   // [16][words] (sparse loss only)
   const int words = (p.Sk + 31) / 32;
+  const int qpitch = p.AH * p.AD + kQPad;                 // elements per query row in LDS
+  unsigned short* qs = reinterpret_cast<unsigned short*>(bits + (p.topk_idx ? kRows * ((words + 3) & ~3) : 0));   // [16][qpitch]
 
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kg = lane >> 4;
@@ -113,6 +119,16 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
       idxstat[r * 2 + 1] = 1.0f / (dsum > 0.0f ? dsum : 1.0f);
     }
   }
+  if (Q_LDS) {
+    const int per_row = p.AH * p.AD / 8;                  // 16-byte pieces of one position's heads
+    for (int piece = tid; piece < kRows * per_row; piece += kThreads) {
+      const int r = piece / per_row, c8 = piece - r * per_row;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (sq0 + r < p.ASq)
+        v = *reinterpret_cast<const uint4*>(p.q + ((size_t)(sq0 + r) * p.AB + b) * (size_t)p.AH * p.AD + c8 * 8);
+      *reinterpret_cast<uint4*>(qs + r * qpitch + c8 * 8) = v;
+    }
+  }
   for (int e = lane; e < p.AH * 16; e += 64) {
     wstat[(wave * p.AH * 16 + e) * 2] = -INFINITY;
     wstat[(wave * p.AH * 16 + e) * 2 + 1] = 0.0f;
@@ -124,7 +140,8 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
   const unsigned short* q_lane = p.q + (size_t)(my_row ? my_sq : 0) * pos_stride + (size_t)b * p.AH * p.AD + 8 * kg;
 
   // operand fragments of one (tile, head): two 16-key blocks of K and the query block
-  struct Frag { uint4 ka[2][KSTEPS]; uint4 qb[KSTEPS]; };
+  struct Frag { uint4 ka[2][KSTEPS]; uint4 qb[Q_LDS ? 1 : KSTEPS]; };
+  const unsigned short* q_lds = qs + l16 * qpitch + 8 * kg;
   auto load_frag = [&](Frag& f, int key0, int h) {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
@@ -133,16 +150,22 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
 #pragma unroll
       for (int kk = 0; kk < KSTEPS; ++kk) f.ka[sub][kk] = *reinterpret_cast<const uint4*>(src + 32 * kk);
     }
+    if (!Q_LDS) {
 #pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) f.qb[kk] = *reinterpret_cast<const uint4*>(q_lane + (size_t)h * head_stride + 32 * kk);
+      for (int kk = 0; kk < KSTEPS; ++kk) f.qb[kk] = *reinterpret_cast<const uint4*>(q_lane + (size_t)h * head_stride + 32 * kk);
+    }
   };
   // scores of this lane: s[sub][i] = key key0 + 16 * sub + 4 * kg + i against query my_sq
-  auto scores = [&](const Frag& f, float (&s)[2][4]) {
+  auto scores = [&](const Frag& f, int h, float (&s)[2][4]) {
+    uint4 qb[KSTEPS];
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk)
+      qb[kk] = Q_LDS ? *reinterpret_cast<const uint4*>(q_lds + h * p.AD + 32 * kk) : f.qb[kk];
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < KSTEPS; ++kk) acc = mfma16<F16>(f.ka[sub][kk], f.qb[kk], acc);
+      for (int kk = 0; kk < KSTEPS; ++kk) acc = mfma16<F16>(f.ka[sub][kk], qb[kk], acc);
 #pragma unroll
       for (int i = 0; i < 4; ++i) s[sub][i] = acc[i] * p.scale;
     }
@@ -178,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
     for (int h = 0; h < p.AH; ++h) {
       if (h + 1 < p.AH) load_frag(nxt, key0, h + 1);
       float s[2][4];
-      scores(cur, s);
+      scores(cur, h, s);
       float tmax = -INFINITY;
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub)
@@ -242,7 +265,7 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
     for (int h = 0; h < p.AH; ++h) {
       if (h + 1 < p.AH) load_frag(nxt, key0, h + 1);
       float s[2][4];
-      scores(cur, s);
+      scores(cur, h, s);
       const float mh = stat[(h * 16 + l16) * 2], invd = stat[(h * 16 + l16) * 2 + 1];
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub)
@@ -280,16 +303,17 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
   }
 }
 
-size_t lds_bytes(int AH, int Sk, bool sparse) {
-  return ((size_t)kWaves * AH * 32 + (size_t)AH * 32 + 32 + kWaves * 16) * 4 + (sparse ? (size_t)kRows * ((Sk + 31) / 32) * 4 : 0);
+size_t lds_base_bytes(int AH, int Sk, bool sparse) {
+  return ((size_t)kWaves * AH * 32 + (size_t)AH * 32 + 32 + kWaves * 16) * 4 + (sparse ? (size_t)kRows * ((((Sk + 31) / 32) + 3) & ~3) * 4 : 0);
 }
+size_t q_lds_bytes(int AH, int AD) { return (size_t)kRows * (AH * AD + kQPad) * 2; }
 
 }  // namespace
 
 bool dsa_indexer_loss_mfma_supports(const cppmega_mi355_dsa_loss_args_t& a) {
   if (a.in_dtype != CPPMEGA_MI355_BF16 && a.in_dtype != CPPMEGA_MI355_F16) return false;
   if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 96 && a.head_dim != 128) return false;
-  return lds_bytes(a.heads, a.seq_k, a.topk_indices != nullptr) <= 160 * 1024;
+  return lds_base_bytes(a.heads, a.seq_k, a.topk_indices != nullptr) <= 160 * 1024;
 }
 
 int dsa_indexer_loss_mfma_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStream_t stream) {
@@ -303,15 +327,19 @@ int dsa_indexer_loss_mfma_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStre
   p.scale = a.softmax_scale;
   const size_t grid = (size_t)p.nblocks * a.batch;
   if (grid > 0x7fffffffull) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "dsa_indexer_loss: too many rows for one launch");
-  const size_t lds = lds_bytes(a.heads, a.seq_k, a.topk_indices != nullptr);
+  size_t lds = lds_base_bytes(a.heads, a.seq_k, a.topk_indices != nullptr);
+  const bool q_lds = lds + q_lds_bytes(a.heads, a.head_dim) <= 64 * 1024;      // the query rows too, while two workgroups still fit a CU
+  if (q_lds) lds += q_lds_bytes(a.heads, a.head_dim);
   const bool f16 = a.in_dtype == CPPMEGA_MI355_F16;
   const void* fn = nullptr;
-#define CM_PICK(F, KS) fn = (const void*)dsa_indexer_loss_mfma_kernel<F, KS>
+#define CM_PICK(KS)                                                                                                   \
+  fn = f16 ? (q_lds ? (const void*)dsa_indexer_loss_mfma_kernel<true, KS, true> : (const void*)dsa_indexer_loss_mfma_kernel<true, KS, false>) \
+           : (q_lds ? (const void*)dsa_indexer_loss_mfma_kernel<false, KS, true> : (const void*)dsa_indexer_loss_mfma_kernel<false, KS, false>)
   switch (a.head_dim / 32) {
-    case 1: if (f16) CM_PICK(true, 1); else CM_PICK(false, 1); break;
-    case 2: if (f16) CM_PICK(true, 2); else CM_PICK(false, 2); break;
-    case 3: if (f16) CM_PICK(true, 3); else CM_PICK(false, 3); break;
-    default: if (f16) CM_PICK(true, 4); else CM_PICK(false, 4); break;
+    case 1: CM_PICK(1); break;
+    case 2: CM_PICK(2); break;
+    case 3: CM_PICK(3); break;
+    default: CM_PICK(4); break;
   }
 #undef CM_PICK
   if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
