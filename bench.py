@@ -542,10 +542,10 @@ PROFILE_WORKLOADS = [
     ("fp8_vecmat_e4m3_activation", ("gemv_stream_kernel<1, 4, 4, 1>",),
      "W e4m3[7168,16384] + fp32 scale per row, x e4m3[16384] + fp32 scale -> f32[7168] (the reference's own vecmat form)"),
     ("fp8_vecmat_m4", ("gemv_stream_kernel<4",), "W e4m3[7168,16384] + fp32 scale/128, x bf16[4,16384]"),
-    ("fp8_vecmat_m16", ("skinny_mfma_kernel<1>", "skinny_reduce"),
-     "W e4m3[7168,16384] + fp32 scale/128, x bf16[16,16384] (the reduce kernel row averages the M = 16 and M = 32 calls of the run)"),
+    ("fp8_vecmat_m16", ("skinny_rows_kernel<1>",),
+     "W e4m3[7168,16384] + fp32 scale/128, x bf16[16,16384] (one kernel, no K split, no workspace)"),
     ("fp8_vecmat_m32", ("skinny_mfma_kernel<2>", "skinny_reduce"),
-     "W e4m3[7168,16384] + fp32 scale/128, x bf16[32,16384] (the reduce kernel row averages the M = 16 and M = 32 calls of the run)"),
+     "W e4m3[7168,16384] + fp32 scale/128, x bf16[32,16384] (split-K kernel + reduce kernel)"),
     ("topk_selector", ("topk_tile_kernel<float, 16, 4, 512, 0>",), "scores fp32[4096 rows,8192] -> int32[4096,2048]"),
     ("topk_selector_decode_shape", ("topk_tile_kernel<float, 16, 4, 512, 1>", "topk_tile_kernel<float, 16, 4, 1024, 2>", "topk_wide_kernel"),
      "scores fp32[32,65536] -> int32[32,2048]: the two-stage path (segment kernel, then candidate kernel) and, for "

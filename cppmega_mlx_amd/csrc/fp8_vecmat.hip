@@ -601,6 +601,186 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
   }
 }
 
+// ---------------------------------------------------------------------------
+// 5 <= M <= 32 without a K split: a workgroup owns up to 32 weight rows for the whole K.
+//
+// Each of its 8 wavefronts takes a contiguous eighth of the 128-channel blocks, so a weight row
+// is streamed as 8 sequential runs.  Per block a wavefront fetches the 32 x 128 weight bytes and
+// the 16 MT x 128 bfloat16 activations with loads in which neighbouring lanes ask for
+// neighbouring 16-byte pieces (8 lanes = one 128-byte weight line, 16 lanes = 256 bytes of an
+// activation row: loads whose lanes all point into different lines move a quarter of the bytes
+// per clock), a few blocks ahead, in registers; the block then passes through a private LDS
+// tile, written in load order and read in matrix-operand order (16-byte slots XOR-swizzled by
+// the row so both directions are free of bank conflicts).  The weight bytes become bfloat16 in
+// registers (v_cvt_scalef32_pk_bf16_fp8, exact) and four v_mfma_f32_16x16x32_bf16 per (row tile,
+// activation tile) multiply them with the activations as they are: no activation planes, no
+// operand exponents, products exact.  A block's tile starts from zero and is added as
+// acc += scale * tile, so any fp32 block scale is applied exactly; the scales of the workgroup's
+// rows are staged in LDS once.  The activations (M x K bf16, 512 KB at M = 16) are re-read by
+// every workgroup out of the L2.  The 8 partial tiles meet in LDS in wavefront order
+// (deterministic); there is no workspace and no second kernel.
+// ---------------------------------------------------------------------------
+constexpr int kRowsMax = 32;              // weight rows per workgroup (two MFMA row tiles)
+__host__ __device__ constexpr int rows_waves(int) { return 8; }
+
+template <int MT>
+__global__ __launch_bounds__(rows_waves(MT) * 64) void skinny_rows_kernel(const VecmatParams p) {
+  constexpr int kRowsWaves = rows_waves(MT);
+  constexpr int DEPTH = MT == 1 ? 3 : 2;               // blocks in flight per wavefront (registers)
+  constexpr int kWTile = 32 * 128;                     // bytes: 32 rows x 8 slots of 16
+  constexpr int kXTile = 16 * 256;                     // bytes: 16 rows x 16 slots of 16
+  constexpr int kWaveBytes = kWTile + MT * kXTile;            // tiles of one wavefront
+  extern __shared__ __align__(16) unsigned char lds_b[];
+  const int KB = p.k / 128;
+  unsigned char* stage = lds_b + (size_t)(threadIdx.x >> 6) * kWaveBytes;            // this wavefront's tiles
+  float* sc = reinterpret_cast<float*>(lds_b + (size_t)kRowsWaves * kWaveBytes);      // [KB][32] block scales of the rows
+  float* red = reinterpret_cast<float*>(lds_b);                                       // [waves][32][16 MT], reuses the tiles
+  const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int n0 = (int)blockIdx.x * p.rows_per_wg;
+  const int rows_here = min(p.rows_per_wg, p.n - n0);
+
+  const int per_wave = (KB + kRowsWaves - 1) / kRowsWaves;
+  const int kb_begin = wave * per_wave, kb_end = min(KB, kb_begin + per_wave);
+  // Workgroups start at different places of their runs, so that at any time they ask for different
+  // activation lines and different memory channels (every workgroup's rows begin at the same
+  // channel alignment).  The order in which a row's blocks are added depends on the workgroup only.
+  const int nblk = max(kb_end - kb_begin, 0);
+  const int rot = nblk > 0 ? (int)((blockIdx.x * 5u) % (unsigned)nblk) : 0;
+  auto block_at = [&](int i) { const int j = i + rot; return kb_begin + (j >= nblk ? j - nblk : j); };
+  // the block scales of this wavefront's run (32 rows x nblk): written and read by this wavefront only
+  for (int e = lane; e < 32 * nblk; e += 64) {
+    const int r = e & 31, kb = kb_begin + (e >> 5);
+    sc[kb * 32 + r] = r < rows_here ? wscale(p, n0 + r, kb) : 0.0f;
+  }
+
+  // load order: position = lane + 64 j holds (row, slot); the piece fetched into a slot is slot ^ swizzle(row)
+  const unsigned char* wsrc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int pos = lane + 64 * j, row = pos >> 3, slot = pos & 7;
+    wsrc[j] = p.w + (size_t)(n0 + min(row, rows_here - 1)) * p.k + 16 * (slot ^ ((row >> 1) & 7));
+  }
+  const unsigned char* xsrc[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int pos = lane + 64 * j, row = pos >> 4, slot = pos & 15;
+      xsrc[mt][j] = (const unsigned char*)p.x + ((size_t)min(16 * mt + row, p.m - 1) * p.k) * 2 + 16 * (slot ^ row);
+    }
+  // operand order: lane (r16, kg)
+  int a_off[2][2], b_off[MT][4];                       // byte offsets inside a tile set
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int row = 16 * rt + r16;
+      a_off[rt][h] = row * 128 + 16 * ((2 * kg + h) ^ ((row >> 1) & 7));
+    }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) b_off[mt][s4] = kWTile + mt * kXTile + r16 * 256 + 16 * ((4 * kg + s4) ^ r16);
+
+  typedef __attribute__((ext_vector_type(4))) unsigned u4;
+  u4 wq[DEPTH][4];
+  u4 xq[DEPTH][MT][4];
+  auto fetch = [&](int slot, int kb) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wq[slot][j] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(wsrc[j] + (size_t)kb * 128));
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xq[slot][mt][j] = *reinterpret_cast<const u4*>(xsrc[mt][j] + (size_t)kb * 256);
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (d < nblk) fetch(d, block_at(d));
+
+  f32x4 acc[2][MT];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // registers -> the wavefront's LDS tiles, in load order
+  auto to_lds = [&](int slot) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u4*>(stage + (lane + 64 * j) * 16) = wq[slot][j];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *reinterpret_cast<u4*>(stage + kWTile + mt * kXTile + (lane + 64 * j) * 16) = xq[slot][mt][j];
+  };
+  for (int i0 = 0; i0 < nblk; i0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int i = i0 + d;
+      if (i < nblk) {                                  // (uniform)
+        const int kb = block_at(i);
+        to_lds(d);
+        if (i + DEPTH < nblk) fetch(d, block_at(i + DEPTH));            // refill the slot just emptied
+        const unsigned char* src = stage;
+        uint4 xb[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) xb[mt][s4] = *reinterpret_cast<const uint4*>(src + b_off[mt][s4]);
+        f32x4 tile[2][MT];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+          const uint4 w0 = *reinterpret_cast<const uint4*>(src + a_off[rt][0]);
+          const uint4 w1 = *reinterpret_cast<const uint4*>(src + a_off[rt][1]);
+          const unsigned wd[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) tile[rt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) {             // MFMA step s4: channels 32 kg + 8 s4 .. + 7 of the block
+            uint4 a;
+            a.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4], 1.0f, false));
+            a.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4], 1.0f, true));
+            a.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4 + 1], 1.0f, false));
+            a.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4 + 1], 1.0f, true));
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              tile[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, xb[mt][s4]),
+                                                                     tile[rt][mt], 0, 0, 0);
+          }
+        }
+        // tile element i: weight row 16 rt + 4 kg + i, activation row 16 mt + r16
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+          const f32x4 s4v = *reinterpret_cast<const f32x4*>(sc + kb * 32 + 16 * rt + 4 * kg);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[rt][mt][e] = fmaf(s4v[e], tile[rt][mt][e], acc[rt][mt][e]);
+        }
+      }
+    }
+  }
+
+  // partial tiles of the 8 wavefronts -> LDS (over the staging tiles) -> sums in wavefront order
+  __syncthreads();
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[(wave * 32 + 16 * rt + 4 * kg + i) * (16 * MT) + 16 * mt + r16] = acc[rt][mt][i];
+  __syncthreads();
+  for (int e = tid; e < 16 * MT * 32; e += kRowsWaves * 64) {
+    const int m = e >> 5, r = e & 31;                  // consecutive threads: consecutive output columns
+    if (m < p.m && r < rows_here) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kRowsWaves; ++w) sum += red[(w * 32 + r) * (16 * MT) + m];
+      store_as(p.out, (size_t)m * p.n + n0 + r, p.out_dtype, sum);
+    }
+  }
+}
+
 // out[m][n] = sum over the K splits of partial[split][m][n], in split order
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const VecmatParams p) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -672,17 +852,24 @@ static bool stream_k(const cppmega_mi355_vecmat_args_t& a) {
 static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) { return stream_k(a) && a.m <= stream_row_cap(a.x_dtype); }
 // the split-K MFMA kernel: bf16 activations, M >= 5 (in passes of 32 rows), K in eighths of whole scale blocks that fit the LDS slice
 constexpr int kSkinnyMaxRows = 32;
+constexpr int kRowsMaxM = 16;             // activation rows the kernel without a K split takes (measured: faster up to here)
 static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
   return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 &&
          (a.k % (kSkinnySplits * 128) == 0) && a.k / kSkinnySplits <= kSkinnyMaxKw;
 }
 static bool skinny_ok(const cppmega_mi355_vecmat_args_t& a) { return vecmat_aligned(a) && skinny_shape(a); }
+// the kernel without a K split: bf16 activations, M >= 5 (in passes of 32 rows), whole 128-channel blocks,
+// scales of 32 rows and partial tiles within the LDS
+static size_t rows_lds_bytes(int k, int mt) { return (size_t)rows_waves(mt) * (32 * 128 + mt * 16 * 256) + (size_t)(k / 128) * 32 * sizeof(float); }
+static bool rows_shape(const cppmega_mi355_vecmat_args_t& a) {
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 && a.m <= kRowsMaxM && a.k % 128 == 0 && rows_lds_bytes(a.k, 1) <= 160 * 1024;
+}
 
 int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes) {
   if (!bytes) return fail(CPPMEGA_MI355_ERR_NULL, "vecmat: bytes is NULL");
   // pointers may be absent in a sizing call: decided from the shape alone (a misaligned call then
   // simply does not use the workspace)
-  *bytes = skinny_shape(a) ? (size_t)kSkinnySplits * (a.m < kSkinnyMaxRows ? a.m : kSkinnyMaxRows) * a.n * sizeof(float) : 0;
+  *bytes = (skinny_shape(a) && !rows_shape(a)) ? (size_t)kSkinnySplits * (a.m < kSkinnyMaxRows ? a.m : kSkinnyMaxRows) * a.n * sizeof(float) : 0;
   return 0;
 }
 
@@ -798,6 +985,17 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
   if (aligned && stream_shape(a)) {
     rc = stream_pass(p, 0, a.m);
     if (rc) return rc;
+  } else if (aligned && rows_shape(a)) {
+    // about one workgroup per CU, whole MFMA row tiles where that is possible
+    int rows = (a.n + device_cus() - 1) / device_cus();
+    rows = rows < 16 ? 16 : (rows > kRowsMax ? kRowsMax : rows);
+    p.rows_per_wg = rows;
+    const dim3 grid((unsigned)((a.n + rows - 1) / rows));
+    const size_t smem = rows_lds_bytes(a.k, 1);
+    const void* fn = (const void*)skinny_rows_kernel<1>;
+    if (smem > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    void* kargs[] = {(void*)&p};
+    CM_HIP_CHECK(hipLaunchKernel(fn, grid, dim3(rows_waves(1) * 64), kargs, smem, stream));
   } else if (skinny_ok(a)) {
     // more than 32 activation rows: passes of 32 over the same workspace (stream order keeps them apart)
     const int cap = a.m < kSkinnyMaxRows ? a.m : kSkinnyMaxRows;
