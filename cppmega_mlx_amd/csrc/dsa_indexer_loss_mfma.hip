@@ -51,14 +51,18 @@ struct LossMfmaParams {
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 
 template <bool F16>
-__device__ __forceinline__ f32x4 mfma16(const uint4 a, const uint4 b, const f32x4 c) {
+__device__ __forceinline__ f32x4 mfma16(const __attribute__((ext_vector_type(4))) unsigned a, const __attribute__((ext_vector_type(4))) unsigned b, const f32x4 c) {
   if (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
 constexpr int kQPad = 8;              // bfloat16 elements of padding per query row in LDS
 
-template <bool F16, int KSTEPS, bool Q_LDS>
+// K_LDS (head sizes 64 and 128): the 32 key rows of a step are fetched with neighbouring lanes on
+// neighbouring 16-byte pieces of a row (loads whose lanes each point into another row move a quarter
+// of the bytes per clock) and reach operand order through a private LDS tile whose 16-byte slots are
+// XOR-swizzled by the row.
+template <bool F16, int KSTEPS, bool Q_LDS, bool K_LDS>
 __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const LossMfmaParams p) {
   extern __shared__ __align__(16) float lds[];
   float* wstat = lds;                                     // [kWaves][AH][16][2]: running max, sum
@@ -69,6 +73,9 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
   const int words = (p.Sk + 31) / 32;
   const int qpitch = p.AH * p.AD + kQPad;                 // elements per query row in LDS
   unsigned short* qs = reinterpret_cast<unsigned short*>(bits + (p.topk_idx ? kRows * ((words + 3) & ~3) : 0));   // [16][qpitch]
+  constexpr int PPR = 4 * KSTEPS;                         // 16-byte pieces per key row of one head
+  constexpr int RP = PPR >= 16 ? 1 : 16 / PPR;            // rows per 256 bytes
+  unsigned char* kstage = reinterpret_cast<unsigned char*>(qs + (Q_LDS ? kRows * qpitch : 0)) + (threadIdx.x >> 6) * (32 * PPR * 16);
 
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kg = lane >> 4;
@@ -140,32 +147,56 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
   const unsigned short* q_lane = p.q + (size_t)(my_row ? my_sq : 0) * pos_stride + (size_t)b * p.AH * p.AD + 8 * kg;
 
   // operand fragments of one (tile, head): two 16-key blocks of K and the query block
-  struct Frag { uint4 ka[2][KSTEPS]; uint4 qb[Q_LDS ? 1 : KSTEPS]; };
+  typedef __attribute__((ext_vector_type(4))) unsigned u4;
+  struct Frag { u4 ka[2 * KSTEPS]; u4 qb[Q_LDS ? 1 : KSTEPS]; };   // ka: [sub][step] in operand order, or the pieces in load order (K_LDS)
   const unsigned short* q_lds = qs + l16 * qpitch + 8 * kg;
   auto load_frag = [&](Frag& f, int key0, int h) {
+    if (K_LDS) {
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      const int key = key0 + 16 * sub + l16;
-      const unsigned short* src = p.k + (size_t)min(key, p.Sk - 1) * pos_stride + ((size_t)b * p.AH + h) * head_stride + 8 * kg;
+      for (int t = 0; t < 2 * KSTEPS; ++t) {
+        const int P = lane + 64 * t, row = P / PPR, c = P % PPR;
+        f.ka[t] = *reinterpret_cast<const u4*>(
+            p.k + (size_t)min(key0 + row, p.Sk - 1) * pos_stride + ((size_t)b * p.AH + h) * head_stride + 8 * c);
+      }
+    } else {
 #pragma unroll
-      for (int kk = 0; kk < KSTEPS; ++kk) f.ka[sub][kk] = *reinterpret_cast<const uint4*>(src + 32 * kk);
+      for (int sub = 0; sub < 2; ++sub) {
+        const int key = key0 + 16 * sub + l16;
+        const unsigned short* src = p.k + (size_t)min(key, p.Sk - 1) * pos_stride + ((size_t)b * p.AH + h) * head_stride + 8 * kg;
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; ++kk) f.ka[sub * KSTEPS + kk] = *reinterpret_cast<const u4*>(src + 32 * kk);
+      }
     }
     if (!Q_LDS) {
 #pragma unroll
-      for (int kk = 0; kk < KSTEPS; ++kk) f.qb[kk] = *reinterpret_cast<const uint4*>(q_lane + (size_t)h * head_stride + 32 * kk);
+      for (int kk = 0; kk < KSTEPS; ++kk) f.qb[kk] = *reinterpret_cast<const u4*>(q_lane + (size_t)h * head_stride + 32 * kk);
     }
   };
   // scores of this lane: s[sub][i] = key key0 + 16 * sub + 4 * kg + i against query my_sq
   auto scores = [&](const Frag& f, int h, float (&s)[2][4]) {
-    uint4 qb[KSTEPS];
+    u4 qb[KSTEPS];
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk)
-      qb[kk] = Q_LDS ? *reinterpret_cast<const uint4*>(q_lds + h * p.AD + 32 * kk) : f.qb[kk];
+      qb[kk] = Q_LDS ? *reinterpret_cast<const u4*>(q_lds + h * p.AD + 32 * kk) : f.qb[Q_LDS ? 0 : kk];
+    if (K_LDS) {                                          // load order -> the wavefront's LDS tile
+#pragma unroll
+      for (int t = 0; t < 2 * KSTEPS; ++t) {
+        const int P = lane + 64 * t, row = P / PPR, c = P % PPR;
+        *reinterpret_cast<u4*>(kstage + (row * PPR + (c ^ ((row / RP) % PPR))) * 16) = f.ka[t];
+      }
+    }
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < KSTEPS; ++kk) acc = mfma16<F16>(f.ka[sub][kk], qb[kk], acc);
+      for (int kk = 0; kk < KSTEPS; ++kk) {
+        u4 ka = f.ka[sub * KSTEPS + kk];
+        if (K_LDS) {
+          const int row = 16 * sub + l16, c = 4 * kk + kg;
+          ka = *reinterpret_cast<const u4*>(kstage + (row * PPR + (c ^ ((row / RP) % PPR))) * 16);
+        }
+        acc = mfma16<F16>(ka, qb[kk], acc);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) s[sub][i] = acc[i] * p.scale;
     }
@@ -330,18 +361,21 @@ int dsa_indexer_loss_mfma_launch(const cppmega_mi355_dsa_loss_args_t& a, hipStre
   size_t lds = lds_base_bytes(a.heads, a.seq_k, a.topk_indices != nullptr);
   const bool q_lds = lds + q_lds_bytes(a.heads, a.head_dim) <= 64 * 1024;      // the query rows too, while two workgroups still fit a CU
   if (q_lds) lds += q_lds_bytes(a.heads, a.head_dim);
+  const size_t k_bytes = (size_t)kWaves * 32 * (a.head_dim / 8) * 16;          // a 32-row key tile per wavefront
+  const bool k_lds = (a.head_dim == 64 || a.head_dim == 128) && lds + k_bytes <= 160 * 1024;
+  if (k_lds) lds += k_bytes;
   const bool f16 = a.in_dtype == CPPMEGA_MI355_F16;
   const void* fn = nullptr;
-#define CM_PICK(KS)                                                                                                   \
-  fn = f16 ? (q_lds ? (const void*)dsa_indexer_loss_mfma_kernel<true, KS, true> : (const void*)dsa_indexer_loss_mfma_kernel<true, KS, false>) \
-           : (q_lds ? (const void*)dsa_indexer_loss_mfma_kernel<false, KS, true> : (const void*)dsa_indexer_loss_mfma_kernel<false, KS, false>)
+#define CM_PICK2(KS, KL)                                                                                                \
+  fn = f16 ? (q_lds ? (const void*)dsa_indexer_loss_mfma_kernel<true, KS, true, KL> : (const void*)dsa_indexer_loss_mfma_kernel<true, KS, false, KL>) \
+           : (q_lds ? (const void*)dsa_indexer_loss_mfma_kernel<false, KS, true, KL> : (const void*)dsa_indexer_loss_mfma_kernel<false, KS, false, KL>)
   switch (a.head_dim / 32) {
-    case 1: CM_PICK(1); break;
-    case 2: CM_PICK(2); break;
-    case 3: CM_PICK(3); break;
-    default: CM_PICK(4); break;
+    case 1: CM_PICK2(1, false); break;
+    case 2: if (k_lds) { CM_PICK2(2, true); } else { CM_PICK2(2, false); } break;
+    case 3: CM_PICK2(3, false); break;
+    default: if (k_lds) { CM_PICK2(4, true); } else { CM_PICK2(4, false); } break;
   }
-#undef CM_PICK
+#undef CM_PICK2
   if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   void* kargs[] = {(void*)&p};
   CM_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(kThreads), kargs, lds, stream));

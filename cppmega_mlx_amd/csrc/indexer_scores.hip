@@ -131,9 +131,19 @@ __global__ __launch_bounds__(kThreads) void indexer_qw_kernel(const IndexerParam
 // 4 kg .. 4 kg + 3 of tile j, i.e. four consecutive keys key0 + 16 j + 4 kg + i of query n, and
 // writes them as one 16-byte store; the four lanes of a query cover 64 contiguous bytes.
 // A workgroup holds QT query tiles (16 QT rows): every key fragment it loads is used for all of them.
-template <bool K_F32, int KSTEPS, int QT>
+// STAGED (bf16 keys whose rows are exactly 32 KSTEPS channels, Skv a multiple of 4): the 64 keys of a
+// wavefront step are one contiguous piece of memory and are fetched as such - neighbouring lanes,
+// neighbouring 16 bytes; loads whose lanes each point into another row move a quarter of the bytes
+// per clock - and pass through a private LDS tile (32 rows at a time, 16-byte slots XOR-swizzled by
+// the row) on their way to operand order.  The finished 16 x 64 score tiles take the same way back:
+// through the LDS tile into stores of whole 256-byte row segments, with the mask read the same way.
+constexpr int kStageBytes = 32 * 2 * kMaxD / 2;    // 8 KB per wavefront: 32 key rows of 256 bytes, or a 16 x 64 float tile (+ padding)
+constexpr int kCPitch = 68;                        // floats per row of the score tile in LDS (64 + 4: rows on distinct banks)
+static_assert(16 * kCPitch * 4 <= kStageBytes, "the score tile reuses the key tile");
+
+template <bool K_F32, int KSTEPS, int QT, bool STAGED = false>
 __global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerParams p) {
-  extern __shared__ __align__(16) unsigned short q_lds[];     // [2][16 QT][Dp + 8]: hi plane, lo plane
+  extern __shared__ __align__(16) unsigned short q_lds[];     // [2][16 QT][Dp + 8]: hi plane, lo plane; then the staging tiles
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bz = (int)blockIdx.z;
   const int b = p.b_begin + bz;
@@ -183,6 +193,89 @@ __global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerP
       }
     }
   };
+  if constexpr (STAGED) {
+    constexpr int PPR = 4 * KSTEPS;                      // 16-byte pieces per key row (4, 8 or 16)
+    constexpr int RP = 16 / PPR;                         // rows per 256 bytes
+    constexpr int NT = 4 * KSTEPS;                       // pieces per lane of a 64-key step
+    unsigned char* stage = reinterpret_cast<unsigned char*>(q_lds + 2 * kQRows * QT * pitch) + wave * kStageBytes;
+    float* ctile = reinterpret_cast<float*>(stage);
+    typedef __attribute__((ext_vector_type(4))) unsigned u4;
+    u4 kc[NT], kn[NT];
+    auto fetch_rows = [&](int key0, u4 (&buf)[NT]) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int P = lane + 64 * t, row = P / PPR, c = P % PPR;
+        const int key = min(key0 + row, p.Skv - 1);      // clamped: keys past the end are never stored
+        buf[t] = *reinterpret_cast<const u4*>((const unsigned short*)p.k + ((size_t)b * p.Skv + (size_t)key) * D + 8 * c);
+      }
+    };
+    int a_off[2][KSTEPS];                                // operand order inside a 32-row half: tile jj, step ks
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int row = 16 * jj + n, c = 4 * ks + kg;
+        a_off[jj][ks] = (row * PPR + (c ^ ((row / RP) % PPR))) * 16;
+      }
+    if (key_begin + 64 * wave < key_end) fetch_rows(key_begin + 64 * wave, kc);
+    for (int key0 = key_begin + 64 * wave; key0 < key_end; key0 += kKeysPerIter) {
+      f32x4 acc[QT][4];
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[qt][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (key0 + kKeysPerIter < key_end) fetch_rows(key0 + kKeysPerIter, kn);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        // rows 32 half .. 32 half + 31 of the step: registers -> LDS in load order (slot swizzled by the row)
+#pragma unroll
+        for (int t = 0; t < NT / 2; ++t) {
+          const int P = lane + 64 * t, row = P / PPR, c = P % PPR;      // position within the half
+          *reinterpret_cast<u4*>(stage + (row * PPR + (c ^ ((row / RP) % PPR))) * 16) = kc[half * (NT / 2) + t];
+        }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const int j = 2 * half + jj;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const bf16x8 ka = *reinterpret_cast<const bf16x8*>(stage + a_off[jj][ks]);
+            const int d0 = 32 * ks + 8 * kg;
+#pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+              const bf16x8 b_hi = *reinterpret_cast<const bf16x8*>(&q_hi[(16 * qt + n) * pitch + d0]);
+              const bf16x8 b_lo = *reinterpret_cast<const bf16x8*>(&q_lo[(16 * qt + n) * pitch + d0]);
+              acc[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, b_hi, acc[qt][j], 0, 0, 0);
+              acc[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, b_lo, acc[qt][j], 0, 0, 0);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) kc[t] = kn[t];
+      // score tiles: lane (n, kg) holds query 16 qt + n, keys 16 j + 4 kg + i -> LDS [query][key] -> row segments
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<f32x4*>(ctile + n * kCPitch + 16 * j + 4 * kg) = acc[qt][j] * p.sm_scale;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int r = 16 * qt + 4 * u + (lane >> 4), col = 4 * (lane & 15);
+          f32x4 v = *reinterpret_cast<const f32x4*>(ctile + (4 * u + (lane >> 4)) * kCPitch + col);
+          const int key = key0 + col;
+          if (r < rows_here && key < key_end) {          // (Skv is a multiple of 4: a group of four keys is in or out as a whole)
+            if (p.mask) {
+              const size_t mrow = ((size_t)b * p.Sq + (size_t)(p.s_begin + s_off + r)) * p.Skv + key;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) v[i] += load_as(p.mask, mrow + i, p.mask_dtype);
+            }
+            *reinterpret_cast<f32x4*>(p.scores + (out_row0 + r) * (size_t)p.Skv + key) = v;
+          }
+        }
+      }
+    }
+    return;
+  }
   const bool prefetch = kPrefetch && p.k_vec;
   if (prefetch && key_begin + 64 * wave < key_end) fetch(key_begin + 64 * wave, cur);
   for (int key0 = key_begin + 64 * wave; key0 < key_end; key0 += kKeysPerIter) {
@@ -360,14 +453,29 @@ int indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t& a, size_t* 
 }
 
 template <bool K_F32, int QT>
-static void launch_scores(const IndexerParams& p, dim3 grid, hipStream_t stream) {
-  const size_t lds = (size_t)2 * kQRows * QT * (((p.D + 31) & ~31) + 8) * sizeof(unsigned short);   // <= 67.6 KB at QT = 4, D = 256: QT = 4 is only used up to D = 128
-  switch ((p.D + 31) / 32) {
-    case 1: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 1, QT>), grid, dim3(kThreads), lds, stream, p); break;
-    case 2: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 2, QT>), grid, dim3(kThreads), lds, stream, p); break;
-    case 4: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 4, QT>), grid, dim3(kThreads), lds, stream, p); break;
-    default: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 0, QT>), grid, dim3(kThreads), lds, stream, p); break;
+static int launch_scores(const IndexerParams& p, dim3 grid, hipStream_t stream) {
+  const size_t q_bytes = (size_t)2 * kQRows * QT * (((p.D + 31) & ~31) + 8) * sizeof(unsigned short);   // <= 67.6 KB at QT = 4, D = 256: QT = 4 is only used up to D = 128
+  const int ks = (p.D + 31) / 32;
+  if constexpr (!K_F32) {
+    if (p.k_vec && p.s_vec && p.D % 32 == 0 && (ks == 1 || ks == 2 || ks == 4)) {
+      const size_t lds = q_bytes + (size_t)(kThreads / 64) * kStageBytes;
+      const void* fn = ks == 1 ? (const void*)indexer_scores_kernel<false, 1, QT, true>
+                     : ks == 2 ? (const void*)indexer_scores_kernel<false, 2, QT, true>
+                               : (const void*)indexer_scores_kernel<false, 4, QT, true>;
+      if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      IndexerParams q = p;
+      void* kargs[] = {(void*)&q};
+      CM_HIP_CHECK(hipLaunchKernel(fn, grid, dim3(kThreads), kargs, lds, stream));
+      return 0;
+    }
   }
+  switch (ks) {
+    case 1: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 1, QT>), grid, dim3(kThreads), q_bytes, stream, p); break;
+    case 2: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 2, QT>), grid, dim3(kThreads), q_bytes, stream, p); break;
+    case 4: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 4, QT>), grid, dim3(kThreads), q_bytes, stream, p); break;
+    default: hipLaunchKernelGGL((indexer_scores_kernel<K_F32, 0, QT>), grid, dim3(kThreads), q_bytes, stream, p); break;
+  }
+  return 0;
 }
 
 int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t stream) {
@@ -407,11 +515,9 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
       const int per = (a.seq_kv + splits - 1) / splits;
       p.keys_per_wg = (per + kKeysPerIter - 1) / kKeysPerIter * kKeysPerIter;
       const dim3 grid((unsigned)((a.seq_kv + p.keys_per_wg - 1) / p.keys_per_wg), (unsigned)tiles, (unsigned)nb);
-      if (a.k_dtype == CPPMEGA_MI355_F32) {
-        if (qt == 4) launch_scores<true, 4>(p, grid, stream); else launch_scores<true, 1>(p, grid, stream);
-      } else {
-        if (qt == 4) launch_scores<false, 4>(p, grid, stream); else launch_scores<false, 1>(p, grid, stream);
-      }
+      if (a.k_dtype == CPPMEGA_MI355_F32) rc = qt == 4 ? launch_scores<true, 4>(p, grid, stream) : launch_scores<true, 1>(p, grid, stream);
+      else rc = qt == 4 ? launch_scores<false, 4>(p, grid, stream) : launch_scores<false, 1>(p, grid, stream);
+      if (rc) return rc;
       CM_HIP_CHECK(hipGetLastError());
 
       const size_t row0 = (size_t)b0 * a.seq_q + (size_t)s_begin;    // first flattened query row of the pass
