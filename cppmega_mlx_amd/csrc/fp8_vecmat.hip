@@ -11,7 +11,10 @@
 //    bytes per instruction and accumulated with v_dot2 (bf16 / fp16) or v_fma (fp32) in fp32 per
 //    128-wide scale block; a row pair's sums are reduced together across the wavefront.
 //  * M == 1, other K or misaligned rows (gemv_kernel): the same shape with bounds tests, fp32 math.
-//  * 5 <= M <= 32, bf16 activations (skinny_mfma_kernel): split-K over 8 workgroup columns with
+//  * 5 <= M <= 16, bf16 activations, K a multiple of 128 (skinny_rows_kernel): a workgroup owns up to
+//    32 weight rows for the whole K; weights converted to bf16 in registers, v_mfma_f32_16x16x32_bf16 on
+//    the activations as they are; one kernel, no workspace.
+//  * 17 <= M <= 32, bf16 activations (skinny_mfma_kernel): split-K over 8 workgroup columns with
 //    v_mfma_scale_f32_16x16x128_f8f6f4.  The weights feed the matrix cores as the e4m3 bytes
 //    they are; the activations are split once per workgroup into two e4m3 planes in LDS.  The
 //    per-split partial sums go to a workspace and a second kernel adds them in split order.
@@ -852,7 +855,7 @@ static bool stream_k(const cppmega_mi355_vecmat_args_t& a) {
 static bool stream_shape(const cppmega_mi355_vecmat_args_t& a) { return stream_k(a) && a.m <= stream_row_cap(a.x_dtype); }
 // the split-K MFMA kernel: bf16 activations, M >= 5 (in passes of 32 rows), K in eighths of whole scale blocks that fit the LDS slice
 constexpr int kSkinnyMaxRows = 32;
-constexpr int kRowsMaxM = 16;             // activation rows the kernel without a K split takes (measured: faster up to here)
+constexpr int kRowsMaxM = 16;             // activation rows the kernel without a K split takes (17..32 measured no faster than the split-K kernel)
 static bool skinny_shape(const cppmega_mi355_vecmat_args_t& a) {
   return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 &&
          (a.k % (kSkinnySplits * 128) == 0) && a.k / kSkinnySplits <= kSkinnyMaxKw;
@@ -862,7 +865,7 @@ static bool skinny_ok(const cppmega_mi355_vecmat_args_t& a) { return vecmat_alig
 // scales of 32 rows and partial tiles within the LDS
 static size_t rows_lds_bytes(int k, int mt) { return (size_t)rows_waves(mt) * (32 * 128 + mt * 16 * 256) + (size_t)(k / 128) * 32 * sizeof(float); }
 static bool rows_shape(const cppmega_mi355_vecmat_args_t& a) {
-  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 && a.m <= kRowsMaxM && a.k % 128 == 0 && rows_lds_bytes(a.k, 1) <= 160 * 1024;
+  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 && a.m <= kRowsMaxM && a.k % 128 == 0 && rows_lds_bytes(a.k, a.m <= 16 ? 1 : 2) <= 160 * 1024;
 }
 
 int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes) {
@@ -991,8 +994,9 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     rows = rows < 16 ? 16 : (rows > kRowsMax ? kRowsMax : rows);
     p.rows_per_wg = rows;
     const dim3 grid((unsigned)((a.n + rows - 1) / rows));
-    const size_t smem = rows_lds_bytes(a.k, 1);
-    const void* fn = (const void*)skinny_rows_kernel<1>;
+    const int mt = a.m <= 16 ? 1 : 2;
+    const size_t smem = rows_lds_bytes(a.k, mt);
+    const void* fn = mt == 1 ? (const void*)skinny_rows_kernel<1> : (const void*)skinny_rows_kernel<2>;
     if (smem > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     void* kargs[] = {(void*)&p};
     CM_HIP_CHECK(hipLaunchKernel(fn, grid, dim3(rows_waves(1) * 64), kargs, smem, stream));
