@@ -300,21 +300,39 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     const int n = lane & 15, kg = lane >> 4;
     // Q^T operands: lane (head n, kg) holds channels 128 blk + 32 kg .. +31 of the latent and
     // channels 512 + 32 r + 8 kg .. +7 of the rope tail
-    uint4 qraw[4][4];
-    bf16x8 qr[2];
-    {
-      const int h = 16 * role + n;
+    // The 16 query rows of this wavefront (18 KB, contiguous when every head exists) are fetched as
+    // they lie in memory - piece lane + 64 t, neighbouring lanes on neighbouring 16 bytes; a load whose
+    // lanes each point into another row moves a quarter of the bytes per clock - and reach operand
+    // order through the ring slot 1 + role, which holds no tile before the first barrier of the
+    // pipeline (rows padded by 16 bytes: the 16 lanes of an operand read fall on distinct banks).
+    typedef __attribute__((ext_vector_type(4))) unsigned u4;
+    constexpr int kQPieces = kDqk / 8;              // 72 pieces of 16 bytes per head row
+    constexpr int kQPitch = kDqk * 2 + 16;          // 1168
+    static_assert(16 * kQPitch <= kLatBytes + kRopeBytes, "the query rows fit a slot without touching its scale area");
+    u4 qload[18];
+#pragma unroll
+    for (int t = 0; t < 18; ++t) {
+      const int P = lane + 64 * t, hl = P / kQPieces, piece = P - hl * kQPieces;
+      const int h = 16 * role + hl;
       // heads past the end of the group repeat head 0: their columns stay finite and are never stored
-      const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (h < heads_here ? h : 0)) * (size_t)kDqk;
-#pragma unroll
-      for (int blk = 0; blk < 4; ++blk)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qraw[blk][j] = *reinterpret_cast<const uint4*>(qrow + 128 * blk + 32 * kg + 8 * j);
-#pragma unroll
-      for (int r = 0; r < 2; ++r) qr[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + kLat + 32 * r + 8 * kg));
+      qload[t] = *reinterpret_cast<const u4*>((const unsigned short*)p.q + (bs * p.H + head0 + (h < heads_here ? h : 0)) * (size_t)kDqk + 8 * piece);
     }
     __builtin_amdgcn_sched_barrier(0);
     stage_keys();
+    unsigned char* qstage = smem + (1 + role) * kSlotBytes;
+#pragma unroll
+    for (int t = 0; t < 18; ++t) {
+      const int P = lane + 64 * t, hl = P / kQPieces, piece = P - hl * kQPieces;
+      *reinterpret_cast<u4*>(qstage + hl * kQPitch + piece * 16) = qload[t];
+    }
+    uint4 qraw[4][4];
+    bf16x8 qr[2];
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) qraw[blk][j] = *reinterpret_cast<const uint4*>(qstage + n * kQPitch + (16 * blk + 4 * kg + j) * 16);
+#pragma unroll
+    for (int r = 0; r < 2; ++r) qr[r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qstage + n * kQPitch + (64 + 4 * r + kg) * 16));
     __syncthreads();                                // keys[] is complete
     const int n_tiles = count_tiles();
     i32x8 qh[4], ql[4];
