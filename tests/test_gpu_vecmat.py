@@ -117,6 +117,37 @@ def test_reference_shaped_fp8_activation_per_row_and_scalar_scales(device, N, K)
         assert err <= F32_TOL * ref
 
 
+@pytest.mark.parametrize("M,N,K", [(5, 7, 128), (16, 33, 384), (12, 300, 16384), (7, 530, 7168), (16, 100, 32768),
+                                   (9, 29, 2176), (16, 7200, 1024), (6, 31, 640)])
+@pytest.mark.parametrize("pow2", [True, False])
+def test_five_to_sixteen_rows_without_a_k_split(device, M, N, K, pow2):
+    """5 <= M <= 16, bf16 activations, K a multiple of 128: one kernel, no workspace; products of bf16 and e4m3
+    values are exact, so float32 outputs are held to the bar of the streaming kernels (1e-5), general scales too."""
+    import ctypes as C
+
+    from cppmega_mlx_amd import _lib
+    rng = np.random.default_rng(M * 7919 + N * 13 + K)
+    codes, scale = _weights(rng, N, K, pow2=pow2)
+    xt, xf = bf16_pair(rng.standard_normal((M, K)), device)
+    a = _lib.VecmatArgs()
+    a.struct_size, a.x_dtype, a.out_dtype, a.scale_w_kind = C.sizeof(a), _lib.BF16, _lib.BF16, _lib.WSCALE_ROW_BLOCK
+    a.m, a.n, a.k = M, N, K
+    need = C.c_size_t(1)
+    assert _lib.load().cppmega_mi355_fp8_vecmat_workspace_bytes(C.byref(a), C.sizeof(a), C.byref(need)) == 0 and need.value == 0
+    want = _oracle_blocked(codes, scale, xf)
+    for out_dtype, tol in ((torch.float32, F32_TOL), (torch.bfloat16, HALF_TOL)):
+        out = torch.full((M, N), 7.0, dtype=out_dtype, device=device)
+        vm.fp8_scaled_vecmat_path_c(xt, to_dev(codes, device), scale_x=None, scale_w=to_dev(scale, device), out=out)
+        torch.cuda.synchronize()
+        err, ref = error_report(out.float().cpu().numpy(), want)
+        assert err <= tol * ref, (err, ref)
+    # the same inputs give the same bits on a second call (fixed summation order)
+    again = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    vm.fp8_scaled_vecmat_path_c(xt, to_dev(codes, device), scale_x=None, scale_w=to_dev(scale, device), out=again)
+    torch.cuda.synchronize()
+    assert torch.equal(again, out)
+
+
 def test_fused_fp8_gemm_grid_scales_and_leading_dims(device):
     rng = np.random.default_rng(6)
     N, K = 300, 1024
