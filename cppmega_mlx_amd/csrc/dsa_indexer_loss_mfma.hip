@@ -279,6 +279,7 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
 
   // ---- pass 2: the divergence -------------------------------------------------------------------
   const float m1 = idxstat[l16 * 2], inv1 = idxstat[l16 * 2 + 1];
+  const bool idx_vec = (p.Sk & 3) == 0 && (reinterpret_cast<uintptr_t>(p.index_scores) & 15) == 0;
   const float inv_heads = 1.0f / (float)p.AH;
   float kl = 0.0f;
   for (int t = wave; t < ntiles; t += kWaves) {
@@ -308,6 +309,18 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       const int kb = key0 + 16 * sub + 4 * kg;
+      // the lane's four index scores: one 16-byte load where the row allows it
+      float iv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (my_row && kb <= my_sq && kb < p.Sk) {
+        if (idx_vec) {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(p.index_scores + my_idx_row + kb);
+          iv[0] = t[0]; iv[1] = t[1]; iv[2] = t[2]; iv[3] = t[3];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (kb + i < p.Sk) iv[i] = p.index_scores[my_idx_row + kb + i];
+        }
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = kb + i;
@@ -315,7 +328,7 @@ __global__ __launch_bounds__(kThreads) void dsa_indexer_loss_mfma_kernel(const L
           const float pj = pacc[sub][i] * inv_heads;
           float qj = 0.0f;
           if (ok[sub][i]) {
-            const float v = p.index_scores[my_idx_row + key] + add[sub][i];
+            const float v = iv[i] + add[sub][i];
             if (v > -INFINITY) qj = __expf(v - m1) * inv1;
           }
           kl += pj * (__logf(pj + kEps) - __logf(qj + kEps));

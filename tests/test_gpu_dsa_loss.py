@@ -128,3 +128,31 @@ def test_long_rows_use_the_large_lds_window():
         for b in range(AB):
             want[b, i] = od.row_loss(idx.double().numpy()[b, i], q.double().numpy()[i, b], k.double().numpy()[:, b], qpos + i + 1, 0.125, mask[b, i])
     np.testing.assert_allclose(got, want, atol=2e-5, rtol=2e-4)
+
+
+@pytest.mark.gpu
+def test_bench_size_properties():
+    """At the size the bench times (4096 positions, 8 heads of 64): the closed form for zero rows and a uniform index,
+    and non-negativity / finiteness of the divergence for random rows, dense and sparse."""
+    ASq = Sk = 4096
+    AB, AH, AD, topk = 1, 8, 64, 1024
+    z = lambda *s: torch.zeros(s, device="cuda", dtype=torch.bfloat16)
+    got = dsa_splitk_indexer_loss_per_position(torch.zeros((AB, ASq, Sk), device="cuda"), None, z(ASq, AB, AH, AD), z(Sk, AB, AH, AD),
+                                               0.125, False).cpu().numpy()
+    want = np.log(Sk) - np.log(np.arange(1, ASq + 1))
+    np.testing.assert_allclose(got[0], want, atol=2e-5, rtol=2e-4)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randn((ASq, AB, AH, AD), generator=g, device="cuda").to(torch.bfloat16)
+    k = torch.randn((Sk, AB, AH, AD), generator=g, device="cuda").to(torch.bfloat16)
+    idx = torch.randn((AB, ASq, Sk), generator=g, device="cuda")
+    top = torch.topk(idx, topk, dim=-1).indices
+    for sparse in (False, True):
+        loss = dsa_splitk_indexer_loss_per_position(idx, top, q, k, AD ** -0.5, sparse)
+        assert torch.isfinite(loss).all() and (loss >= -1e-4).all()       # a divergence of p against a sub-normalised q
+    # a few rows against the float64 oracle row function
+    mask = None
+    for sq in (0, 17, 2047, 4095):
+        w = od.row_loss(idx[0, sq].double().cpu().numpy(), q[sq, 0].double().cpu().numpy(), k[:, 0].double().cpu().numpy(), sq + 1,
+                        AD ** -0.5, mask)
+        d = float(dsa_splitk_indexer_loss_per_position(idx, top, q, k, AD ** -0.5, False)[0, sq])
+        assert abs(d - w) <= 2e-5 + 2e-4 * abs(w), (sq, d, w)

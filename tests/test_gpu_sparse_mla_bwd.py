@@ -216,3 +216,32 @@ def test_per_token_fp8_backward_over_prepared_buffers(device):
         o2.sum().backward()
     with pytest.raises(RuntimeError, match="requires prepared FP8 buffers"):
         f8.sparse_mla_fp8_path_c_apply_from_float(qf, kf, to_dev(idx, device), sm_scale=0.2)
+
+
+def test_bench_size_invariants_of_the_backward(device):
+    """At the size the bench times: the columns of dkv sum to the cotangents of the queries that had a valid key on the
+    first d_v channels (every softmax row sums to 1) and to zero on the rest (every dS row sums to 0); the gradients
+    are linear in d_out."""
+    B, S, H, D, d_v, Skv, topk = 1, 1024, 16, 576, 512, 4096, 256
+    gen = torch.Generator(device=device).manual_seed(5)
+    q = torch.randn((B, S, H, D), generator=gen, device=device).to(torch.bfloat16)
+    kv = (torch.randn((B, Skv, 1, D), generator=gen, device=device) * 0.5).to(torch.bfloat16)
+    d_out = torch.randn((B, S, H, d_v), generator=gen, device=device).to(torch.bfloat16)
+    idx = torch.stack([torch.randperm(Skv, generator=gen, device=device)[:topk] for _ in range(S)]).to(torch.int32).view(B, S, 1, topk).clone()
+    idx[0, 5] = -1                                            # one query without keys
+    dq = torch.empty((B, S, H, D), dtype=torch.float32, device=device)
+    dkv = torch.empty((B, Skv, 1, D), dtype=torch.float32, device=device)
+    ops.sparse_mla_backward(q, kv, d_out, idx, sm_scale=D ** -0.5, d_v=d_v, dq=dq, dkv=dkv)
+    torch.cuda.synchronize()
+    cols = dkv.double().sum(dim=(0, 1, 2)).cpu().numpy()
+    live = torch.ones(S, dtype=torch.bool, device=device); live[5] = False
+    want = d_out[0, live].double().sum(dim=(0, 1)).cpu().numpy()
+    scale = float(np.abs(dkv.cpu().numpy()).sum(axis=(0, 1, 2)).max())      # what the column sums are sums of
+    assert np.abs(cols[:d_v] - want).max() <= 1e-5 * scale
+    assert np.abs(cols[d_v:]).max() <= 1e-5 * scale
+    assert (dq[0, 5] == 0).all()
+    dq2 = torch.empty_like(dq); dkv2 = torch.empty_like(dkv)
+    ops.sparse_mla_backward(q, kv, d_out * 2, idx, sm_scale=D ** -0.5, d_v=d_v, dq=dq2, dkv=dkv2)
+    torch.cuda.synchronize()
+    assert torch.equal(dq2, dq * 2)                            # doubling is exact in every step of dq
+    assert float((dkv2 - 2 * dkv).abs().max()) <= 1e-5 * float(dkv.abs().max())   # atomic order only
