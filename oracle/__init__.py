@@ -35,4 +35,12 @@ Pinning status (what fixes each function besides its own formula):
   set on distinct scores and the reference's rope known answers.
 * ``vecmat.*``                   -- pinned against float64 ``W_deq @ x`` with
   torch's independent e4m3 decoder.
+* ``mla_absorb.*``               -- pinned by the reference's identity absorbed == standard
+  decode and by explicit einsum loops.
+* ``sparse_mla.sparse_mla_bwd_oracle`` -- pinned by central finite differences of the forward
+  oracle in float64 and by torch autograd through a dense softmax attention restricted to the
+  selected keys.
+* ``dsa_loss.*``                 -- pinned by closed forms (zero rows and a uniform index give
+  log(Sk) - log(sq + 1); an index equal to the log of the attention distribution on a full
+  row gives 0) and an explicit triple loop with a sparse mask.
 """
