@@ -11,7 +11,8 @@
 //    bytes per instruction and accumulated with v_dot2 (bf16 / fp16) or v_fma (fp32) in fp32 per
 //    128-wide scale block; a row pair's sums are reduced together across the wavefront.
 //  * M == 1, other K or misaligned rows (gemv_kernel): the same shape with bounds tests, fp32 math.
-//  * 5 <= M <= 16, bf16 activations, K a multiple of 128 (skinny_rows_kernel): a workgroup owns up to
+//  * 5 <= M <= 16 bf16 activations (any M >= 5 for fp16, in passes of 16), K a multiple of 128
+//    (skinny_rows_kernel): a workgroup owns up to
 //    32 weight rows for the whole K; weights converted to bf16 in registers, v_mfma_f32_16x16x32_bf16 on
 //    the activations as they are; one kernel, no workspace.
 //  * 17 <= M <= 32, bf16 activations (skinny_mfma_kernel): split-K over 8 workgroup columns with
@@ -626,7 +627,10 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_mfma_kernel(const Ve
 constexpr int kRowsMax = 32;              // weight rows per workgroup (two MFMA row tiles)
 __host__ __device__ constexpr int rows_waves(int) { return 8; }
 
-template <int MT>
+typedef _Float16 f16x8v __attribute__((ext_vector_type(8)));
+
+// F16: float16 activations (weights become float16 pairs, exact; v_mfma_f32_16x16x32_f16)
+template <int MT, bool F16 = false>
 __global__ __launch_bounds__(rows_waves(MT) * 64) void skinny_rows_kernel(const VecmatParams p) {
   constexpr int kRowsWaves = rows_waves(MT);
   constexpr int DEPTH = MT == 1 ? 3 : 2;               // blocks in flight per wavefront (registers)
@@ -741,14 +745,26 @@ __global__ __launch_bounds__(rows_waves(MT) * 64) void skinny_rows_kernel(const 
 #pragma unroll
           for (int s4 = 0; s4 < 4; ++s4) {             // MFMA step s4: channels 32 kg + 8 s4 .. + 7 of the block
             uint4 a;
-            a.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4], 1.0f, false));
-            a.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4], 1.0f, true));
-            a.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4 + 1], 1.0f, false));
-            a.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4 + 1], 1.0f, true));
+            if (F16) {
+              a.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wd[2 * s4], 1.0f, false));
+              a.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wd[2 * s4], 1.0f, true));
+              a.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wd[2 * s4 + 1], 1.0f, false));
+              a.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wd[2 * s4 + 1], 1.0f, true));
+            } else {
+              a.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4], 1.0f, false));
+              a.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4], 1.0f, true));
+              a.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4 + 1], 1.0f, false));
+              a.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wd[2 * s4 + 1], 1.0f, true));
+            }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-              tile[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, xb[mt][s4]),
-                                                                     tile[rt][mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) {
+              if (F16)
+                tile[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8v, a), __builtin_bit_cast(f16x8v, xb[mt][s4]),
+                                                                      tile[rt][mt], 0, 0, 0);
+              else
+                tile[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, xb[mt][s4]),
+                                                                       tile[rt][mt], 0, 0, 0);
+            }
           }
         }
         // tile element i: weight row 16 rt + 4 kg + i, activation row 16 mt + r16
@@ -865,7 +881,10 @@ static bool skinny_ok(const cppmega_mi355_vecmat_args_t& a) { return vecmat_alig
 // scales of 32 rows and partial tiles within the LDS
 static size_t rows_lds_bytes(int k, int mt) { return (size_t)rows_waves(mt) * (32 * 128 + mt * 16 * 256) + (size_t)(k / 128) * 32 * sizeof(float); }
 static bool rows_shape(const cppmega_mi355_vecmat_args_t& a) {
-  return a.x_dtype == CPPMEGA_MI355_BF16 && a.m >= 5 && a.m <= kRowsMaxM && a.k % 128 == 0 && rows_lds_bytes(a.k, a.m <= 16 ? 1 : 2) <= 160 * 1024;
+  const bool bf16 = a.x_dtype == CPPMEGA_MI355_BF16;
+  // float16 rows have no split-K kernel behind them (they would run in passes of 4 on the streaming kernel): any M >= 5
+  if (a.x_dtype == CPPMEGA_MI355_F16) return a.m >= 5 && a.k % 128 == 0 && rows_lds_bytes(a.k, 1) <= 160 * 1024;
+  return bf16 && a.m >= 5 && a.m <= kRowsMaxM && a.k % 128 == 0 && rows_lds_bytes(a.k, a.m <= 16 ? 1 : 2) <= 160 * 1024;
 }
 
 int fp8_vecmat_workspace_bytes(const cppmega_mi355_vecmat_args_t& a, size_t* bytes) {
@@ -994,12 +1013,18 @@ int fp8_vecmat_launch(const cppmega_mi355_vecmat_args_t& a, hipStream_t stream) 
     rows = rows < 16 ? 16 : (rows > kRowsMax ? kRowsMax : rows);
     p.rows_per_wg = rows;
     const dim3 grid((unsigned)((a.n + rows - 1) / rows));
-    const int mt = a.m <= 16 ? 1 : 2;
-    const size_t smem = rows_lds_bytes(a.k, mt);
-    const void* fn = mt == 1 ? (const void*)skinny_rows_kernel<1> : (const void*)skinny_rows_kernel<2>;
+    const size_t smem = rows_lds_bytes(a.k, 1);
+    const bool f16 = a.x_dtype == CPPMEGA_MI355_F16;
+    const void* fn = f16 ? (const void*)skinny_rows_kernel<1, true> : (const void*)skinny_rows_kernel<1, false>;
     if (smem > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    void* kargs[] = {(void*)&p};
-    CM_HIP_CHECK(hipLaunchKernel(fn, grid, dim3(rows_waves(1) * 64), kargs, smem, stream));
+    for (int m0 = 0; m0 < a.m; m0 += 16) {             // (more than 16 rows: float16 only, in passes)
+      VecmatParams q = p;
+      q.m = a.m - m0 < 16 ? a.m - m0 : 16;
+      q.x = (const char*)a.x + (size_t)m0 * a.k * dtype_size(a.x_dtype);
+      q.out = (char*)a.out + (size_t)m0 * a.n * dtype_size(a.out_dtype);
+      void* kargs[] = {(void*)&q};
+      CM_HIP_CHECK(hipLaunchKernel(fn, grid, dim3(rows_waves(1) * 64), kargs, smem, stream));
+    }
   } else if (skinny_ok(a)) {
     // more than 32 activation rows: passes of 32 over the same workspace (stream order keeps them apart)
     const int cap = a.m < kSkinnyMaxRows ? a.m : kSkinnyMaxRows;

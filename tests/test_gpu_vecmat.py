@@ -78,7 +78,8 @@ def test_block_scaled_bf16_small_batch_arbitrary_scales(device, M, N, K):
 
 @pytest.mark.parametrize("x_dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("M,N,K", [(1, 100, 4096), (1, 130, 7168), (1, 64, 16384), (1, 40, 1536), (1, 33, 29696),
-                                   (1, 7, 100), (2, 77, 2048), (3, 129, 7168), (4, 64, 16384), (5, 48, 1024), (7, 64, 2048), (3, 50, 1040)])
+                                   (1, 7, 100), (2, 77, 2048), (3, 129, 7168), (4, 64, 16384), (5, 48, 1024), (7, 64, 2048), (3, 50, 1040),
+                                   (16, 300, 7168), (40, 33, 384), (12, 7, 128)])
 def test_block_scaled_fp16_fp32_activation(device, M, N, K, x_dtype):
     """fp16 / fp32 activations (exact inputs for the oracle: the values are rounded to the carrier first)."""
     rng = np.random.default_rng(M * 7919 + N * 31 + K)
