@@ -662,19 +662,22 @@ __global__ __launch_bounds__(rows_waves(MT) * 64) void skinny_rows_kernel(const 
   }
 
   // load order: position = lane + 64 j holds (row, slot); the piece fetched into a slot is slot ^ swizzle(row)
-  const unsigned char* wsrc[4];
+  // (32-bit lane offsets from a uniform base: the address of a load is scalar base + lane offset, no vector arithmetic)
+  const unsigned char* wbase = p.w + (size_t)n0 * p.k;
+  unsigned woff[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int pos = lane + 64 * j, row = pos >> 3, slot = pos & 7;
-    wsrc[j] = p.w + (size_t)(n0 + min(row, rows_here - 1)) * p.k + 16 * (slot ^ ((row >> 1) & 7));
+    woff[j] = (unsigned)min(row, rows_here - 1) * (unsigned)p.k + 16u * (unsigned)(slot ^ ((row >> 1) & 7));
   }
-  const unsigned char* xsrc[MT][4];
+  const unsigned char* xbase = (const unsigned char*)p.x;
+  unsigned xoff[MT][4];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int pos = lane + 64 * j, row = pos >> 4, slot = pos & 15;
-      xsrc[mt][j] = (const unsigned char*)p.x + ((size_t)min(16 * mt + row, p.m - 1) * p.k) * 2 + 16 * (slot ^ row);
+      xoff[mt][j] = (unsigned)min(16 * mt + row, p.m - 1) * (unsigned)p.k * 2u + 16u * (unsigned)(slot ^ row);
     }
   // operand order: lane (r16, kg)
   int a_off[2][2], b_off[MT][4];                       // byte offsets inside a tile set
@@ -694,12 +697,14 @@ __global__ __launch_bounds__(rows_waves(MT) * 64) void skinny_rows_kernel(const 
   u4 wq[DEPTH][4];
   u4 xq[DEPTH][MT][4];
   auto fetch = [&](int slot, int kb) {
+    const unsigned char* wb = wbase + (size_t)kb * 128;
+    const unsigned char* xb_ = xbase + (size_t)kb * 256;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) wq[slot][j] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(wsrc[j] + (size_t)kb * 128));
+    for (int j = 0; j < 4; ++j) wq[slot][j] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(wb + woff[j]));
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xq[slot][mt][j] = *reinterpret_cast<const u4*>(xsrc[mt][j] + (size_t)kb * 256);
+      for (int j = 0; j < 4; ++j) xq[slot][mt][j] = *reinterpret_cast<const u4*>(xb_ + xoff[mt][j]);
   };
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d)
