@@ -337,6 +337,13 @@ def bench_topk(args, device):
         "roofline": {"bound": "hbm", "achieved": bytes_alg / per / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bytes_alg / per / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic("topk_selector")},
     }
+    # the same rows with the selection ordered by value (the order of the reference's kernel; the attention path takes index order)
+    secs_v, _ = timed_graph([lambda i=i: tk.topk_selector_tilelang_direct(scores[i], k, out=outs[i], ends=ends, order="value")
+                             for i in range(n_sets)], steps, args.warmup)
+    res["value_order"] = {"workload": res["workload"] + ", value-descending output", "us_per_launch": secs_v / steps * 1e6,
+                          "algorithmic_bytes": bytes_alg,
+                          "roofline": {"bound": "hbm", "achieved": bytes_alg / (secs_v / steps) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                       "frac": bytes_alg / (secs_v / steps) / 1e9 / HBM_PEAK_GBS, "traffic": None}}
     # the decode-time shape: one row per sequence over the whole cache, two-stage selection
     from cppmega_mlx_amd import ops
     wide = [torch.randn((32, 65536), generator=gen, device=device) for _ in range(n_sets)]
