@@ -245,3 +245,62 @@ def test_bench_size_invariants_of_the_backward(device):
     torch.cuda.synchronize()
     assert torch.equal(dq2, dq * 2)                            # doubling is exact in every step of dq
     assert float((dkv2 - 2 * dkv).abs().max()) <= 1e-5 * float(dkv.abs().max())   # atomic order only
+
+
+def test_training_entry_points_replay_from_a_hip_graph(device):
+    """The backward (with its dkv clear, a fill kernel) and the indexer loss captured once; each replay, with the
+    inputs rewritten and eager launches in between, must reproduce the eager result for the contents at that moment."""
+    from cppmega_mlx_amd.nn._tilelang.dsa_splitk_indexer_loss import dsa_splitk_indexer_loss_per_position
+
+    gen = torch.Generator(device=device).manual_seed(21)
+    B, S, H, D, d_v, Skv, topk = 1, 12, 16, 128, 64, 96, 40
+    q = torch.randn((B, S, H, D), generator=gen, device=device).to(torch.bfloat16)
+    kv = torch.randn((B, Skv, 1, D), generator=gen, device=device).to(torch.bfloat16)
+    d_out = torch.randn((B, S, H, d_v), generator=gen, device=device).to(torch.bfloat16)
+    idx = torch.stack([torch.randperm(Skv, generator=gen, device=device)[:topk] for _ in range(S)]).to(torch.int32).view(B, S, 1, topk)
+    sm = torch.tensor([D ** -0.5], dtype=torch.float32, device=device)
+    ASq = Sk = 48
+    lq = torch.randn((ASq, 1, 4, 64), generator=gen, device=device).to(torch.bfloat16)
+    lk = torch.randn((Sk, 1, 4, 64), generator=gen, device=device).to(torch.bfloat16)
+    lidx = torch.randn((1, ASq, Sk), generator=gen, device=device)
+    ltop = torch.topk(lidx, 8, dim=-1).indices.to(torch.int32).contiguous()
+
+    def buffers():
+        return dict(dq=torch.zeros((B, S, H, D), dtype=torch.float32, device=device),
+                    dkv=torch.zeros((B, Skv, 1, D), dtype=torch.float32, device=device),
+                    loss=torch.zeros((1, ASq), dtype=torch.float32, device=device))
+
+    def launch(o):
+        ops.sparse_mla_backward(q, kv, d_out, idx, sm_scale=sm, d_v=d_v, dq=o["dq"], dkv=o["dkv"])
+        ops.dsa_indexer_loss(lq, lk, lidx, softmax_scale=0.125, out=o["loss"], topk_indices=ltop)
+
+    captured, eager = buffers(), buffers()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        launch(captured)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        launch(captured)
+    for step in range(3):
+        sm.fill_(D ** -0.5 * (1 + step))
+        d_out.mul_(-1.5)
+        lidx.add_(0.25 * step * torch.arange(Sk, device=device, dtype=torch.float32))
+        for t in captured.values():
+            t.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        launch(eager)
+        torch.cuda.synchronize()
+        assert torch.equal(captured["dq"], eager["dq"]) and torch.equal(captured["loss"], eager["loss"]), step
+        assert float((captured["dkv"] - eager["dkv"]).abs().max()) <= 1e-5 * float(eager["dkv"].abs().max())   # atomic order
+        want_dq, want_dkv = om.sparse_mla_bwd_oracle(q.double().cpu().numpy(), kv.double().cpu().numpy(), idx.cpu().numpy(),
+                                                     d_out.double().cpu().numpy(), sm_scale=float(sm), d_v=d_v)
+        err, ref = error_report(captured["dq"].cpu().numpy(), want_dq)
+        assert err <= 1e-4 * ref
+        err, ref = error_report(captured["dkv"].cpu().numpy(), want_dkv)
+        assert err <= 1e-4 * ref
+    want_loss = dsa_splitk_indexer_loss_per_position(lidx, ltop, lq, lk, 0.125, True)
+    assert torch.equal(captured["loss"], want_loss)
