@@ -180,7 +180,7 @@ int sparse_mla_bwd_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hipStrea
     return fail(CPPMEGA_MI355_ERR_NULL, "sparse_mla_bwd: e4m3 operands need their per-token scales");
   if (a.index_dtype != CPPMEGA_MI355_I32 && a.index_dtype != CPPMEGA_MI355_I64)
     return fail(CPPMEGA_MI355_ERR_DTYPE, "sparse_mla_bwd: indices must be int32 or int64");
-  const bool on_matrix_cores = sparse_mla_bwd_mfma_supports(a);      // bfloat16 (or per-token e4m3) q / kv with a bfloat16 d_out
+  const bool on_matrix_cores = sparse_mla_bwd_mfma_supports(a);      // bfloat16 / float16 (or per-token e4m3) operands
   const size_t lds = ((size_t)3 * a.topk + a.d_qk + a.d_v + 8) * sizeof(float);
   if (!on_matrix_cores && lds > 160 * 1024) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: topk %d with d_qk %d needs %zu bytes of LDS (limit 160 KiB)", a.topk, a.d_qk, lds);
   const size_t n_dkv = (size_t)a.batch * a.seq_kv * a.kv_groups * a.d_qk;

@@ -1,5 +1,5 @@
-// Sparse MLA backward on the matrix cores: bfloat16 operands, or e4m3 q / kv with per-token
-// scales (gfx950).
+// Sparse MLA backward on the matrix cores: bfloat16 or float16 operands, or e4m3 q / kv with
+// per-token scales (gfx950).
 //
 // Same gradients as sparse_mla_bwd.hip (the reference's sparse_mla_bwd_direct,
 // cppmega_mlx/nn/_tilelang/sparse_mla_path_c.py:2644-2816), organised so that the heads of a KV
@@ -87,12 +87,31 @@ __device__ __forceinline__ uint4 e4m3x8_to_bf16(const uint2 v) {
   r.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.y, 1.0f, true));
   return r;
 }
+typedef _Float16 f16x8b __attribute__((ext_vector_type(8)));
+// one matrix instruction on operands held as 8 x 16 bits: bfloat16, or float16 when F16
+template <bool F16>
+__device__ __forceinline__ f32x4 mm(const bf16x8 a, const bf16x8 b, const f32x4 c) {
+  if (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8b, a), __builtin_bit_cast(f16x8b, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ unsigned pack_f16(float a, float b) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 r;
+  r[0] = (_Float16)a;
+  r[1] = (_Float16)b;
+  return __builtin_bit_cast(unsigned, r);
+}
 __device__ __forceinline__ bf16x8 zero8() {
   return __builtin_bit_cast(bf16x8, make_uint4(0u, 0u, 0u, 0u));
 }
 
-template <int HB, bool FP8>
+// EL: 0 bfloat16 operands, 1 per-token e4m3 operands (bfloat16 arithmetic), 2 float16 operands
+template <int HB, int EL>
 __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const BwdMfmaParams p) {
+  constexpr bool FP8 = EL == 1, F16 = EL == 2;
+  // float16 planes of P and dS are kept at 16 times their value: a float16 is flushed below 6e-8 and overflows above
+  // 65504, so entries down to 4e-9 survive and |dS| may reach 4000
+  constexpr float kPlaneScale = F16 ? 16.0f : 1.0f, kPlaneUnscale = F16 ? 1.0f / 16.0f : 1.0f;
   constexpr int HC = 16 * HB;            // heads per workgroup
   constexpr int KT = 64 / HB;            // keys per tile
   constexpr int KSUB = KT / 16;          // 16-key blocks per tile
@@ -218,11 +237,11 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
     dp = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int kk = 0; kk < dv32; ++kk) {
       const bf16x8 a = lds_b128(a_base + kk * 32);
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, lds_b128(q_base + kk * 32), s, 0, 0, 0);
-      dp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, lds_b128(o_base + kk * 32), dp, 0, 0, 0);
+      s = mm<F16>(a, lds_b128(q_base + kk * 32), s);
+      dp = mm<F16>(a, lds_b128(o_base + kk * 32), dp);
     }
     for (int kk = dv32; kk < d32; ++kk)
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_b128(a_base + kk * 32), lds_b128(q_base + kk * 32), s, 0, 0, 0);
+      s = mm<F16>(lds_b128(a_base + kk * 32), lds_b128(q_base + kk * 32), s);
     if (FP8) {                                        // code-value products -> products of the dequantised values
       const f32x4 kscale = *reinterpret_cast<const f32x4*>(ksc + 16 * ks + 4 * kg);
       const float qscale = qsc[16 * hb + l16];
@@ -319,11 +338,19 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
       }
       const int off = (16 * hb + l16) * Kp + 16 * ks + 4 * kg;
       auto planes = [&](unsigned short* base, const float (&v)[4]) {      // hi and lo bfloat16 planes of 4 values
-        float lo[4];
+        float hi[4], lo[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lo[i] = v[i] - (float)(__bf16)v[i];
-        *reinterpret_cast<uint2*>(base + off) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
-        *reinterpret_cast<uint2*>(base + kPlane + off) = make_uint2(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]));
+        for (int i = 0; i < 4; ++i) {
+          hi[i] = v[i] * kPlaneScale;
+          lo[i] = hi[i] - (F16 ? (float)(_Float16)hi[i] : (float)(__bf16)hi[i]);
+        }
+        if (F16) {
+          *reinterpret_cast<uint2*>(base + off) = make_uint2(pack_f16(hi[0], hi[1]), pack_f16(hi[2], hi[3]));
+          *reinterpret_cast<uint2*>(base + kPlane + off) = make_uint2(pack_f16(lo[0], lo[1]), pack_f16(lo[2], lo[3]));
+        } else {
+          *reinterpret_cast<uint2*>(base + off) = make_uint2(pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]));
+          *reinterpret_cast<uint2*>(base + kPlane + off) = make_uint2(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]));
+        }
       };
       planes(Ps, pv);
       if (FP8) {
@@ -359,8 +386,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
           const bf16x8 a = join(lds_tr16(src), lds_tr16(src + 4 * Dp));
 #pragma unroll
           for (int h2 = 0; h2 < HB; ++h2) {
-            accq[j][h2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bds[h2][0], accq[j][h2], 0, 0, 0);
-            accq[j][h2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bds[h2][1], accq[j][h2], 0, 0, 0);
+            accq[j][h2] = mm<F16>(a, bds[h2][0], accq[j][h2]);
+            accq[j][h2] = mm<F16>(a, bds[h2][1], accq[j][h2]);
           }
         }
       }
@@ -394,13 +421,13 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
           if (HB == 2) {
             const unsigned short* qsrc = Qs + (8 * kg + tr_row) * Dp + cb * 16 + tr_col;
             const bf16x8 bq = join(lds_tr16(qsrc), lds_tr16(qsrc + 4 * Dp));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_ds[0], bq, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_ds[1], bq, acc, 0, 0, 0);
+            acc = mm<F16>(a_ds[0], bq, acc);
+            acc = mm<F16>(a_ds[1], bq, acc);
             if (has_v) {
               const unsigned short* osrc = dOs + (8 * kg + tr_row) * Dvp + cb * 16 + tr_col;
               const bf16x8 bo = join(lds_tr16(osrc), lds_tr16(osrc + 4 * Dvp));
-              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_p[0], bo, acc, 0, 0, 0);
-              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_p[1], bo, acc, 0, 0, 0);
+              acc = mm<F16>(a_p[0], bo, acc);
+              acc = mm<F16>(a_p[1], bo, acc);
             }
           } else {
             // every lane issues the transposing read (it moves data between the lanes of a group of
@@ -411,14 +438,14 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
             const int pitch4 = 4 * (from_q ? Dp : Dvp);
             bf16x8 bq = join(lds_tr16(src), lds_tr16(src + pitch4));
             if (kg >= 2 && !has_v) bq = zero8();
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_ds[0], bq, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_ds[1], bq, acc, 0, 0, 0);
+            acc = mm<F16>(a_ds[0], bq, acc);
+            acc = mm<F16>(a_ds[1], bq, acc);
           }
           // element i: key kb * 16 + 4 * kg + i of the tile, channel cb * 16 + l16
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             if (row_i[i] >= 0)
-              atomicAdd(p.dkv + (((size_t)b * p.Skv + (size_t)row_i[i]) * p.G + g) * (size_t)D + cb * 16 + l16, acc[i]);
+              atomicAdd(p.dkv + (((size_t)b * p.Skv + (size_t)row_i[i]) * p.G + g) * (size_t)D + cb * 16 + l16, acc[i] * kPlaneUnscale);
         }
       }
     }
@@ -436,7 +463,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
         if (h < nh) {
           const size_t base = (bs * p.H + h0 + h) * (size_t)D + cb * 16 + 4 * kg;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) store_as(p.dq, base + i, p.dq_dtype, accq[j][h2][i]);
+          for (int i = 0; i < 4; ++i) store_as(p.dq, base + i, p.dq_dtype, accq[j][h2][i] * kPlaneUnscale);
         }
       }
     }
@@ -459,12 +486,13 @@ bool fp8_operands(const cppmega_mi355_sparse_mla_bwd_args_t& a) {
 // Whether the matrix-core kernel takes this problem (else the fp32 kernel runs).
 bool sparse_mla_bwd_mfma_supports(const cppmega_mi355_sparse_mla_bwd_args_t& a) {
   const bool bf16 = a.q_dtype == CPPMEGA_MI355_BF16 && a.kv_dtype == CPPMEGA_MI355_BF16;
-  if ((!bf16 && !fp8_operands(a)) || a.d_out_dtype != CPPMEGA_MI355_BF16) return false;
+  const bool f16 = a.q_dtype == CPPMEGA_MI355_F16 && a.kv_dtype == CPPMEGA_MI355_F16;
+  if (f16 ? a.d_out_dtype != CPPMEGA_MI355_F16 : ((!bf16 && !fp8_operands(a)) || a.d_out_dtype != CPPMEGA_MI355_BF16)) return false;
   if (a.d_qk % 32 != 0 || a.d_v % 32 != 0 || a.d_qk > kMaxBlk * 64 || a.topk < 1) return false;
   const int hg = a.heads / a.kv_groups;
   const int kt = hg > 16 ? 32 : 64;
   const int ntiles = (a.topk + kt - 1) / kt;
-  const size_t lds = hg > 16 ? lds_bytes<2>(a.d_qk, a.d_v, ntiles, !bf16) : lds_bytes<1>(a.d_qk, a.d_v, ntiles, !bf16);
+  const size_t lds = hg > 16 ? lds_bytes<2>(a.d_qk, a.d_v, ntiles, fp8_operands(a)) : lds_bytes<1>(a.d_qk, a.d_v, ntiles, fp8_operands(a));
   return lds <= 160 * 1024;
 }
 
@@ -485,8 +513,9 @@ int sparse_mla_bwd_mfma_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hip
   if (grid == 0) return 0;
   if (grid > 0x7fffffffull) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: too many (batch, query, head chunk) workgroups for one launch");
   const size_t lds = wide ? lds_bytes<2>(a.d_qk, a.d_v, p.ntiles, fp8) : lds_bytes<1>(a.d_qk, a.d_v, p.ntiles, fp8);
-  const void* fn = wide ? (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<2, true> : (const void*)sparse_mla_bwd_mfma_kernel<2, false>)
-                        : (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<1, true> : (const void*)sparse_mla_bwd_mfma_kernel<1, false>);
+  const bool f16 = a.q_dtype == CPPMEGA_MI355_F16;
+  const void* fn = wide ? (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<2, 1> : f16 ? (const void*)sparse_mla_bwd_mfma_kernel<2, 2> : (const void*)sparse_mla_bwd_mfma_kernel<2, 0>)
+                        : (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<1, 1> : f16 ? (const void*)sparse_mla_bwd_mfma_kernel<1, 2> : (const void*)sparse_mla_bwd_mfma_kernel<1, 0>);
   if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   void* kargs[] = {(void*)&p};
   CM_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(kThreads), kargs, lds, stream));

@@ -70,14 +70,15 @@ MATRIX_CORE_CASES = [
 
 @pytest.mark.parametrize("shape", MATRIX_CORE_CASES, ids=lambda c: "B%dS%dH%dG%dT%dk%dD%ddv%d" % tuple(c.values()))
 @pytest.mark.parametrize("index_dtype", [np.int32, np.int64])
-def test_bfloat16_backward_on_the_matrix_cores(device, shape, index_dtype):
-    """bfloat16 q / kv / d_out take the matrix-core kernel; with float32 dq both gradients are held to
-    1e-4 of their scale (P and dS enter the second products as hi + lo bfloat16 planes)."""
+@pytest.mark.parametrize("carrier", [torch.bfloat16, torch.float16])
+def test_bfloat16_backward_on_the_matrix_cores(device, shape, index_dtype, carrier):
+    """bfloat16 (or float16: the reference kernel's own carrier) q / kv / d_out take the matrix-core kernel; with
+    float32 dq both gradients are held to 1e-4 of their scale (P and dS enter the second products as hi + lo planes)."""
     B, S, H, G, Skv, topk, D, d_v = shape.values()
     rng = np.random.default_rng(B * 1000 + H * 10 + topk)
-    qt = to_dev(rng.standard_normal((B, S, H, D)).astype(np.float32), device).to(torch.bfloat16)
-    kt = to_dev(rng.standard_normal((B, Skv, G, D)).astype(np.float32), device).to(torch.bfloat16)
-    dt = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(torch.bfloat16)
+    qt = to_dev(rng.standard_normal((B, S, H, D)).astype(np.float32), device).to(carrier)
+    kt = to_dev(rng.standard_normal((B, Skv, G, D)).astype(np.float32), device).to(carrier)
+    dt = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(carrier)
     idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
     idx[rng.random(idx.shape) < 0.15] = -1
     idx[0, 1] = -1
@@ -93,12 +94,12 @@ def test_bfloat16_backward_on_the_matrix_cores(device, shape, index_dtype):
         err, ref = error_report(got.cpu().numpy(), want)
         assert err <= 1e-4 * ref, (err, ref)
     assert (dq[0, 1] == 0).all()
-    # bfloat16 dq: one rounding of the same values
-    dq16 = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=device)
+    # dq in the carrier: one rounding of the same values
+    dq16 = torch.empty((B, S, H, D), dtype=carrier, device=device)
     ops.sparse_mla_backward(qt, kt, dt, to_dev(idx.astype(index_dtype), device), sm_scale=torch.tensor([sm], device=device), d_v=d_v,
                             dq=dq16, dkv=dkv)
     torch.cuda.synchronize()
-    assert torch.equal(dq16, dq.to(torch.bfloat16))
+    assert torch.equal(dq16, dq.to(carrier))
 
 
 @pytest.mark.parametrize("shape", [
