@@ -78,7 +78,15 @@ __device__ __forceinline__ bf16x8 join(const bf16x4 a, const bf16x4 b) {
   r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
   return r;
 }
-// 8 e4m3 bytes -> 8 bfloat16, exact
+// 8 e4m3 bytes -> 8 float16 / 8 bfloat16, exact
+__device__ __forceinline__ uint4 e4m3x8_to_f16(const uint2 v) {
+  uint4 r;
+  r.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(v.x, 1.0f, false));
+  r.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(v.x, 1.0f, true));
+  r.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(v.y, 1.0f, false));
+  r.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(v.y, 1.0f, true));
+  return r;
+}
 __device__ __forceinline__ uint4 e4m3x8_to_bf16(const uint2 v) {
   uint4 r;
   r.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(v.x, 1.0f, false));
@@ -105,10 +113,11 @@ __device__ __forceinline__ bf16x8 zero8() {
   return __builtin_bit_cast(bf16x8, make_uint4(0u, 0u, 0u, 0u));
 }
 
-// EL: 0 bfloat16 operands, 1 per-token e4m3 operands (bfloat16 arithmetic), 2 float16 operands
+// EL: 0 bfloat16 operands, 1 per-token e4m3 operands with a bfloat16 cotangent, 2 float16 operands,
+//     3 per-token e4m3 operands with a float16 cotangent
 template <int HB, int EL>
 __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const BwdMfmaParams p) {
-  constexpr bool FP8 = EL == 1, F16 = EL == 2;
+  constexpr bool FP8 = EL == 1 || EL == 3, F16 = EL == 2 || EL == 3;
   // float16 planes of P and dS are kept at 16 times their value: a float16 is flushed below 6e-8 and overflows above
   // 65504, so entries down to 4e-9 survive and |dS| may reach 4000
   constexpr float kPlaneScale = F16 ? 16.0f : 1.0f, kPlaneUnscale = F16 ? 1.0f / 16.0f : 1.0f;
@@ -165,7 +174,10 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
       uint4 v = make_uint4(0u, 0u, 0u, 0u);
       if (h < nh) {
         const size_t at = (bs * p.H + h0 + h) * (size_t)D + c8 * 8;
-        if (FP8) v = e4m3x8_to_bf16(*reinterpret_cast<const uint2*>(static_cast<const unsigned char*>(p.q) + at));
+        if (FP8) {
+          const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const unsigned char*>(p.q) + at);
+          v = F16 ? e4m3x8_to_f16(raw) : e4m3x8_to_bf16(raw);
+        }
         else v = *reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(p.q) + at);
       }
       *reinterpret_cast<uint4*>(Qs + h * Dp + c8 * 8) = v;
@@ -219,7 +231,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_mla_bwd_mfma_kernel(const 
       if (pre_off[i] >= 0) {
         const int r = pre_off[i] >> 16, c8 = pre_off[i] & 0xffff;
         if (FP8) {
-          *reinterpret_cast<uint4*>(Ks + r * Dp + c8 * 8) = e4m3x8_to_bf16(make_uint2(pre[i].x, pre[i].y));
+          *reinterpret_cast<uint4*>(Ks + r * Dp + c8 * 8) = F16 ? e4m3x8_to_f16(make_uint2(pre[i].x, pre[i].y)) : e4m3x8_to_bf16(make_uint2(pre[i].x, pre[i].y));
           if (c8 == 0) ksc[r] = __uint_as_float(pre[i].z);
         } else {
           *reinterpret_cast<uint4*>(Ks + r * Dp + c8 * 8) = pre[i];
@@ -487,7 +499,11 @@ bool fp8_operands(const cppmega_mi355_sparse_mla_bwd_args_t& a) {
 bool sparse_mla_bwd_mfma_supports(const cppmega_mi355_sparse_mla_bwd_args_t& a) {
   const bool bf16 = a.q_dtype == CPPMEGA_MI355_BF16 && a.kv_dtype == CPPMEGA_MI355_BF16;
   const bool f16 = a.q_dtype == CPPMEGA_MI355_F16 && a.kv_dtype == CPPMEGA_MI355_F16;
-  if (f16 ? a.d_out_dtype != CPPMEGA_MI355_F16 : ((!bf16 && !fp8_operands(a)) || a.d_out_dtype != CPPMEGA_MI355_BF16)) return false;
+  if (fp8_operands(a)) {
+    if (a.d_out_dtype != CPPMEGA_MI355_BF16 && a.d_out_dtype != CPPMEGA_MI355_F16) return false;
+  } else if (f16 ? a.d_out_dtype != CPPMEGA_MI355_F16 : (!bf16 || a.d_out_dtype != CPPMEGA_MI355_BF16)) {
+    return false;
+  }
   if (a.d_qk % 32 != 0 || a.d_v % 32 != 0 || a.d_qk > kMaxBlk * 64 || a.topk < 1) return false;
   const int hg = a.heads / a.kv_groups;
   const int kt = hg > 16 ? 32 : 64;
@@ -513,9 +529,14 @@ int sparse_mla_bwd_mfma_launch(const cppmega_mi355_sparse_mla_bwd_args_t& a, hip
   if (grid == 0) return 0;
   if (grid > 0x7fffffffull) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_mla_bwd: too many (batch, query, head chunk) workgroups for one launch");
   const size_t lds = wide ? lds_bytes<2>(a.d_qk, a.d_v, p.ntiles, fp8) : lds_bytes<1>(a.d_qk, a.d_v, p.ntiles, fp8);
-  const bool f16 = a.q_dtype == CPPMEGA_MI355_F16;
-  const void* fn = wide ? (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<2, 1> : f16 ? (const void*)sparse_mla_bwd_mfma_kernel<2, 2> : (const void*)sparse_mla_bwd_mfma_kernel<2, 0>)
-                        : (fp8 ? (const void*)sparse_mla_bwd_mfma_kernel<1, 1> : f16 ? (const void*)sparse_mla_bwd_mfma_kernel<1, 2> : (const void*)sparse_mla_bwd_mfma_kernel<1, 0>);
+  const bool f16 = a.d_out_dtype == CPPMEGA_MI355_F16;     // the cotangent's carrier decides the arithmetic type
+  const int el = fp8 ? (f16 ? 3 : 1) : (f16 ? 2 : 0);
+  const void* fns[2][4] = {
+      {(const void*)sparse_mla_bwd_mfma_kernel<1, 0>, (const void*)sparse_mla_bwd_mfma_kernel<1, 1>, (const void*)sparse_mla_bwd_mfma_kernel<1, 2>,
+       (const void*)sparse_mla_bwd_mfma_kernel<1, 3>},
+      {(const void*)sparse_mla_bwd_mfma_kernel<2, 0>, (const void*)sparse_mla_bwd_mfma_kernel<2, 1>, (const void*)sparse_mla_bwd_mfma_kernel<2, 2>,
+       (const void*)sparse_mla_bwd_mfma_kernel<2, 3>}};
+  const void* fn = fns[wide ? 1 : 0][el];
   if (lds > 64 * 1024) CM_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   void* kargs[] = {(void*)&p};
   CM_HIP_CHECK(hipLaunchKernel(fn, dim3((unsigned)grid), dim3(kThreads), kargs, lds, stream));

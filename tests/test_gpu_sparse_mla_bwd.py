@@ -107,7 +107,8 @@ def test_bfloat16_backward_on_the_matrix_cores(device, shape, index_dtype, carri
     dict(B=1, S=2, H=48, G=1, Skv=300, topk=45, D=576, d_v=512),
     dict(B=1, S=3, H=16, G=1, Skv=200, topk=130, D=128, d_v=128),
 ], ids=lambda c: "B%dS%dH%dG%dT%dk%dD%ddv%d" % tuple(c.values()))
-def test_per_token_fp8_backward_on_the_matrix_cores(device, shape):
+@pytest.mark.parametrize("cotangent", [torch.bfloat16, torch.float16])
+def test_per_token_fp8_backward_on_the_matrix_cores(device, shape, cotangent):
     """e4m3 q / kv with per-token scales and a bfloat16 cotangent take the matrix-core kernel: the code
     values are exact in bfloat16 and the scales are applied in fp32, so the 1e-4 bar of the fp32 kernel holds."""
     from cppmega_mlx_amd.nn._tilelang import sparse_mla_fp8_path_c as f8
@@ -118,7 +119,7 @@ def test_per_token_fp8_backward_on_the_matrix_cores(device, shape):
     qc, qs = fp8.quantize_per_token((rng.standard_normal((B * S * H, D)) * rng.uniform(0.2, 3.0, (B * S * H, 1))).astype(np.float32))
     kc, ks = fp8.quantize_per_token((rng.standard_normal((B * Skv * G, D)) * rng.uniform(0.2, 3.0, (B * Skv * G, 1))).astype(np.float32))
     qc, qs, kc, ks = qc.reshape(B, S, H, D), qs.reshape(B, S, H), kc.reshape(B, Skv, G, D), ks.reshape(B, Skv, G)
-    d_out = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(torch.bfloat16)
+    d_out = to_dev(rng.standard_normal((B, S, H, d_v)).astype(np.float32), device).to(cotangent)
     idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
     idx[rng.random(idx.shape) < 0.15] = -1
     idx[0, 1] = -1
