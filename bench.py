@@ -400,6 +400,33 @@ def bench_prefill(args, device):
             "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
 
 
+def bench_prefill_rows(args, device):
+    """The same prefill on unquantised 16-bit rows of 576 (the carrier of the reference's float
+    Path C kernels, float16): the 32-head tile kernel with its four wavefronts sharing one key stream."""
+    from cppmega_mlx_amd import ops
+    from cppmega_mlx_amd.nn._tilelang import topk_selector as tk
+
+    S, H, topk = 8192, 128, 2048
+    gen = torch.Generator(device=device).manual_seed(556)
+    kv = torch.randn((1, S, 1, 576), generator=gen, device=device).to(torch.float16)
+    q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.float16)
+    idx_scores = torch.randn((S, S), generator=gen, device=device)
+    ends = torch.arange(1, S + 1, device=device, dtype=torch.int32)
+    idx = torch.empty((S, topk), dtype=torch.int32, device=device)
+    tk.topk_selector_tilelang_direct(idx_scores, topk, out=idx, ends=ends, order="index")
+    idx = idx.view(1, S, 1, topk)
+    out = torch.empty((1, S, H, 512), dtype=torch.float16, device=device)
+    lse = torch.empty((1, S, H), dtype=torch.float32, device=device)
+    fn = lambda: ops.sparse_mla_forward(q, kv, idx, sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse)
+    steps = max(1, min(args.steps, 5))
+    secs, _ = timed_graph([fn], steps, 1)
+    per = secs / steps
+    pairs = int(torch.minimum(ends.long(), torch.tensor(topk, device=device)).sum().item())
+    flops = 2.0 * H * pairs * (576 + 512)
+    return {"workload": "sparse_mla_prefill float16 rows B=1 S=8192 H=128 topk=2048 causal", "ms_per_step": per * 1e3,
+            "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+
+
 def bench_copy(args, device):
     """A plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     counters of the other kernels are scaled by."""
@@ -732,6 +759,7 @@ def main() -> int:
         torch.cuda.empty_cache()
     if "prefill" in parts:
         line["prefill"] = bench_prefill(args, device)
+        line["prefill_float_rows"] = bench_prefill_rows(args, device)
     if "copy" in parts:
         line["copy"] = bench_copy(args, device)
     if "next" in parts:

@@ -91,7 +91,7 @@ static int build_mla_params(const cppmega_mi355_sparse_mla_args_t& a, MlaParams&
   p.rope_dtype = a.rope_dtype; p.rope_dim = a.rope_dim; p.index_dtype = a.index_dtype; p.out_dtype = a.out_dtype;
   p.B = a.batch; p.S = a.seq_q; p.H = a.heads; p.G = a.kv_groups; p.Skv = a.seq_kv; p.topk = a.topk;
   p.d_qk = a.d_qk; p.d_kv = d_kv; p.d_v = a.d_v; p.heads_per_group = a.heads / a.kv_groups;
-  p.num_splits = 1; p.keys_per_split = a.topk; p.sm_scale = a.sm_scale;
+  p.num_splits = 1; p.keys_per_split = a.topk; p.heads_per_wg = 0; p.tile_sharing = 0; p.sm_scale = a.sm_scale;
   p.sm_scale_dev = a.sm_scale_dev; p.has_sinks_dev = a.has_sinks_dev;
   if (a.seq_kv_pitch != 0 && a.seq_kv_pitch < a.seq_kv)
     return fail(CPPMEGA_MI355_ERR_SHAPE, "sparse_mla: seq_kv_pitch %d is below seq_kv %d", a.seq_kv_pitch, a.seq_kv);

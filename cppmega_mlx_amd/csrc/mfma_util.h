@@ -26,6 +26,13 @@ __device__ __forceinline__ void mfma_qk(f32x4& acc, const bf16x8& a, const bf16x
 __device__ __forceinline__ void mfma_pv(f32x16& acc, const bf16x8& a, const bf16x8& b) {
   asm("s_nop 0\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
+// the same two shapes on float16 operands
+__device__ __forceinline__ void mfma_qk_f16(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  asm("s_nop 0\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_pv_f16(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  asm("s_nop 0\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
 // wait states between the last MFMA writing these registers and the first non-MFMA use
 __device__ __forceinline__ void mfma_settle(f32x4& s0, f32x4& s1) {
   asm volatile("s_nop 15\n\ts_nop 3" : "+v"(s0), "+v"(s1));
@@ -42,6 +49,14 @@ __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
   v2 r;
   r[0] = (__bf16)a;
   r[1] = (__bf16)b;
+  return __builtin_bit_cast(unsigned, r);
+}
+
+__device__ __forceinline__ unsigned pack_f16(float a, float b) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 r;
+  r[0] = (_Float16)a;
+  r[1] = (_Float16)b;
   return __builtin_bit_cast(unsigned, r);
 }
 

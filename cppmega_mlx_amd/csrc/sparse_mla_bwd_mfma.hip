@@ -102,13 +102,6 @@ __device__ __forceinline__ f32x4 mm(const bf16x8 a, const bf16x8 b, const f32x4 
   if (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8b, a), __builtin_bit_cast(f16x8b, b), c, 0, 0, 0);
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
-__device__ __forceinline__ unsigned pack_f16(float a, float b) {
-  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-  h2 r;
-  r[0] = (_Float16)a;
-  r[1] = (_Float16)b;
-  return __builtin_bit_cast(unsigned, r);
-}
 __device__ __forceinline__ bf16x8 zero8() {
   return __builtin_bit_cast(bf16x8, make_uint4(0u, 0u, 0u, 0u));
 }

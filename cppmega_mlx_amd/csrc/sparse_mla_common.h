@@ -27,6 +27,7 @@ struct MlaParams {
   int num_splits;       // split-KV factor of the MFMA kernel
   int keys_per_split;
   int heads_per_wg;     // 0: 32-head tile kernel; 64: shared-tile latent kernel (sparse_mla_latent.hip)
+  int tile_sharing;     // tile kernel on 16-bit rows: the 4 wavefronts take 4 head groups over one key stream
   float sm_scale;
   const float* sm_scale_dev;     // device copy of the softmax scale; read in place of sm_scale when set
   const int* has_sinks_dev;      // device flag; sinks are ignored when it is set and holds 0

@@ -217,6 +217,42 @@ def test_mfma_kernel_matches_scalar_kernel_bf16_cache(device):
         _assert_close(out, lse, want_out, want_lse, lse_tol=LSE_TOL if kernel == "scalar" else LSE_TOL_MFMA)
 
 
+@pytest.mark.parametrize("shape", [
+    dict(B=1, S=4, H=16, G=1, Skv=256, topk=64),
+    dict(B=2, S=3, H=40, G=1, Skv=700, topk=333),             # a partial head group, ragged tiles
+    dict(B=1, S=2, H=64, G=2, Skv=5000, topk=2048),           # two KV groups, key splits + combine
+    dict(B=1, S=3, H=128, G=1, Skv=3000, topk=1000),          # 4 head groups share one key stream
+    dict(B=2, S=2, H=144, G=2, Skv=900, topk=130),            # 72 heads per KV group: 32 + 32 + 8, a wavefront without heads
+    dict(B=1, S=2, H=160, G=1, Skv=9000, topk=4096),          # 5 head groups: two workgroups per query, key splits
+    dict(B=1, S=2, H=64, G=1, Skv=100, topk=7),               # less than one tile
+], ids=["h16", "h40_ragged", "g2_splits", "h128_shared", "h144_g2_shared", "h160_shared_splits", "h64_tiny"])
+@pytest.mark.parametrize("rope_tail", [False, True], ids=["packed576", "latent_plus_rope"])
+def test_mfma_kernel_float16_rows(device, shape, rope_tail):
+    """float16 queries and rows of 576 (the carrier the reference's float Path C kernels compute in,
+    cppmega_mlx/nn/_tilelang/sparse_mla_path_c.py) on the float16 matrix instructions."""
+    rng = np.random.default_rng(shape["H"] * 7 + shape["topk"] + rope_tail)
+    B, S, H, G, Skv, topk = (shape[k] for k in ("B", "S", "H", "G", "Skv", "topk"))
+    q = to_dev(rng.standard_normal((B, S, H, 576)).astype(np.float32), device).to(torch.float16)
+    kv = to_dev(rng.standard_normal((B, Skv, G, 576)).astype(np.float32), device).to(torch.float16)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[rng.random(idx.shape) < 0.15] = -1
+    idx[0, 1] = -1
+    want_out, want_lse = om.sparse_mla_oracle(q.float().cpu().numpy(), kv.float().cpu().numpy(), idx,
+                                              sm_scale=576 ** -0.5, d_v=512)
+    kw = {}
+    rows = kv
+    if rope_tail:
+        rows = kv[..., :512].contiguous()
+        kw["kv_rope"] = kv[..., 512:].contiguous()
+    out = torch.zeros((B, S, H, 512), dtype=torch.float16, device=device)
+    lse = torch.zeros((B, S, H), dtype=torch.float32, device=device)
+    ops.sparse_mla_forward(q, rows, to_dev(idx.astype(np.int32), device), sm_scale=576 ** -0.5, d_v=512, out=out,
+                           lse=lse, kernel="mfma", **kw)
+    torch.cuda.synchronize()
+    _assert_close(out, lse, want_out, want_lse, lse_tol=LSE_TOL_MFMA)
+    assert (out[0, 1] == 0).all() and (lse[0, 1] == 0).all()
+
+
 @pytest.mark.parametrize("pow2", [True, False], ids=["pow2_scales", "general_scales"])
 def test_decode_full_config_sampled_batches(device, pow2):
     """B=32, S_q=1, H=128, topk=2048 over a 65536-token FP8 cache (the headline
