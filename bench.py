@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode,vecmat,topk,prefill]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode,vecmat,topk,prefill,prefill_rows,copy,next]
 
 Prints ONE JSON line.  The headline (`metric`/`value`) is sparse-MLA decode
 throughput on the B=32, H=128, topk=2048, 64K-token FP8 latent-cache
@@ -558,11 +558,11 @@ def measured_traffic(name):
 # profiles/traffic.json.  Each is run from /tmp (`cd /tmp && export TMPDIR=/tmp`) with DIR as below.
 PROFILE_RUNS = {
     "prof_all": "rocprofv3 --kernel-trace --stats --output-format csv -d DIR/prof_all -o all -- python3 bench.py "
-                "--only decode,vecmat,topk,copy,next --steps 20 --no-cpu-baseline",
+                "--only decode,vecmat,topk,copy,next,prefill_rows --steps 20 --no-cpu-baseline",
     "pmc_fetch": "rocprofv3 --pmc FETCH_SIZE --output-format csv -d DIR/pmc_fetch -o f -- python3 bench.py "
-                 "--only decode,vecmat,topk,copy,next --steps 3 --warmup 1 --no-cpu-baseline",
+                 "--only decode,vecmat,topk,copy,next,prefill_rows --steps 3 --warmup 1 --no-cpu-baseline",
     "pmc_write": "rocprofv3 --pmc WRITE_SIZE --output-format csv -d DIR/pmc_write -o w -- python3 bench.py "
-                 "--only decode,vecmat,topk,copy,next --steps 3 --warmup 1 --no-cpu-baseline",
+                 "--only decode,vecmat,topk,copy,next,prefill_rows --steps 3 --warmup 1 --no-cpu-baseline",
     "pmc_sq": "rocprofv3 --pmc SQ_WAVE_CYCLES SQ_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES "
               "SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY SQ_ACTIVE_INST_LDS --output-format csv -d DIR/pmc_sq -o s -- python3 bench.py "
               "--only decode --steps 3 --warmup 1 --no-cpu-baseline",
@@ -591,6 +591,9 @@ PROFILE_WORKLOADS = [
     ("kv_cache_append", ("cache_append_kernel",),
      "bf16 latent[B,S,1,512] + rope[..,64] -> e4m3 + fp32/128 scales + bf16 rope in the cache: one dispatch of 8192 rows "
      "(prefill chunk) and one of 32 rows (decode step) per step"),
+    ("sparse_mla_prefill_float16_rows", ("sparse_mla_mfma_kernel<false, true, true>",),
+     "sparse_mla_fwd q f16[1,8192,128,576], kv f16[1,8192,1,576] (unquantised rows), causal top-2048 indices -> f16[1,8192,128,512]: "
+     "the 32-head tile kernel, four wavefronts sharing one key stream"),
     ("sparse_mla_backward", ("sparse_mla_bwd", "fill_zero_kernel"),
      "sparse_mla_bwd q bf16[1,1024,16,576], kv bf16[1,4096,1,576], d_out bf16[1,1024,16,512], topk 256 -> dq bf16, dkv f32 "
      "(the dkv clear, then the matrix-core kernel with its float32 atomic adds)"),
@@ -759,6 +762,7 @@ def main() -> int:
         torch.cuda.empty_cache()
     if "prefill" in parts:
         line["prefill"] = bench_prefill(args, device)
+    if "prefill" in parts or "prefill_rows" in parts:
         line["prefill_float_rows"] = bench_prefill_rows(args, device)
     if "copy" in parts:
         line["copy"] = bench_copy(args, device)

@@ -87,7 +87,11 @@ __device__ __forceinline__ bf16x4 lds_read_tr16_b64(const unsigned char* addr) {
 // SHARE (16-bit rows, more than 32 heads per KV group): the 4 wavefronts take 4 groups of 32
 // heads and walk the same keys - every wavefront fetches one tile of a round of 4 and all compute
 // on all 4, so a gathered row is read from the cache once per 128 heads instead of once per 32.
-template <bool KV_FP8, bool F16 = false, bool SHARE = false>
+// TOK (with KV_FP8): rows of 576 e4m3 codes with one fp32 scale per row and e4m3 queries with one
+// fp32 scale per (query, head) - the prepared buffers of cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py.
+// Codes become bfloat16 exactly; the two scales multiply the scores (and the key's scale its
+// probability on the way into P.V), so no operand is rounded.
+template <bool KV_FP8, bool F16 = false, bool SHARE = false, bool TOK = false>
 __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const MlaParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -122,10 +126,20 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       const int h = hh * 16 + n;
       const bool live = h < heads_here;
       const unsigned short* qrow = (const unsigned short*)p.q + (bs * p.H + head0 + (live ? h : 0)) * (size_t)kDqk;
+      const unsigned char* qcodes = (const unsigned char*)p.q + (bs * p.H + head0 + (live ? h : 0)) * (size_t)kDqk;
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
         uint4 t = make_uint4(0, 0, 0, 0);
-        if (live) t = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * kq);
+        if (TOK) {
+          uint2 c = make_uint2(0, 0);
+          if (live) c = *reinterpret_cast<const uint2*>(qcodes + 32 * ks + 8 * kq);
+          t.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.x, 1.0f, false));
+          t.y = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.x, 1.0f, true));
+          t.z = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.y, 1.0f, false));
+          t.w = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.y, 1.0f, true));
+        } else if (live) {
+          t = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * kq);
+        }
         qf[hh][ks] = __builtin_bit_cast(bf16x8, t);
       }
     }
@@ -139,6 +153,14 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   float m_run[2] = {-INFINITY, -INFINITY};   // base-2 running reference of heads (lane%16) and 16+(lane%16)
   float l_run[2] = {0.0f, 0.0f};             // this lane's share of the denominators
   const float qk_scale = mla_sm_scale(p) * kLog2e;
+  float sfac[2] = {qk_scale, qk_scale};      // what a raw score of heads (lane%16), 16+(lane%16) is multiplied with
+  if (TOK) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int h = hh * 16 + (lane & 15);
+      sfac[hh] = h < heads_here ? qk_scale * ((const float*)p.q_scale)[bs * p.H + head0 + h] : 0.0f;
+    }
+  }
 
   // ---- staging ---------------------------------------------------------------------
   // The gathered rows travel HBM -> LDS by the load unit itself (no registers are held
@@ -174,12 +196,20 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     for (int it = 0; it < 8; ++it) {
       if (rows[it] >= 0) {
         const size_t krow = (row_base + (size_t)rows[it]) * p.G + g;
-        const unsigned char* src = (const unsigned char*)p.kv + krow * kLat + (lane & 31) * 16;
+        const unsigned char* src = (const unsigned char*)p.kv + krow * (TOK ? kDqk : kLat) + (lane & 31) * 16;
         __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_lat + it * 1024), 16, 0, 0);
       }
     }
+    if (TOK) {                                    // the last 64 codes of all 16 rows: 4 lanes x 16 bytes each
+      const int r = __shfl(keyv, lane >> 2, 64);
+      if (r >= 0) {
+        const size_t krow = (row_base + (size_t)r) * p.G + g;
+        const unsigned char* src = (const unsigned char*)p.kv + krow * kDqk + kLat + (lane & 3) * 16;
+        __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)raw_rope, 16, 0, 0);
+      }
+    }
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
+    for (int it = 0; it < (TOK ? 0 : 2); ++it) {
       const int r = it ? rope_r1 : rope_r0;
       if (r >= 0) {
         const size_t krow = (row_base + (size_t)r) * p.G + g;
@@ -212,7 +242,8 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       for (int i = 0; i < 4; ++i) {
         const int it = half * 4 + i;
         raw[i] = *reinterpret_cast<const uint4*>(raw_lat + it * 1024 + lane * 16);
-        sc[i] = has_scale ? *reinterpret_cast<const float*>(raw_sc + ((2 * it + hi_row) * nblk + blk) * 4) : 1.0f;
+        // (TOK: the row's scale goes onto its score and its probability instead)
+        sc[i] = has_scale && !TOK ? *reinterpret_cast<const float*>(raw_sc + ((2 * it + hi_row) * nblk + blk) * 4) : 1.0f;
         all_pow2 = all_pow2 && scale_is_pow2(sc[i]);
       }
       const bool fast = __ballot(!all_pow2) == 0ull;      // uniform
@@ -226,8 +257,15 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c + 1, r) * 16) = hi;
       }
     }
+    if (TOK) {
+      const int r = lane >> 2, c = lane & 3;
+      uint4 lo, hi;
+      dequant16<true>(*reinterpret_cast<const uint4*>(raw_rope + lane * 16), 1.0f, lo, hi);
+      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + 2 * c, r) * 16) = lo;
+      *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + 2 * c + 1, r) * 16) = hi;
+    }
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
+    for (int it = 0; it < (TOK ? 0 : 2); ++it) {
       const int r = 8 * it + (lane >> 3);
       const uint4 v = *reinterpret_cast<const uint4*>(raw_rope + it * 1024 + lane * 16);
       *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + (lane & 7), r) * 16) = v;
@@ -369,6 +407,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   const int steps = SHARE ? rounds * kWaves : my_tiles;
   for (int t = 0; t < steps; ++t) {
     unsigned vmask;
+    f32x4 ksc = {1.0f, 1.0f, 1.0f, 1.0f};
     if (SHARE) {
       const int r = t >> 2, j = t & 3;
       if (j == 0) {
@@ -394,6 +433,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     if (KV_FP8) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // tile t has landed in the raw area
       stage();
+      if (TOK) ksc = *reinterpret_cast<const f32x4*>(raw_sc + 16 * (lane >> 4));   // scales of keys 4 (lane / 16) + i
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // raw area fully read before it is refilled
       if (t + 1 < my_tiles) issue_dma(key_nxt);
     } else {
@@ -432,8 +472,8 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool ok = (vmask >> (4 * gq + i)) & 1u;
-      sv[0][i] = ok ? s0[i] * qk_scale : -INFINITY;
-      sv[1][i] = ok ? s1[i] * qk_scale : -INFINITY;
+      sv[0][i] = ok ? s0[i] * (TOK ? sfac[0] * ksc[i] : qk_scale) : -INFINITY;
+      sv[1][i] = ok ? s1[i] * (TOK ? sfac[1] * ksc[i] : qk_scale) : -INFINITY;
       mx[0] = fmaxf(mx[0], sv[0][i]);
       mx[1] = fmaxf(mx[1], sv[1][i]);
     }
@@ -478,6 +518,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       for (int i = 0; i < 4; ++i) {
         pr[i] = exp2f(sv[hh][i] - m_run[hh]);      // -inf -> 0; m_run is finite once any key was valid
         l_run[hh] += pr[i];
+        if (TOK) pr[i] *= ksc[i];                  // V = scale x codes
       }
       pk[hh][0] = F16 ? pack_f16(pr[0], pr[1]) : pack_bf16(pr[0], pr[1]);
       pk[hh][1] = F16 ? pack_f16(pr[2], pr[3]) : pack_bf16(pr[2], pr[3]);
@@ -689,6 +730,12 @@ __global__ __launch_bounds__(256) void sparse_mla_combine_kernel(const MlaParams
 
 bool sparse_mla_mfma_supported(const MlaParams& p) {
   if (sparse_mla_latent_supported(p)) return true;
+  if (p.q_dtype == CPPMEGA_MI355_E4M3) {          // per-token FP8 prepared buffers: rows of 576 codes
+    return p.q_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN && p.kv_dtype == CPPMEGA_MI355_E4M3 &&
+           p.kv_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN && p.d_qk == kDqk && p.d_kv == kDqk && p.d_v == kLat &&
+           p.rope_dim == 0 && p.q_scale && p.kv_scale && p.topk >= 1 && (size_t)p.B * p.S != 0 &&
+           (((uintptr_t)p.q | (uintptr_t)p.kv) & 15) == 0 && (((uintptr_t)p.q_scale | (uintptr_t)p.kv_scale) & 3) == 0;
+  }
   const bool f16 = p.q_dtype == CPPMEGA_MI355_F16;
   if ((p.q_dtype != CPPMEGA_MI355_BF16 && !f16) || p.q_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
   if (p.d_qk != kDqk || p.d_v != kLat) return false;
@@ -751,7 +798,7 @@ int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
   void (*kernel)(MlaParams) = nullptr;
   int smem = kRowsSmemBytes;
   if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
-    kernel = sparse_mla_mfma_kernel<true>;
+    kernel = p.q_dtype == CPPMEGA_MI355_E4M3 ? sparse_mla_mfma_kernel<true, false, false, true> : sparse_mla_mfma_kernel<true>;
     smem = kSmemBytes;
   } else if (p.kv_dtype == CPPMEGA_MI355_F16) {
     kernel = p.tile_sharing ? sparse_mla_mfma_kernel<false, true, true> : sparse_mla_mfma_kernel<false, true, false>;

@@ -142,6 +142,43 @@ def test_per_token_fp8_prepared_buffers_with_sinks(device, with_sinks, out_dtype
         np.testing.assert_allclose(lse[0, 2].cpu().numpy(), sinks, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [
+    dict(B=1, S=4, H=16, G=1, Skv=256, topk=64),
+    dict(B=2, S=3, H=40, G=1, Skv=700, topk=333),             # a partial head group, ragged tiles
+    dict(B=1, S=2, H=64, G=2, Skv=5000, topk=2048),           # two KV groups, key splits + combine
+    dict(B=1, S=3, H=128, G=1, Skv=3000, topk=1000),
+    dict(B=1, S=2, H=64, G=1, Skv=100, topk=7),               # less than one tile
+], ids=["h16", "h40_ragged", "g2_splits", "h128", "h64_tiny"])
+@pytest.mark.parametrize("with_sinks", [False, True], ids=["plain", "sinks"])
+def test_mfma_kernel_per_token_fp8_rows(device, shape, with_sinks):
+    """Per-token FP8 prepared buffers at the attention shape (rows of 576 codes, d_v 512; reference:
+    cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py:1701-3004) on the matrix cores: codes enter the
+    products exactly, the scales multiply the scores, so the result is held to the fp32 kernel's lse bound."""
+    rng = np.random.default_rng(shape["H"] * 11 + shape["topk"] + with_sinks)
+    B, S, H, G, Skv, topk = (shape[k] for k in ("B", "S", "H", "G", "Skv", "topk"))
+    qc, qs = fp8.quantize_per_token(rng.standard_normal((B, S, H, 576)).astype(np.float32) * 3.0)
+    kc, ks = fp8.quantize_per_token(rng.standard_normal((B, Skv, G, 576)).astype(np.float32) * 0.5)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[rng.random(idx.shape) < 0.15] = -1
+    idx[0, 1] = -1
+    sinks = rng.standard_normal(H).astype(np.float32) if with_sinks else None
+    want_out, want_lse = om.sparse_mla_oracle(om.dequant_per_token(qc, qs), om.dequant_per_token(kc, ks), idx,
+                                              sm_scale=576 ** -0.5, d_v=512, sinks=sinks)
+    out = torch.zeros((B, S, H, 512), dtype=torch.bfloat16, device=device)
+    lse = torch.zeros((B, S, H), dtype=torch.float32, device=device)
+    got = f8.sparse_mla_fp8_path_c_apply_direct(
+        to_dev(qc, device), to_dev(qs, device), to_dev(kc, device), to_dev(ks, device), to_dev(idx.astype(np.int32), device),
+        sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse, sinks=None if sinks is None else to_dev(sinks, device), kernel="mfma")
+    torch.cuda.synchronize()
+    assert got[0] is out and got[1] is lse
+    _assert_close(out, lse, want_out, want_lse, lse_tol=LSE_TOL)
+    if with_sinks:
+        assert (out[0, 1] == 0).all()
+        np.testing.assert_allclose(lse[0, 1].cpu().numpy(), sinks, atol=1e-6)
+    else:
+        assert (out[0, 1] == 0).all() and (lse[0, 1] == 0).all()
+
+
 def _latent_case(device, rng, *, B, S, H, Skv, topk, pow2, causal_offset=None, d_latent=512, d_rope=64):
     q, qf = bf16_pair(rng.standard_normal((B, S, H, d_latent + d_rope)), device)
     codes, scale, rope, rows = latent_cache(rng, B, Skv, 1, d_latent, d_rope, device, pow2=pow2)
