@@ -87,11 +87,14 @@ __device__ __forceinline__ bf16x4 lds_read_tr16_b64(const unsigned char* addr) {
 // SHARE (16-bit rows, more than 32 heads per KV group): the 4 wavefronts take 4 groups of 32
 // heads and walk the same keys - every wavefront fetches one tile of a round of 4 and all compute
 // on all 4, so a gathered row is read from the cache once per 128 heads instead of once per 32.
-// TOK (with KV_FP8): rows of 576 e4m3 codes with one fp32 scale per row and e4m3 queries with one
-// fp32 scale per (query, head) - the prepared buffers of cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py.
-// Codes become bfloat16 exactly; the two scales multiply the scores (and the key's scale its
-// probability on the way into P.V), so no operand is rounded.
-template <bool KV_FP8, bool F16 = false, bool SHARE = false, bool TOK = false>
+// ROWS (with KV_FP8): key rows of 576 e4m3 codes and e4m3 queries, the prepared buffers of
+//   1: cppmega_mlx/nn/_tilelang/sparse_mla_fp8_path_c.py - one fp32 scale per row and per (query,
+//      head).  Codes become bfloat16 exactly; the two scales multiply the scores (and the key's
+//      scale its probability on the way into P.V), so no operand is rounded;
+//   2: cppmega_mlx/nn/_tilelang/sparse_mla_blockscaled_path_c.py - one E8M0 byte per 32 channels
+//      on both sides.  A power of two times an e4m3 code is a bfloat16, so the scaled values enter
+//      the products exactly as well.
+template <bool KV_FP8, bool F16 = false, bool SHARE = false, int ROWS = 0>
 __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const MlaParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -99,6 +102,8 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   unsigned char* raw_lat = tile + kTileBytes;
   unsigned char* raw_rope = raw_lat + kRawLat;
   unsigned char* raw_sc = raw_rope + kRawRope;
+  constexpr bool TOK = ROWS == 1, E8 = ROWS == 2, R576 = ROWS != 0;
+  constexpr int kE8Row = kDqk / 32;              // 18 scale bytes per row
 
   // ---- which (query, head group, split) ------------------------------------
   const int groups_per_kv = (p.heads_per_group + kHeads - 1) / kHeads;
@@ -130,7 +135,17 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
         uint4 t = make_uint4(0, 0, 0, 0);
-        if (TOK) {
+        if (E8) {
+          uint2 c = make_uint2(0, 0);
+          float sc = 0.0f;
+          if (live) {
+            c = *reinterpret_cast<const uint2*>(qcodes + 32 * ks + 8 * kq);
+            sc = e8m0_to_f32(((const unsigned char*)p.q_scale)[(bs * p.H + head0 + h) * (size_t)kE8Row + ks]);
+          }
+          const f32x2 v0 = e4m3x2_lo(c.x), v1 = e4m3x2_hi(c.x), v2 = e4m3x2_lo(c.y), v3 = e4m3x2_hi(c.y);
+          t = make_uint4(pack_bf16(v0[0] * sc, v0[1] * sc), pack_bf16(v1[0] * sc, v1[1] * sc),
+                         pack_bf16(v2[0] * sc, v2[1] * sc), pack_bf16(v3[0] * sc, v3[1] * sc));
+        } else if (TOK) {
           uint2 c = make_uint2(0, 0);
           if (live) c = *reinterpret_cast<const uint2*>(qcodes + 32 * ks + 8 * kq);
           t.x = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(c.x, 1.0f, false));
@@ -182,6 +197,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   auto tile_key = [&](int t) -> int {            // lane l reports key (l % 16) of tile t
     return t < my_tiles ? key_row(key_begin + (t * kWaves + wave) * kTile + (lane & 15)) : -1;
   };
+  unsigned short e8n[3] = {0, 0, 0};              // E8: scale bytes of the tile in flight
   auto issue_dma = [&](int keyv) {                // keyv: this lane's tile_key() of the tile to fetch
     const bool upper = lane >= 32;
     int rows[8];
@@ -196,11 +212,11 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     for (int it = 0; it < 8; ++it) {
       if (rows[it] >= 0) {
         const size_t krow = (row_base + (size_t)rows[it]) * p.G + g;
-        const unsigned char* src = (const unsigned char*)p.kv + krow * (TOK ? kDqk : kLat) + (lane & 31) * 16;
+        const unsigned char* src = (const unsigned char*)p.kv + krow * (R576 ? kDqk : kLat) + (lane & 31) * 16;
         __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_lat + it * 1024), 16, 0, 0);
       }
     }
-    if (TOK) {                                    // the last 64 codes of all 16 rows: 4 lanes x 16 bytes each
+    if (R576) {                                   // the last 64 codes of all 16 rows: 4 lanes x 16 bytes each
       const int r = __shfl(keyv, lane >> 2, 64);
       if (r >= 0) {
         const size_t krow = (row_base + (size_t)r) * p.G + g;
@@ -209,7 +225,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       }
     }
 #pragma unroll
-    for (int it = 0; it < (TOK ? 0 : 2); ++it) {
+    for (int it = 0; it < (R576 ? 0 : 2); ++it) {
       const int r = it ? rope_r1 : rope_r0;
       if (r >= 0) {
         const size_t krow = (row_base + (size_t)r) * p.G + g;
@@ -217,7 +233,20 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(raw_rope + it * 1024), 16, 0, 0);
       }
     }
-    if (has_scale) {
+    if (E8) {
+      // 16 rows x 18 scale bytes as 144 two-byte pieces (a row's bytes start on an even address
+      // only), through registers: written to the raw area when the tile is staged
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        const int P = lane + 64 * i;
+        const int r = __shfl(keyv, (P / 9) & 15, 64);
+        e8n[i] = 0;
+        if (P < kTile * 9 && r >= 0) {
+          const size_t krow = (row_base + (size_t)r) * p.G + g;
+          e8n[i] = *reinterpret_cast<const unsigned short*>((const unsigned char*)p.kv_scale + krow * kE8Row + (P % 9) * 2);
+        }
+      }
+    } else if (has_scale) {
       for (int e0 = 0; e0 < kTile * nblk; e0 += 64) {   // uniform trip count (1 or 2)
         const int e = e0 + lane;
         const int r = __shfl(keyv, (e / nblk) & 15, 64);
@@ -243,7 +272,8 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         const int it = half * 4 + i;
         raw[i] = *reinterpret_cast<const uint4*>(raw_lat + it * 1024 + lane * 16);
         // (TOK: the row's scale goes onto its score and its probability instead)
-        sc[i] = has_scale && !TOK ? *reinterpret_cast<const float*>(raw_sc + ((2 * it + hi_row) * nblk + blk) * 4) : 1.0f;
+        if (E8) sc[i] = e8m0_to_f32(raw_sc[(2 * it + hi_row) * kE8Row + (c >> 1)]);
+        else sc[i] = has_scale && !TOK ? *reinterpret_cast<const float*>(raw_sc + ((2 * it + hi_row) * nblk + blk) * 4) : 1.0f;
         all_pow2 = all_pow2 && scale_is_pow2(sc[i]);
       }
       const bool fast = __ballot(!all_pow2) == 0ull;      // uniform
@@ -257,15 +287,18 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(2 * c + 1, r) * 16) = hi;
       }
     }
-    if (TOK) {
+    if (R576) {
       const int r = lane >> 2, c = lane & 3;
+      const uint4 raw = *reinterpret_cast<const uint4*>(raw_rope + lane * 16);
+      const float sc = E8 ? e8m0_to_f32(raw_sc[r * kE8Row + 16 + (c >> 1)]) : 1.0f;
       uint4 lo, hi;
-      dequant16<true>(*reinterpret_cast<const uint4*>(raw_rope + lane * 16), 1.0f, lo, hi);
+      if (__ballot(!scale_is_pow2(sc)) == 0ull) dequant16<true>(raw, sc, lo, hi);
+      else dequant16<false>(raw, sc, lo, hi);
       *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + 2 * c, r) * 16) = lo;
       *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + 2 * c + 1, r) * 16) = hi;
     }
 #pragma unroll
-    for (int it = 0; it < (TOK ? 0 : 2); ++it) {
+    for (int it = 0; it < (R576 ? 0 : 2); ++it) {
       const int r = 8 * it + (lane >> 3);
       const uint4 v = *reinterpret_cast<const uint4*>(raw_rope + it * 1024 + lane * 16);
       *reinterpret_cast<uint4*>(tile + r * kRowBytes + swz(64 + (lane & 7), r) * 16) = v;
@@ -432,6 +465,11 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     vmask = (unsigned)(__ballot(key_cur >= 0) & 0xffffull);
     if (KV_FP8) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // tile t has landed in the raw area
+      if (E8) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+          if (lane + 64 * i < kTile * 9) *reinterpret_cast<unsigned short*>(raw_sc + (lane + 64 * i) * 2) = e8n[i];
+      }
       stage();
       if (TOK) ksc = *reinterpret_cast<const f32x4*>(raw_sc + 16 * (lane >> 4));   // scales of keys 4 (lane / 16) + i
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // raw area fully read before it is refilled
@@ -730,11 +768,14 @@ __global__ __launch_bounds__(256) void sparse_mla_combine_kernel(const MlaParams
 
 bool sparse_mla_mfma_supported(const MlaParams& p) {
   if (sparse_mla_latent_supported(p)) return true;
-  if (p.q_dtype == CPPMEGA_MI355_E4M3) {          // per-token FP8 prepared buffers: rows of 576 codes
-    return p.q_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN && p.kv_dtype == CPPMEGA_MI355_E4M3 &&
-           p.kv_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN && p.d_qk == kDqk && p.d_kv == kDqk && p.d_v == kLat &&
+  if (p.q_dtype == CPPMEGA_MI355_E4M3) {          // FP8 prepared buffers: rows of 576 codes, both sides scaled alike
+    const bool tok = p.q_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN && p.kv_scale_kind == CPPMEGA_MI355_SCALE_PER_TOKEN &&
+                     (((uintptr_t)p.q_scale | (uintptr_t)p.kv_scale) & 3) == 0;
+    const bool e8 = p.q_scale_kind == CPPMEGA_MI355_SCALE_E8M0 && p.kv_scale_kind == CPPMEGA_MI355_SCALE_E8M0 &&
+                    p.q_scale_block == 32 && p.kv_scale_block == 32 && ((uintptr_t)p.kv_scale & 1) == 0;
+    return (tok || e8) && p.kv_dtype == CPPMEGA_MI355_E4M3 && p.d_qk == kDqk && p.d_kv == kDqk && p.d_v == kLat &&
            p.rope_dim == 0 && p.q_scale && p.kv_scale && p.topk >= 1 && (size_t)p.B * p.S != 0 &&
-           (((uintptr_t)p.q | (uintptr_t)p.kv) & 15) == 0 && (((uintptr_t)p.q_scale | (uintptr_t)p.kv_scale) & 3) == 0;
+           (((uintptr_t)p.q | (uintptr_t)p.kv) & 15) == 0;
   }
   const bool f16 = p.q_dtype == CPPMEGA_MI355_F16;
   if ((p.q_dtype != CPPMEGA_MI355_BF16 && !f16) || p.q_scale_kind != CPPMEGA_MI355_SCALE_NONE) return false;
@@ -798,7 +839,9 @@ int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
   void (*kernel)(MlaParams) = nullptr;
   int smem = kRowsSmemBytes;
   if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
-    kernel = p.q_dtype == CPPMEGA_MI355_E4M3 ? sparse_mla_mfma_kernel<true, false, false, true> : sparse_mla_mfma_kernel<true>;
+    kernel = p.q_dtype != CPPMEGA_MI355_E4M3 ? sparse_mla_mfma_kernel<true>
+             : p.q_scale_kind == CPPMEGA_MI355_SCALE_E8M0 ? sparse_mla_mfma_kernel<true, false, false, 2>
+                                                          : sparse_mla_mfma_kernel<true, false, false, 1>;
     smem = kSmemBytes;
   } else if (p.kv_dtype == CPPMEGA_MI355_F16) {
     kernel = p.tile_sharing ? sparse_mla_mfma_kernel<false, true, true> : sparse_mla_mfma_kernel<false, true, false>;

@@ -179,6 +179,40 @@ def test_mfma_kernel_per_token_fp8_rows(device, shape, with_sinks):
         assert (out[0, 1] == 0).all() and (lse[0, 1] == 0).all()
 
 
+@pytest.mark.parametrize("shape", [
+    dict(B=1, S=4, H=16, G=1, Skv=255, topk=64),              # an odd number of rows: the last row's scale bytes end the buffer
+    dict(B=2, S=3, H=40, G=1, Skv=700, topk=333),
+    dict(B=1, S=2, H=64, G=2, Skv=5000, topk=2048),
+    dict(B=1, S=3, H=128, G=1, Skv=3000, topk=1000),
+], ids=["h16_odd_rows", "h40_ragged", "g2_splits", "h128"])
+def test_mfma_kernel_e8m0_rows(device, shape):
+    """E8M0-per-32 prepared buffers at the attention shape (rows of 576 codes + 18 scale bytes, d_v 512;
+    reference: cppmega_mlx/nn/_tilelang/sparse_mla_blockscaled_path_c.py:943-1504) on the matrix cores.
+    A power of two times an e4m3 code is a bfloat16: the operands enter the products exactly."""
+    rng = np.random.default_rng(shape["H"] * 13 + shape["topk"])
+    B, S, H, G, Skv, topk = (shape[k] for k in ("B", "S", "H", "G", "Skv", "topk"))
+    qc, qb = fp8.quantize_mxfp8(rng.standard_normal((B, S, H, 576)).astype(np.float32) * 2.0)
+    kc, kb = fp8.quantize_mxfp8(rng.standard_normal((B, Skv, G, 576)).astype(np.float32) *
+                                np.exp2(rng.integers(-6, 3, size=(B, Skv, G, 1))).astype(np.float32))
+    kb[0, 0, 0, 0] = 0                                               # E8M0 byte 0 decodes to 0
+    kb[0, 1, 0, 17] = 255                                            # ... and so does 255
+    idx = sparse_indices(rng, B, S, G, Skv, topk, replace=True)
+    idx[rng.random(idx.shape) < 0.15] = -1
+    idx[0, 1] = -1
+    idx[0, 0, 0, :4] = [0, 1, Skv - 1, Skv + 3]                      # the patched rows, the last row, one out of range
+    want_out, want_lse = om.sparse_mla_oracle(om.dequant_e8m0(qc, qb), om.dequant_e8m0(kc, kb), idx,
+                                              sm_scale=576 ** -0.5, d_v=512)
+    out = torch.zeros((B, S, H, 512), dtype=torch.bfloat16, device=device)
+    lse = torch.zeros((B, S, H), dtype=torch.float32, device=device)
+    got = bs.sparse_mla_blockscaled_path_c_apply_direct(
+        to_dev(qc, device), to_dev(qb, device), to_dev(kc, device), to_dev(kb, device), to_dev(idx.astype(np.int32), device),
+        sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse, kernel="mfma")
+    torch.cuda.synchronize()
+    assert got[0] is out and got[1] is lse
+    _assert_close(out, lse, want_out, want_lse, lse_tol=LSE_TOL)
+    assert (out[0, 1] == 0).all() and (lse[0, 1] == 0).all()
+
+
 def _latent_case(device, rng, *, B, S, H, Skv, topk, pow2, causal_offset=None, d_latent=512, d_rope=64):
     q, qf = bf16_pair(rng.standard_normal((B, S, H, d_latent + d_rope)), device)
     codes, scale, rope, rows = latent_cache(rng, B, Skv, 1, d_latent, d_rope, device, pow2=pow2)
