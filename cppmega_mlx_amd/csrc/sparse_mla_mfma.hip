@@ -59,7 +59,9 @@ static_assert(kWaves * kWaveBytes <= kXBytes, "the merge buffer reuses the tile 
 constexpr int kRowsWaveBytes = 2 * kTileBytes;                            // 36864 per wavefront
 constexpr int kRowsStatOff = kWaves * kRowsWaveBytes > kXBytes ? kWaves * kRowsWaveBytes : kXBytes;   // 147456
 constexpr int kRowsSmemBytes = kRowsStatOff + kWaves * kHeads * 2 * 4;   // 148480 of the 160 KB
-static_assert(kRowsSmemBytes <= 160 * 1024, "two 16-bit tiles per wavefront fit the LDS of a CU");
+constexpr int kRowsKscOff = kRowsSmemBytes;                              // shared FP8 rows: [2 rounds][64 keys] fp32 row scales
+constexpr int kRowsFp8SmemBytes = kRowsKscOff + 2 * kWaves * kTile * 4;  // 148992
+static_assert(kRowsFp8SmemBytes <= 160 * 1024, "two 16-bit tiles per wavefront fit the LDS of a CU");
 constexpr float kLazy = 8.0f;      // rescale when the running max grows by more than 2^8
 
 // 16-byte chunk q of row r lives at chunk (q with its low 3 bits xor f(r)):
@@ -98,7 +100,8 @@ template <bool KV_FP8, bool F16 = false, bool SHARE = false, int ROWS = 0>
 __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const MlaParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  unsigned char* tile = smem + wave * (KV_FP8 ? kWaveBytes : kRowsWaveBytes);
+  constexpr bool STAGED = KV_FP8 && !SHARE;      // rows arrive in a raw area and are converted from there
+  unsigned char* tile = smem + wave * (STAGED ? kWaveBytes : kRowsWaveBytes);
   unsigned char* raw_lat = tile + kTileBytes;
   unsigned char* raw_rope = raw_lat + kRawLat;
   unsigned char* raw_sc = raw_rope + kRawRope;
@@ -329,7 +332,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
     return (second ? rb : ra) >= 0 ? base + c * 8 : nullptr;
   };
   auto issue_rows = [&](int keyv, int first, unsigned char* dst) {
-#pragma unroll
+#pragma unroll 1
     for (int t = 0; t < kTileBytes / 1024; ++t) {
       const unsigned short* src = slot_source(keyv, first, t);
       if (src) __builtin_amdgcn_global_load_lds((glb_void*)src, (lds_void*)(dst + t * 1024), 16, 0, 0);
@@ -348,20 +351,52 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   // wavefronts fetching at four different points of the step 5.7 ms.  Clock stamps put ~1.7 k of
   // a step's 5.2 k clocks into the five loads (4.25 ms form) - a wavefront that is alone on its
   // SIMD issues in order and nothing hides what it spends there.
+  // FP8 rows of 576 codes in this mode: 9 loads per tile - load t < 8 carries the first 512 codes of
+  // rows 2t and 2t + 1 (32 lanes x 16 bytes each), load 8 the last 64 codes of all 16 rows (4 lanes
+  // each); the steps take loads 0-2, 3-4, 5-6, 7-8.  A lane's 16 codes become 16 bfloat16 (two
+  // 16-byte slots) on their way into the tile.  E8M0: the lane also fetches the scale byte of its
+  // 16 codes.  Per token: the 16 row scales go to a small array the four wavefronts read.
   typedef __attribute__((ext_vector_type(4))) unsigned u4;
+  constexpr int kLoads = R576 ? 9 : kTileBytes / 1024;     // per tile
+  constexpr int kPerStep = R576 ? 3 : 5;
   unsigned char* dma_dst = smem;                  // this wavefront's tile of the next round
+  float* ksc_dst = reinterpret_cast<float*>(smem + kRowsKscOff);   // ... and its 16 row scales
   bool dma_on = false;
   int key_dma = -1;                               // lane 16 * wave + r: cache row of key r of that tile
-  u4 stg[5];
+  u4 stg[kPerStep];
+  unsigned char stg_e8[kPerStep];
+  float stg_ksc = 0.0f;
+  auto share_load = [&](int j, int i) -> int {    // index of the i-th load of step j, or kLoads
+    if (!R576) return 5 * j + i;
+    return j == 0 ? i : (i < 2 ? 1 + 2 * j + i : kLoads);
+  };
   auto fetch_share = [&](int j) {
     const int first = 16 * __builtin_amdgcn_readfirstlane(wave);
     const size_t row_base = (size_t)b * p.Skv_pitch;
 #pragma unroll
-    for (int i = 0; i < 5; ++i) {
-      const int t = 5 * j + i;                    // uniform
+    for (int i = 0; i < kPerStep; ++i) {
+      const int t = share_load(j, i);             // uniform
       stg[i] = u4{0u, 0u, 0u, 0u};
-      if (!dma_on || t >= kTileBytes / 1024) continue;
-      if (t < kTile) {
+      stg_e8[i] = 0;
+      if (!dma_on || t >= kLoads) continue;
+      if (R576) {
+        int row, off, blk;
+        if (t < 8) {
+          const int ra = __builtin_amdgcn_readlane(key_dma, first + 2 * t), rb = __builtin_amdgcn_readlane(key_dma, first + 2 * t + 1);
+          row = lane < 32 ? ra : rb;
+          off = (lane & 31) * 16;
+          blk = (lane & 31) >> 1;
+        } else {
+          row = __shfl(key_dma, first + (lane >> 2), 64);
+          off = kLat + (lane & 3) * 16;
+          blk = 16 + ((lane & 3) >> 1);
+        }
+        if (row >= 0) {
+          const size_t krow = (row_base + (size_t)row) * p.G + g;
+          stg[i] = *reinterpret_cast<const u4*>((const unsigned char*)p.kv + krow * kDqk + off);
+          if (E8) stg_e8[i] = ((const unsigned char*)p.kv_scale)[krow * kE8Row + blk];
+        }
+      } else if (t < kTile) {
         const int row = __builtin_amdgcn_readlane(key_dma, first + t);
         if (row >= 0) {                           // uniform
           const size_t krow = (row_base + (size_t)row) * p.G + g;
@@ -379,19 +414,37 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         }
       }
     }
+    if (TOK && j == 0 && dma_on) {                // lane r < 16: the scale of the tile's key r
+      const int row = __shfl(key_dma, first + (lane & 15), 64);
+      stg_ksc = 0.0f;
+      if (row >= 0) stg_ksc = ((const float*)p.kv_scale)[(row_base + (size_t)row) * p.G + g];
+    }
   };
   auto store_share = [&](int j) {
 #pragma unroll
-    for (int i = 0; i < 5; ++i) {
-      const int t = 5 * j + i;
-      if (!dma_on || t >= kTileBytes / 1024) continue;
-      const int r = t < kTile ? t : 8 * (t - kTile) + (lane >> 3);
-      const int c = t < kTile ? lane : 64 + (lane & 7);
-      *reinterpret_cast<u4*>(dma_dst + r * kRowBytes + swz(c, r) * 16) = stg[i];
+    for (int i = 0; i < kPerStep; ++i) {
+      const int t = share_load(j, i);
+      if (!dma_on || t >= kLoads) continue;
+      if (R576) {
+        const int r = t < 8 ? 2 * t + (lane >> 5) : lane >> 2;
+        const int c = t < 8 ? 2 * (lane & 31) : 64 + 2 * (lane & 3);      // first of the two slots
+        const float sc = E8 ? e8m0_to_f32(stg_e8[i]) : 1.0f;
+        const uint4 raw = make_uint4(stg[i][0], stg[i][1], stg[i][2], stg[i][3]);
+        uint4 lo, hi;
+        if (__ballot(!scale_is_pow2(sc)) == 0ull) dequant16<true>(raw, sc, lo, hi);
+        else dequant16<false>(raw, sc, lo, hi);
+        *reinterpret_cast<uint4*>(dma_dst + r * kRowBytes + swz(c, r) * 16) = lo;
+        *reinterpret_cast<uint4*>(dma_dst + r * kRowBytes + swz(c + 1, r) * 16) = hi;
+      } else {
+        const int r = t < kTile ? t : 8 * (t - kTile) + (lane >> 3);
+        const int c = t < kTile ? lane : 64 + (lane & 7);
+        *reinterpret_cast<u4*>(dma_dst + r * kRowBytes + swz(c, r) * 16) = stg[i];
+      }
     }
+    if (TOK && j == 0 && dma_on && lane < kTile) ksc_dst[lane] = stg_ksc;
   };
 
-  if (KV_FP8) {                                   // the raw area starts out as zeros
+  if (STAGED) {                                   // the raw area starts out as zeros
     for (int i = lane; i < (kRawLat + kRawRope + kRawScale) / 16; i += 64)
       reinterpret_cast<uint4*>(raw_lat)[i] = make_uint4(0, 0, 0, 0);
   } else {                                        // so do both tiles: rows of invalid keys are never fetched
@@ -428,7 +481,18 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   int key_nxt = SHARE ? round_keys(1) : tile_key(1);
   unsigned long long next_mask = 0ull;
   if (SHARE) {
-    if (rounds > 0) issue_rows(key_cur, 16 * wave_u, smem + wave_u * kTileBytes);
+    if (R576) {                                   // the first round passes through the registers as well
+      dma_dst = smem + wave_u * kTileBytes;
+      ksc_dst = reinterpret_cast<float*>(smem + kRowsKscOff) + kTile * wave_u;
+      dma_on = rounds > 0;
+      key_dma = key_cur;
+      for (int j = 0; j < kWaves; ++j) {
+        fetch_share(j);
+        store_share(j);
+      }
+    } else if (rounds > 0) {
+      issue_rows(key_cur, 16 * wave_u, smem + wave_u * kTileBytes);
+    }
     next_mask = __ballot(key_cur >= 0);
   } else if (my_tiles > 0) {
     if (KV_FP8) issue_dma(key_cur);
@@ -451,10 +515,12 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
         next_mask = __ballot(key_dma >= 0);
         key_nxt = round_keys(r + 2);
         dma_dst = smem + (((r + 1) & 1) * kWaves + wave_u) * kTileBytes;
+        ksc_dst = reinterpret_cast<float*>(smem + kRowsKscOff) + (((r + 1) & 1) * kWaves + wave_u) * kTile;
         dma_on = r + 1 < rounds;
       }
       vmask = (unsigned)(round_mask >> (16 * j)) & 0xffffu;
       cur = smem + ((r & 1) * kWaves + j) * kTileBytes;
+      if (TOK) ksc = *reinterpret_cast<const f32x4*>(smem + kRowsKscOff + (((r & 1) * kWaves + j) * kTile + 4 * (lane >> 4)) * 4);
       const bool idle = heads_here == 0 || vmask == 0u;    // no products in this step
       fetch_share(j);
       if (idle) {                                          // a wavefront without heads only fetches
@@ -463,7 +529,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
       }
     } else {
     vmask = (unsigned)(__ballot(key_cur >= 0) & 0xffffull);
-    if (KV_FP8) {
+    if (STAGED) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // tile t has landed in the raw area
       if (E8) {
 #pragma unroll
@@ -598,7 +664,7 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   __syncthreads();                               // every wavefront is done with its tile
   // SHARE: the wavefronts hold different heads, nothing is merged - the same path with the sums
   // over wavefronts reduced to the wavefront's own entry serves as the transpose to channel order
-  float* stats = reinterpret_cast<float*>(smem + (KV_FP8 ? kStatOff : kRowsStatOff));
+  float* stats = reinterpret_cast<float*>(smem + (STAGED ? kStatOff : kRowsStatOff));
   if (lane < 16) {
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
@@ -814,7 +880,7 @@ void sparse_mla_mfma_plan(MlaParams& p) {
   // 16-bit rows with several head groups per KV group: the wavefronts share one key stream
   // (with two head groups two wavefronts only fetch and it still wins: 4.2 ms against 4.7 ms at
   // 64 heads x 4096 queries x 2048 keys)
-  p.tile_sharing = p.kv_dtype != CPPMEGA_MI355_E4M3 && groups_per_kv >= 2;
+  p.tile_sharing = (p.kv_dtype != CPPMEGA_MI355_E4M3 || p.q_dtype == CPPMEGA_MI355_E4M3) && groups_per_kv >= 2;
   const int units = p.tile_sharing ? (groups_per_kv + kWaves - 1) / kWaves : groups_per_kv;
   const long long base = (long long)p.B * p.S * p.G * units;
   int splits = 1;
@@ -839,10 +905,11 @@ int sparse_mla_mfma_launch(const MlaParams& p, hipStream_t stream) {
   void (*kernel)(MlaParams) = nullptr;
   int smem = kRowsSmemBytes;
   if (p.kv_dtype == CPPMEGA_MI355_E4M3) {
-    kernel = p.q_dtype != CPPMEGA_MI355_E4M3 ? sparse_mla_mfma_kernel<true>
-             : p.q_scale_kind == CPPMEGA_MI355_SCALE_E8M0 ? sparse_mla_mfma_kernel<true, false, false, 2>
-                                                          : sparse_mla_mfma_kernel<true, false, false, 1>;
-    smem = kSmemBytes;
+    const bool e8 = p.q_scale_kind == CPPMEGA_MI355_SCALE_E8M0;
+    if (p.q_dtype != CPPMEGA_MI355_E4M3) kernel = sparse_mla_mfma_kernel<true>;
+    else if (p.tile_sharing) kernel = e8 ? sparse_mla_mfma_kernel<true, false, true, 2> : sparse_mla_mfma_kernel<true, false, true, 1>;
+    else kernel = e8 ? sparse_mla_mfma_kernel<true, false, false, 2> : sparse_mla_mfma_kernel<true, false, false, 1>;
+    smem = p.tile_sharing ? kRowsFp8SmemBytes : kSmemBytes;
   } else if (p.kv_dtype == CPPMEGA_MI355_F16) {
     kernel = p.tile_sharing ? sparse_mla_mfma_kernel<false, true, true> : sparse_mla_mfma_kernel<false, true, false>;
   } else {

@@ -146,9 +146,11 @@ def test_per_token_fp8_prepared_buffers_with_sinks(device, with_sinks, out_dtype
     dict(B=1, S=4, H=16, G=1, Skv=256, topk=64),
     dict(B=2, S=3, H=40, G=1, Skv=700, topk=333),             # a partial head group, ragged tiles
     dict(B=1, S=2, H=64, G=2, Skv=5000, topk=2048),           # two KV groups, key splits + combine
-    dict(B=1, S=3, H=128, G=1, Skv=3000, topk=1000),
+    dict(B=1, S=3, H=128, G=1, Skv=3000, topk=1000),          # 4 head groups share one key stream
+    dict(B=2, S=2, H=144, G=2, Skv=900, topk=130),            # 72 heads per KV group: a wavefront without heads
+    dict(B=1, S=2, H=160, G=1, Skv=9000, topk=4096),          # two workgroups per query, key splits
     dict(B=1, S=2, H=64, G=1, Skv=100, topk=7),               # less than one tile
-], ids=["h16", "h40_ragged", "g2_splits", "h128", "h64_tiny"])
+], ids=["h16", "h40_ragged", "g2_splits", "h128", "h144_g2", "h160_splits", "h64_tiny"])
 @pytest.mark.parametrize("with_sinks", [False, True], ids=["plain", "sinks"])
 def test_mfma_kernel_per_token_fp8_rows(device, shape, with_sinks):
     """Per-token FP8 prepared buffers at the attention shape (rows of 576 codes, d_v 512; reference:
@@ -184,7 +186,9 @@ def test_mfma_kernel_per_token_fp8_rows(device, shape, with_sinks):
     dict(B=2, S=3, H=40, G=1, Skv=700, topk=333),
     dict(B=1, S=2, H=64, G=2, Skv=5000, topk=2048),
     dict(B=1, S=3, H=128, G=1, Skv=3000, topk=1000),
-], ids=["h16_odd_rows", "h40_ragged", "g2_splits", "h128"])
+    dict(B=2, S=2, H=144, G=2, Skv=901, topk=130),
+    dict(B=1, S=2, H=64, G=1, Skv=100, topk=7),
+], ids=["h16_odd_rows", "h40_ragged", "g2_splits", "h128", "h144_g2", "h64_tiny"])
 def test_mfma_kernel_e8m0_rows(device, shape):
     """E8M0-per-32 prepared buffers at the attention shape (rows of 576 codes + 18 scale bytes, d_v 512;
     reference: cppmega_mlx/nn/_tilelang/sparse_mla_blockscaled_path_c.py:943-1504) on the matrix cores.
