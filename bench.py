@@ -401,30 +401,53 @@ def bench_prefill(args, device):
 
 
 def bench_prefill_rows(args, device):
-    """The same prefill on unquantised 16-bit rows of 576 (the carrier of the reference's float
-    Path C kernels, float16): the 32-head tile kernel with its four wavefronts sharing one key stream."""
+    """The same prefill on the other row layouts the reference's Path C kernels take, all rows of 576
+    channels without a separate rope part: unquantised float16 rows (float Path C), e4m3 codes with
+    one fp32 scale per row and per (query, head) (FP8 Path C), e4m3 codes with one E8M0 byte per 32
+    channels (block-scaled Path C).  The 32-head tile kernel, four wavefronts sharing one key stream."""
     from cppmega_mlx_amd import ops
-    from cppmega_mlx_amd.nn._tilelang import topk_selector as tk
+    from cppmega_mlx_amd.nn._tilelang import (sparse_mla_blockscaled_path_c as bs, sparse_mla_fp8_path_c as f8,
+                                              topk_selector as tk)
 
     S, H, topk = 8192, 128, 2048
     gen = torch.Generator(device=device).manual_seed(556)
-    kv = torch.randn((1, S, 1, 576), generator=gen, device=device).to(torch.float16)
-    q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.float16)
     idx_scores = torch.randn((S, S), generator=gen, device=device)
     ends = torch.arange(1, S + 1, device=device, dtype=torch.int32)
     idx = torch.empty((S, topk), dtype=torch.int32, device=device)
     tk.topk_selector_tilelang_direct(idx_scores, topk, out=idx, ends=ends, order="index")
     idx = idx.view(1, S, 1, topk)
-    out = torch.empty((1, S, H, 512), dtype=torch.float16, device=device)
+    del idx_scores
     lse = torch.empty((1, S, H), dtype=torch.float32, device=device)
-    fn = lambda: ops.sparse_mla_forward(q, kv, idx, sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse)
-    steps = max(1, min(args.steps, 5))
-    secs, _ = timed_graph([fn], steps, 1)
-    per = secs / steps
     pairs = int(torch.minimum(ends.long(), torch.tensor(topk, device=device)).sum().item())
     flops = 2.0 * H * pairs * (576 + 512)
-    return {"workload": "sparse_mla_prefill float16 rows B=1 S=8192 H=128 topk=2048 causal", "ms_per_step": per * 1e3,
-            "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+    steps = max(1, min(args.steps, 5))
+    res = {}
+
+    def timed(name, fn, what):
+        secs, _ = timed_graph([fn], steps, 1)
+        per = secs / steps
+        res[name] = {"workload": f"sparse_mla_prefill {what} B=1 S=8192 H=128 topk=2048 causal", "ms_per_step": per * 1e3,
+                     "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+
+    kv = torch.randn((1, S, 1, 576), generator=gen, device=device).to(torch.float16)
+    q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.float16)
+    out = torch.empty((1, S, H, 512), dtype=torch.float16, device=device)
+    timed("float16_rows", lambda: ops.sparse_mla_forward(q, kv, idx, sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse),
+          "float16 rows")
+    qc = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.float8_e4m3fn).view(torch.uint8)
+    kc = torch.randn((1, S, 1, 576), generator=gen, device=device).to(torch.float8_e4m3fn).view(torch.uint8)
+    out = torch.empty((1, S, H, 512), dtype=torch.bfloat16, device=device)
+    qs = torch.rand((1, S, H), generator=gen, device=device) + 0.5
+    ks = torch.rand((1, S, 1), generator=gen, device=device) + 0.5
+    timed("fp8_per_token", lambda: f8.sparse_mla_fp8_path_c_apply_direct(qc, qs, kc, ks, idx, sm_scale=576 ** -0.5, out=out,
+                                                                         lse=lse, d_v=512),
+          "e4m3 rows + fp32 scale per row, e4m3 q + fp32 scale per head")
+    qe = torch.randint(120, 130, (1, S, H, 18), generator=gen, device=device, dtype=torch.uint8)
+    ke = torch.randint(120, 130, (1, S, 1, 18), generator=gen, device=device, dtype=torch.uint8)
+    timed("fp8_e8m0", lambda: bs.sparse_mla_blockscaled_path_c_apply_direct(qc, qe, kc, ke, idx, sm_scale=576 ** -0.5, out=out,
+                                                                           lse=lse, d_v=512),
+          "e4m3 rows and q + one E8M0 byte per 32 channels")
+    return res
 
 
 def bench_copy(args, device):
@@ -591,9 +614,10 @@ PROFILE_WORKLOADS = [
     ("kv_cache_append", ("cache_append_kernel",),
      "bf16 latent[B,S,1,512] + rope[..,64] -> e4m3 + fp32/128 scales + bf16 rope in the cache: one dispatch of 8192 rows "
      "(prefill chunk) and one of 32 rows (decode step) per step"),
-    ("sparse_mla_prefill_float16_rows", ("sparse_mla_mfma_kernel<false, true, true>",),
-     "sparse_mla_fwd q f16[1,8192,128,576], kv f16[1,8192,1,576] (unquantised rows), causal top-2048 indices -> f16[1,8192,128,512]: "
-     "the 32-head tile kernel, four wavefronts sharing one key stream"),
+    ("sparse_mla_prefill_row_layouts", ("sparse_mla_mfma_kernel<",),
+     "sparse_mla_fwd q [1,8192,128,576], kv [1,8192,1,576], causal top-2048 indices -> [1,8192,128,512] on the 32-head tile kernel, "
+     "four wavefronts sharing one key stream: <false, true, true, 0> unquantised float16 rows, <true, false, true, 1> e4m3 rows "
+     "with per-token fp32 scales, <true, false, true, 2> e4m3 rows with E8M0 bytes per 32 channels"),
     ("sparse_mla_backward", ("sparse_mla_bwd", "fill_zero_kernel"),
      "sparse_mla_bwd q bf16[1,1024,16,576], kv bf16[1,4096,1,576], d_out bf16[1,1024,16,512], topk 256 -> dq bf16, dkv f32 "
      "(the dkv clear, then the matrix-core kernel with its float32 atomic adds)"),
@@ -763,7 +787,7 @@ def main() -> int:
     if "prefill" in parts:
         line["prefill"] = bench_prefill(args, device)
     if "prefill" in parts or "prefill_rows" in parts:
-        line["prefill_float_rows"] = bench_prefill_rows(args, device)
+        line["prefill_row_layouts"] = bench_prefill_rows(args, device)
     if "copy" in parts:
         line["copy"] = bench_copy(args, device)
     if "next" in parts:
