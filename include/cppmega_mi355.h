@@ -206,7 +206,7 @@ int cppmega_mi355_indexer_topk(const cppmega_mi355_indexer_args_t* args, size_t 
 enum {
   CPPMEGA_MI355_MLA_KERNEL_AUTO = 0,
   CPPMEGA_MI355_MLA_KERNEL_SCALAR = 1,   /* one wavefront per (b,s,h), fp32 VALU */
-  CPPMEGA_MI355_MLA_KERNEL_MFMA = 2      /* head-batched bf16 MFMA, split-KV     */
+  CPPMEGA_MI355_MLA_KERNEL_MFMA = 2      /* head-batched MFMA, split-KV: d_qk 576, d_v 512; latent cache, 16-bit rows, or FP8 rows with per-token / E8M0 scales */
 };
 
 typedef struct cppmega_mi355_sparse_mla_args {
