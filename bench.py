@@ -712,7 +712,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="decode,vecmat,topk,next")
+    ap.add_argument("--only", type=str, default="decode,vecmat,topk,next,prefill")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.summarise_profiles:
