@@ -340,24 +340,25 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   };
   // SHARE: after the first round the rows travel through registers instead: each step fetches a
   // quarter of the wavefront's tile of the next round before its products and writes it to LDS
-  // after them.  Load t < 16 is the first 64 chunks of row t - one wave-uniform row address plus
-  // 16 bytes per lane, so its address costs no vector arithmetic; loads 16 and 17 are the last
-  // 8 chunks of rows 0..7 and 8..15 (lane = 8 * row + chunk).  The steps take loads 0-4, 5-9,
-  // 10-14, 15-17.
-  // Measured (128 heads x 4096 queries x 2048 keys; rows resident in the L2 or not makes no
-  // difference): 4.09 ms.  The same loads with lanes straddling two rows (a per-lane select and
-  // 64-bit products) 4.25 ms; LDS-writing loads in their place 4.55 ms, all 18 of them at the
-  // start of the round 4.87 ms; one load at a time between the matrix products 4.8 ms; the four
-  // wavefronts fetching at four different points of the step 5.7 ms.  Clock stamps put ~1.7 k of
-  // a step's 5.2 k clocks into the five loads (4.25 ms form) - a wavefront that is alone on its
-  // SIMD issues in order and nothing hides what it spends there.
-  // FP8 rows of 576 codes in this mode: 9 loads per tile - load t < 8 carries the first 512 codes of
-  // rows 2t and 2t + 1 (32 lanes x 16 bytes each), load 8 the last 64 codes of all 16 rows (4 lanes
-  // each); the steps take loads 0-2, 3-4, 5-6, 7-8.  A lane's 16 codes become 16 bfloat16 (two
-  // 16-byte slots) on their way into the tile.  E8M0: the lane also fetches the scale byte of its
-  // 16 codes.  Per token: the 16 row scales go to a small array the four wavefronts read.
+  // after them.
+  // Measured (16-bit rows, 128 heads x 4096 queries x 2048 keys; rows resident in the L2 or not
+  // makes no difference): 3.67 ms, of which 2.83 ms remain with the fetches taken out.  A wavefront
+  // that is alone on its SIMD issues in order, and what it spends on issuing a load the matrix
+  // products do not hide.  Forms that were slower: loads whose lanes straddle two rows with
+  // per-lane 64-bit address products, 18 per tile in four uneven shares, 4.09 - 4.25 ms; the same
+  // as LDS-writing loads 4.55 ms, all 18 at the start of the round 4.87 ms; the loads of a step
+  // spread one at a time between its matrix products 4.2 ms (4.8 ms with the heavier addresses);
+  // the four wavefronts fetching at four different points of the step 5.7 ms.
+  // Step j of a round fetches rows 4j .. 4j + 3 of the wavefront's tile of the next round:
+  //   16-bit rows: four loads of a row's first 64 slots (wave-uniform row address + 16 bytes per
+  //     lane) and one load of the last 8 slots of the four rows (32 lanes);
+  //   FP8 rows of 576 codes: two loads of the first 512 codes of two rows each (32 lanes a row) and
+  //     one of the last 64 codes of the four rows (16 lanes); a lane's 16 codes become 16 bfloat16
+  //     (two slots) on their way into the tile.  E8M0: the lane also fetches the scale byte of
+  //     its 16 codes.  Per token: step 0 fetches the 16 row scales for the array the four
+  //     wavefronts read.
+  // Every step has the same shape, so the address of a load is a handful of scalar instructions.
   typedef __attribute__((ext_vector_type(4))) unsigned u4;
-  constexpr int kLoads = R576 ? 9 : kTileBytes / 1024;     // per tile
   constexpr int kPerStep = R576 ? 3 : 5;
   unsigned char* dma_dst = smem;                  // this wavefront's tile of the next round
   float* ksc_dst = reinterpret_cast<float*>(smem + kRowsKscOff);   // ... and its 16 row scales
@@ -366,82 +367,81 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   u4 stg[kPerStep];
   unsigned char stg_e8[kPerStep];
   float stg_ksc = 0.0f;
-  auto share_load = [&](int j, int i) -> int {    // index of the i-th load of step j, or kLoads
-    if (!R576) return 5 * j + i;
-    return j == 0 ? i : (i < 2 ? 1 + 2 * j + i : kLoads);
-  };
-  auto fetch_share = [&](int j) {
-    const int first = 16 * __builtin_amdgcn_readfirstlane(wave);
-    const size_t row_base = (size_t)b * p.Skv_pitch;
-#pragma unroll
-    for (int i = 0; i < kPerStep; ++i) {
-      const int t = share_load(j, i);             // uniform
-      stg[i] = u4{0u, 0u, 0u, 0u};
-      stg_e8[i] = 0;
-      if (!dma_on || t >= kLoads) continue;
-      if (R576) {
-        int row, off, blk;
-        if (t < 8) {
-          const int ra = __builtin_amdgcn_readlane(key_dma, first + 2 * t), rb = __builtin_amdgcn_readlane(key_dma, first + 2 * t + 1);
-          row = lane < 32 ? ra : rb;
-          off = (lane & 31) * 16;
-          blk = (lane & 31) >> 1;
-        } else {
-          row = __shfl(key_dma, first + (lane >> 2), 64);
-          off = kLat + (lane & 3) * 16;
-          blk = 16 + ((lane & 3) >> 1);
+  // row r of the cache as this (batch, KV group) sees it starts at base + r * stride
+  const size_t krow0 = (size_t)b * p.Skv_pitch * p.G + g;
+  const unsigned row_bytes = R576 ? (unsigned)kDqk : (unsigned)p.d_kv * 2u;
+  const unsigned kv_stride = (unsigned)p.G * row_bytes;
+  const unsigned char* kv0 = (const unsigned char*)p.kv + krow0 * row_bytes;
+  const bool packed = R576 || p.d_kv == kDqk;     // the last 64 channels sit in the row itself, not in p.rope
+  const unsigned char* tail0 = packed ? kv0 + (R576 ? kLat : kLat * 2) : (const unsigned char*)p.rope + krow0 * (kRope * 2);
+  const unsigned tail_stride = packed ? kv_stride : (unsigned)p.G * (kRope * 2);
+  const unsigned sc_stride = (unsigned)p.G * (E8 ? (unsigned)kE8Row : 4u);
+  const unsigned char* sc0 = R576 ? (const unsigned char*)p.kv_scale + krow0 * (E8 ? (size_t)kE8Row : 4) : nullptr;
+  auto fetch_one = [&](int j, int i) {            // load i of step j (j uniform, i a constant)
+    if (i >= kPerStep) return;
+    const int first = 16 * __builtin_amdgcn_readfirstlane(wave) + 4 * j;
+    stg[i] = u4{0u, 0u, 0u, 0u};
+    stg_e8[i] = 127;                              // scale 1
+    if (!dma_on) return;
+    if (R576) {
+      if (i < 2) {
+        const int ra = __builtin_amdgcn_readlane(key_dma, first + 2 * i), rb = __builtin_amdgcn_readlane(key_dma, first + 2 * i + 1);
+        const int key = lane < 32 ? ra : rb;
+        if (key >= 0) {
+          stg[i] = *reinterpret_cast<const u4*>(kv0 + (size_t)key * kv_stride + (lane & 31) * 16);
+          if (E8) stg_e8[i] = sc0[(size_t)key * sc_stride + ((lane & 31) >> 1)];
         }
-        if (row >= 0) {
-          const size_t krow = (row_base + (size_t)row) * p.G + g;
-          stg[i] = *reinterpret_cast<const u4*>((const unsigned char*)p.kv + krow * kDqk + off);
-          if (E8) stg_e8[i] = ((const unsigned char*)p.kv_scale)[krow * kE8Row + blk];
-        }
-      } else if (t < kTile) {
-        const int row = __builtin_amdgcn_readlane(key_dma, first + t);
-        if (row >= 0) {                           // uniform
-          const size_t krow = (row_base + (size_t)row) * p.G + g;
-          const unsigned short* src = (const unsigned short*)p.kv + krow * (size_t)p.d_kv;
-          stg[i] = *reinterpret_cast<const u4*>(src + lane * 8);
+        if (TOK && i == 0 && j == 0) {            // lane r < 16: the scale of the tile's key r
+          const int kr = __shfl(key_dma, first + (lane & 15), 64);
+          stg_ksc = 0.0f;
+          if (kr >= 0) stg_ksc = *reinterpret_cast<const float*>(sc0 + (size_t)kr * sc_stride);
         }
       } else {
-        const int row = __shfl(key_dma, first + 8 * (t - kTile) + (lane >> 3), 64);
-        if (row >= 0) {
-          const size_t krow = (row_base + (size_t)row) * p.G + g;
-          const int c8 = (64 + (lane & 7)) * 8;
-          const unsigned short* src = c8 < p.d_kv ? (const unsigned short*)p.kv + krow * (size_t)p.d_kv + c8
-                                                  : (const unsigned short*)p.rope + krow * kRope + (c8 - p.d_kv);
-          stg[i] = *reinterpret_cast<const u4*>(src);
+        const int key = __shfl(key_dma, first + ((lane >> 2) & 3), 64);
+        if (lane < 16 && key >= 0) {
+          stg[2] = *reinterpret_cast<const u4*>(tail0 + (size_t)key * tail_stride + (lane & 3) * 16);
+          if (E8) stg_e8[2] = sc0[(size_t)key * sc_stride + 16 + ((lane & 3) >> 1)];
         }
       }
-    }
-    if (TOK && j == 0 && dma_on) {                // lane r < 16: the scale of the tile's key r
-      const int row = __shfl(key_dma, first + (lane & 15), 64);
-      stg_ksc = 0.0f;
-      if (row >= 0) stg_ksc = ((const float*)p.kv_scale)[(row_base + (size_t)row) * p.G + g];
+    } else if (i < 4) {
+      const int key = __builtin_amdgcn_readlane(key_dma, first + i);
+      if (key >= 0) stg[i] = *reinterpret_cast<const u4*>(kv0 + (size_t)key * kv_stride + lane * 16);   // uniform branch
+    } else {
+      const int key = __shfl(key_dma, first + ((lane >> 3) & 3), 64);
+      if (lane < 32 && key >= 0) stg[4] = *reinterpret_cast<const u4*>(tail0 + (size_t)key * tail_stride + (lane & 7) * 16);
     }
   };
-  auto store_share = [&](int j) {
+  auto fetch_share = [&](int j) {
 #pragma unroll
-    for (int i = 0; i < kPerStep; ++i) {
-      const int t = share_load(j, i);
-      if (!dma_on || t >= kLoads) continue;
-      if (R576) {
-        const int r = t < 8 ? 2 * t + (lane >> 5) : lane >> 2;
-        const int c = t < 8 ? 2 * (lane & 31) : 64 + 2 * (lane & 3);      // first of the two slots
+    for (int i = 0; i < kPerStep; ++i) fetch_one(j, i);
+  };
+  auto store_share = [&](int j) {
+    if (!dma_on) return;
+    if (R576) {
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        const int r = 4 * j + (i < 2 ? 2 * i + (lane >> 5) : (lane >> 2) & 3);
+        const int c = i < 2 ? 2 * (lane & 31) : 64 + 2 * (lane & 3);         // first of the two slots
         const float sc = E8 ? e8m0_to_f32(stg_e8[i]) : 1.0f;
         const uint4 raw = make_uint4(stg[i][0], stg[i][1], stg[i][2], stg[i][3]);
         uint4 lo, hi;
         if (__ballot(!scale_is_pow2(sc)) == 0ull) dequant16<true>(raw, sc, lo, hi);
         else dequant16<false>(raw, sc, lo, hi);
-        *reinterpret_cast<uint4*>(dma_dst + r * kRowBytes + swz(c, r) * 16) = lo;
-        *reinterpret_cast<uint4*>(dma_dst + r * kRowBytes + swz(c + 1, r) * 16) = hi;
-      } else {
-        const int r = t < kTile ? t : 8 * (t - kTile) + (lane >> 3);
-        const int c = t < kTile ? lane : 64 + (lane & 7);
-        *reinterpret_cast<u4*>(dma_dst + r * kRowBytes + swz(c, r) * 16) = stg[i];
+        if (i < 2 || lane < 16) {
+          *reinterpret_cast<uint4*>(dma_dst + r * kRowBytes + swz(c, r) * 16) = lo;
+          *reinterpret_cast<uint4*>(dma_dst + r * kRowBytes + swz(c + 1, r) * 16) = hi;
+        }
       }
+      if (TOK && j == 0 && lane < kTile) ksc_dst[lane] = stg_ksc;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 4 * j + i;
+        *reinterpret_cast<u4*>(dma_dst + r * kRowBytes + swz(lane, r) * 16) = stg[i];
+      }
+      const int r = 4 * j + ((lane >> 3) & 3);
+      if (lane < 32) *reinterpret_cast<u4*>(dma_dst + r * kRowBytes + swz(64 + (lane & 7), r) * 16) = stg[4];
     }
-    if (TOK && j == 0 && dma_on && lane < kTile) ksc_dst[lane] = stg_ksc;
   };
 
   if (STAGED) {                                   // the raw area starts out as zeros
