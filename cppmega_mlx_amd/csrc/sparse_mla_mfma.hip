@@ -342,7 +342,8 @@ __global__ __launch_bounds__(kWaves * 64, 1) void sparse_mla_mfma_kernel(const M
   // quarter of the wavefront's tile of the next round before its products and writes it to LDS
   // after them.
   // Measured (16-bit rows, 128 heads x 4096 queries x 2048 keys; rows resident in the L2 or not
-  // makes no difference): 3.67 ms, of which 2.83 ms remain with the fetches taken out.  A wavefront
+  // makes no difference, nor do four hot rows that stay in the L1: 3.71 against 3.86 ms in one
+  // run): 3.7 ms, of which 2.83 ms remain with the fetches taken out.  A wavefront
   // that is alone on its SIMD issues in order, and what it spends on issuing a load the matrix
   // products do not hide.  Forms that were slower: loads whose lanes straddle two rows with
   // per-lane 64-bit address products, 18 per tile in four uneven shares, 4.09 - 4.25 ms; the same
