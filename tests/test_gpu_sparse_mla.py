@@ -328,6 +328,26 @@ def test_mfma_kernel_float16_rows(device, shape, rope_tail):
     assert (out[0, 1] == 0).all() and (lse[0, 1] == 0).all()
 
 
+def test_shared_key_stream_int64_indices_and_cache_views(device):
+    """128 heads on bf16 rows of 576: int64 indices, and the rows passed as the live prefix of a larger
+    cache buffer (batch pitch = capacity), as `update_and_fetch` hands them out."""
+    rng = np.random.default_rng(4242)
+    B, S, H, cap, Skv, topk = 2, 3, 128, 600, 500, 200
+    q, qf = bf16_pair(rng.standard_normal((B, S, H, 576)), device)
+    buf, buf_f = bf16_pair(rng.standard_normal((B, cap, 1, 576)), device)
+    kv = buf[:, :Skv]
+    idx = sparse_indices(rng, B, S, 1, Skv, topk, replace=True)
+    idx[rng.random(idx.shape) < 0.1] = -1
+    idx[1, 0, 0, :3] = [Skv, Skv + 50, cap - 1]                      # beyond the live length: skipped, though inside the buffer
+    want_out, want_lse = om.sparse_mla_oracle(qf, buf_f[:, :Skv], idx, sm_scale=576 ** -0.5, d_v=512)
+    out = torch.zeros((B, S, H, 512), dtype=torch.bfloat16, device=device)
+    lse = torch.zeros((B, S, H), dtype=torch.float32, device=device)
+    ops.sparse_mla_forward(q, kv, to_dev(idx.astype(np.int64), device), sm_scale=576 ** -0.5, d_v=512, out=out, lse=lse,
+                           kernel="mfma")
+    torch.cuda.synchronize()
+    _assert_close(out, lse, want_out, want_lse, lse_tol=LSE_TOL_MFMA)
+
+
 @pytest.mark.parametrize("pow2", [True, False], ids=["pow2_scales", "general_scales"])
 def test_decode_full_config_sampled_batches(device, pow2):
     """B=32, S_q=1, H=128, topk=2048 over a 65536-token FP8 cache (the headline
