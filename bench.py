@@ -397,7 +397,9 @@ def bench_prefill(args, device):
     pairs = int(torch.minimum(ends.long(), torch.tensor(topk, device=device)).sum().item())
     flops = 2.0 * H * pairs * (576 + 512)
     return {"workload": "sparse_mla_prefill B=1 S=8192 H=128 topk=2048 causal", "ms_per_step": per * 1e3,
-            "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+            "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "roofline": {"bound": "mfma", "achieved": flops / per / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None}}
 
 
 def bench_prefill_rows(args, device):
@@ -427,7 +429,9 @@ def bench_prefill_rows(args, device):
         secs, _ = timed_graph([fn], steps, 1)
         per = secs / steps
         res[name] = {"workload": f"sparse_mla_prefill {what} B=1 S=8192 H=128 topk=2048 causal", "ms_per_step": per * 1e3,
-                     "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+                     "tflops_valid_pairs": flops / per / 1e12, "frac_of_bf16_mfma_peak": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                     "roofline": {"bound": "mfma", "achieved": flops / per / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
+                                  "unit": "TFLOP/s", "frac": flops / per / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None}}
 
     kv = torch.randn((1, S, 1, 576), generator=gen, device=device).to(torch.float16)
     q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.float16)
