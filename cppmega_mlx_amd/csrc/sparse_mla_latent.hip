@@ -69,7 +69,7 @@ constexpr int kMaxKeys = 2048;                  // keys of one split (their rows
 constexpr int kKeyInts = kMaxKeys + kTK;
 constexpr int kHeadsWg = 64;
 constexpr int kXPitch = 132;                    // floats per head row of the output transpose (128 + 4)
-constexpr int kPartFloats = 4 * 16 * 64 * 4;    // partial values of one 32-head group: [4 consumers][16 rows][64 lanes][4]
+constexpr int kPartFloats = 4 * 16 * 64 * 4;    // partial values of one 32-head group: [4 consumers][8 row pairs][64 lanes][8]
 constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
 
 constexpr int kPBytes = 2 * 2 * 1024;           // P of one tile: [k-step][head block][64 lanes x 16 B]
@@ -773,15 +773,17 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       // key split: the unnormalised accumulators leave exactly as the lanes hold them (rounded to
       // bf16: the values are relative to the split's own maximum, so their range is that of the
       // output times the split's probability mass)
+      // (two accumulator rows of a lane per 16-byte store: [consumer][head half][dvb][row pair][lane][8])
       unsigned short* blk = (unsigned short*)p.workspace + part_block * (size_t)(2 * kPartFloats) +
-                            ((size_t)((role * 2 + hb) * 16) * 64 + lane) * 4;
+                            ((size_t)((role * 2 + hb) * 8) * 64 + lane) * 8;
 #pragma unroll
       for (int dvb = 0; dvb < 4; ++dvb) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j2 = 0; j2 < 2; ++j2) {
           const f32x16& acc = o[dvb][hb];
-          *reinterpret_cast<uint2*>(blk + (size_t)(dvb * 4 + j) * 256) =
-              make_uint2(pack_bf16(acc[4 * j], acc[4 * j + 1]), pack_bf16(acc[4 * j + 2], acc[4 * j + 3]));
+          *reinterpret_cast<uint4*>(blk + (size_t)(dvb * 2 + j2) * 512) =
+              make_uint4(pack_bf16(acc[8 * j2], acc[8 * j2 + 1]), pack_bf16(acc[8 * j2 + 2], acc[8 * j2 + 3]),
+                         pack_bf16(acc[8 * j2 + 4], acc[8 * j2 + 5]), pack_bf16(acc[8 * j2 + 6], acc[8 * j2 + 7]));
         }
       }
       if (role == 0 && lane < 32) {
@@ -893,25 +895,28 @@ __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const Ml
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   const unsigned short* src0 = (const unsigned short*)p.workspace + block0 * (size_t)(HG * kPartFloats) +
-                               ((size_t)((w * HG + hg) * 16 + 4 * r4) * 64 + lane) * 4;
+                               ((size_t)((w * HG + hg) * 8 + 2 * r4) * 64 + lane) * 8;
 #pragma unroll
   for (int s0 = 0; s0 < 16; s0 += 4) {
     if (s0 >= p.num_splits) break;                            // (uniform)
-    uint2 raw[4][4];
+    uint4 raw[4][2];                                           // two accumulator rows per 16-byte load
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int s = min(s0 + u, p.num_splits - 1);             // a repeated last split gets weight 0
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        raw[u][i] = *reinterpret_cast<const uint2*>(src0 + (size_t)s * (HG * kPartFloats) + (size_t)i * 256);
+      for (int i2 = 0; i2 < 2; ++i2)
+        raw[u][i2] = *reinterpret_cast<const uint4*>(src0 + (size_t)s * (HG * kPartFloats) + (size_t)i2 * 512);
     }
     float4 v[4][4];
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        v[u][i] = make_float4(__uint_as_float(raw[u][i].x << 16), __uint_as_float(raw[u][i].x & 0xffff0000u),
-                              __uint_as_float(raw[u][i].y << 16), __uint_as_float(raw[u][i].y & 0xffff0000u));
+      for (int i2 = 0; i2 < 2; ++i2) {
+        v[u][2 * i2] = make_float4(__uint_as_float(raw[u][i2].x << 16), __uint_as_float(raw[u][i2].x & 0xffff0000u),
+                                   __uint_as_float(raw[u][i2].y << 16), __uint_as_float(raw[u][i2].y & 0xffff0000u));
+        v[u][2 * i2 + 1] = make_float4(__uint_as_float(raw[u][i2].z << 16), __uint_as_float(raw[u][i2].z & 0xffff0000u),
+                                       __uint_as_float(raw[u][i2].w << 16), __uint_as_float(raw[u][i2].w & 0xffff0000u));
+      }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const float f = (s0 + u < p.num_splits && ms[s0 + u] != -INFINITY) ? exp2f(ms[s0 + u] - m_fin) : 0.0f;
