@@ -823,22 +823,24 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    // rows of 128 channels leave coalesced: 32 lanes x 4 channels, two heads per step
+    // rows of 128 channels leave coalesced: 16 lanes x 8 channels, four heads per step
 #pragma unroll 4
-    for (int it = 0; it < 16; ++it) {
-      const int row = 2 * it + gq2;
+    for (int it = 0; it < 8; ++it) {
+      const int row = 4 * it + (lane >> 4), c8 = (lane & 15) * 8;
       const int hl = 32 * hb + row;
       if (hl >= heads_here) continue;
-      const float4 v = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + hd * 4);
-      const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + 128 * role + hd * 4;
+      const float4 v = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + c8);
+      const float4 u = *reinterpret_cast<const float4*>(xbuf + row * kXPitch + c8 + 4);
+      const size_t off = (q_index * p.H + head0 + hl) * (size_t)kLat + 128 * role + c8;
       if (p.out_dtype == CPPMEGA_MI355_F32) {
         *reinterpret_cast<float4*>((float*)p.out + off) = v;
+        *reinterpret_cast<float4*>((float*)p.out + off + 4) = u;
       } else if (p.out_dtype == CPPMEGA_MI355_BF16) {
-        *reinterpret_cast<uint2*>((unsigned short*)p.out + off) = make_uint2(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w));
+        *reinterpret_cast<uint4*>((unsigned short*)p.out + off) =
+            make_uint4(pack_bf16(v.x, v.y), pack_bf16(v.z, v.w), pack_bf16(u.x, u.y), pack_bf16(u.z, u.w));
       } else {
-        unsigned short* dst = (unsigned short*)p.out + off;
-        dst[0] = f32_to_f16_bits(v.x); dst[1] = f32_to_f16_bits(v.y);
-        dst[2] = f32_to_f16_bits(v.z); dst[3] = f32_to_f16_bits(v.w);
+        *reinterpret_cast<uint4*>((unsigned short*)p.out + off) =
+            make_uint4(pack_f16(v.x, v.y), pack_f16(v.z, v.w), pack_f16(u.x, u.y), pack_f16(u.z, u.w));
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
