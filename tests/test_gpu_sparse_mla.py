@@ -404,18 +404,21 @@ def test_decode_full_config_sampled_batches(device, pow2):
     assert np.abs(lse_m - got_lse).max() <= 1e-4
 
 
-def test_prefill_full_config_sampled_queries(device):
+@pytest.mark.parametrize("pow2", [True, False], ids=["pow2_scales", "general_scales"])
+def test_prefill_full_config_sampled_queries(device, pow2):
     """B=1, S=8192, H=128, topk=2048 with causal top-k indices over an 8192-token FP8 cache: the
     whole chunk runs on the GPU (indices from the GPU selector), sampled queries -- heavily
     padded early ones, the 2047/2048 boundary, the last -- are checked against the oracle, and
-    every query with no visible key beyond itself must reproduce its own value row."""
+    every query with no visible key beyond itself must reproduce its own value row.  Block scales
+    are powers of two (2^ceil(log2(amax/448))) or general fp32 values (amax/448)."""
     from cppmega_mlx_amd import _lib
     from cppmega_mlx_amd.nn._tilelang import topk_selector as tk
     S, H, topk = 8192, 128, 2048
     gen = torch.Generator(device=device).manual_seed(17)
     lat = torch.randn((S, 1, 4, 128), generator=gen, device=device)
-    sc = torch.exp2(torch.ceil(torch.log2(lat.abs().amax(dim=-1) / 448.0)))
-    codes = (lat / sc[..., None]).to(torch.float8_e4m3fn).view(torch.uint8).reshape(1, S, 1, 512)
+    amax = lat.abs().amax(dim=-1)
+    sc = torch.exp2(torch.ceil(torch.log2(amax / 448.0))) if pow2 else amax / 448.0
+    codes = (lat / sc[..., None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).reshape(1, S, 1, 512)
     scale = sc.reshape(1, S, 1, 4).contiguous()
     rope = torch.randn((1, S, 1, 64), generator=gen, device=device).to(torch.bfloat16)
     q = torch.randn((1, S, H, 576), generator=gen, device=device).to(torch.bfloat16)
