@@ -12,17 +12,17 @@
 //
 //   producers (wavefronts 0..3): producer p owns heads 16p..16p+15 of the chunk.
 //     S^T = K.Q^T on v_mfma_scale_f32_16x16x128_f8f6f4: the key bytes are the A operand as they
-//     lie in the tile (no conversion instructions); the power-of-two part of a key's block scale
-//     is the operand exponent, the mantissa part multiplies the block's fp32 partial sum.  Q^T is
+//     lie in the tile (no conversion instructions, operand exponent 2^0); every 128-channel block is
+//     accumulated from zero and enters the score times its keys' fp32 block scales.  Q^T is
 //     split once per workgroup into two e4m3 planes hi + lo (hi + lo = the bf16 value, one
 //     exponent per head and 128 channels), kept in registers.  The rope tail is a bf16 product.
 //     Softmax in base 2 with a lazily moved private running maximum per head; P goes to LDS as
-//     bf16 in the B-operand layout of the value product, once per scale block with V's block
-//     scale folded in.
+//     bf16 in the B-operand layout of the value product, one plane per scale block: plane b is P
+//     times the keys' scales of block b (one fp32 product, rounded once).
 //   consumers (wavefronts 4..7): consumer c owns value channels 128c..128c+127 (= scale block c
-//     when there are four) for all 64 heads: O^T += V^T.P^T on v_mfma_f32_32x32x16_bf16, V^T
-//     fragments by transposing LDS reads of the raw tile, converted unscaled (exactly).  They
-//     also issue the row loads.
+//     when there are four) for all 64 heads: O^T += V^T.P_c^T on v_mfma_f32_32x32x16_bf16, V^T
+//     fragments by transposing LDS reads of the raw tile, converted unscaled (exactly), P_c the
+//     plane of its block.  They also issue the row loads.
 //   pipeline  iteration t: barrier; producers: scores and P of tile t+1; consumers: issue tile
 //             t+4, value product of tile t.  One barrier per tile.
 //
@@ -61,8 +61,7 @@ constexpr int kPlane = 1024 + 128;              // bytes from plane 0 to plane 1
 constexpr int kPair = 2 * kPlane;               // one (sub-tile, block)
 constexpr int kLatBytes = 8 * kPair;            // 18432
 constexpr int kRopeBytes = 4 * 1024;            // [sj][s] planes
-constexpr int kScaleBytes = 2 * kTK * 4 * 4;    // up to four fp32 scales per row, twice: [row][block], then [block][row]
-constexpr int kScaleT = kTK * 4 * 4;            // offset of the [block][row] copy inside the scale area
+constexpr int kScaleBytes = kTK * 4 * 4;        // up to four fp32 scales per row: [row][block]
 constexpr int kSlotBytes = kLatBytes + kRopeBytes + kScaleBytes;   // 23552
 constexpr int kRingBytes = kRing * kSlotBytes;  // 104960
 constexpr int kMaxKeys = 2048;                  // keys of one split (their rows are staged in LDS)
@@ -72,7 +71,8 @@ constexpr int kXPitch = 132;                    // floats per head row of the ou
 constexpr int kPartFloats = 4 * 16 * 64 * 4;    // partial values of one 32-head group: [4 consumers][8 row pairs][64 lanes][8]
 constexpr float kLazy = 8.0f;                   // move a running maximum only when it grows by > 2^8
 
-constexpr int kPBytes = 2 * 2 * 1024;           // P of one tile: [k-step][head block][64 lanes x 16 B]
+constexpr int kPPlane = 2 * 2 * 1024;           // one plane of P of one tile: [k-step][head block][64 lanes x 16 B]
+constexpr int kPBytes = 4 * kPPlane;            // up to four planes per tile: P times V's scale of block b
 constexpr int kPOff = kRingBytes;
 constexpr int kFacOff = kPOff + 2 * kPBytes;        // [parity][4 producers][16 heads] fp32
 constexpr int kFlagOff = kFacOff + 2 * 4 * 16 * 4;  // [parity][4 producers] int
@@ -91,11 +91,6 @@ __device__ __forceinline__ bf16x8 cvt8(unsigned w0, unsigned w1) {
   const unsigned o2 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, false));
   const unsigned o3 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w1, 1.0f, true));
   return __builtin_bit_cast(bf16x8, make_uint4(o0, o1, o2, o3));
-}
-
-// sign and mantissa of a scale with the exponent of 1.0: scale = 2^(exponent field - 127) * this
-__device__ __forceinline__ float scale_mant(float s) {
-  return __uint_as_float((__float_as_uint(s) & 0x807fffffu) | 0x3f800000u);
 }
 
 // 16 x 16 x 128 over e4m3 bytes, operands scaled by 2^(byte - 127): the byte is byte SEL of `a_exp`
@@ -343,44 +338,27 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     float l_run = 0.0f;                           // this lane's share of its denominator
     const float qk_scale = sm_scale * kLog2e;
 
-    // K operands of a tile -> registers: per sub-tile four 32-byte block fragments, two rope
-    // fragments and the scales of this lane's key row (they give the operand exponents).  They are
-    // requested one tile ahead, right after the previous tile's products, so that they land
-    // under its softmax.
+    // K operands of a tile -> registers: per sub-tile four 32-byte block fragments and two rope
+    // fragments.  The first sub-tile is requested one tile ahead, right after the previous tile's
+    // products, so that it lands under its softmax; the second one at the start of the tile, under
+    // the first one's products.
     i32x8 kf[2][4];
     bf16x8 rf[2][2];
-    float own[2][nblk];
-    auto load_k = [&](int tau) {
+    auto load_k = [&](int tau, int sj) {
       const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
-      const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
+      // the lane's 32 bytes of a block are its 16 bytes of the block's two planes
+      const unsigned char* lat = slot + sj * (4 * kPair) + lane * 16;
+      const unsigned char* rope = slot + kLatBytes + sj * 2048 + lane * 16;
 #pragma unroll
-      for (int sj = 0; sj < 2; ++sj) {
-        const float* scl = scl_base + (16 * sj + n) * nblk;
-        if (nblk == 4) {
-          const float4 o4 = *reinterpret_cast<const float4*>(scl);
-          own[sj][0] = o4.x; own[sj][1 % nblk] = o4.y; own[sj][2 % nblk] = o4.z; own[sj][3 % nblk] = o4.w;
-        } else if (nblk == 2) {
-          const float2 o2 = *reinterpret_cast<const float2*>(scl);
-          own[sj][0] = o2.x; own[sj][1 % nblk] = o2.y;
-        } else {
-          own[sj][0] = scl[0];
-        }
+      for (int blk = 0; blk < 4; ++blk) {
+        const uint4 c0 = *reinterpret_cast<const uint4*>(lat + blk * kPair);
+        const uint4 c1 = *reinterpret_cast<const uint4*>(lat + blk * kPair + kPlane);
+        kf[sj][blk] = i32x8{(int)c0.x, (int)c0.y, (int)c0.z, (int)c0.w, (int)c1.x, (int)c1.y, (int)c1.z, (int)c1.w};
       }
-#pragma unroll
-      for (int sj = 0; sj < 2; ++sj) {
-        // the lane's 32 bytes of a block are its 16 bytes of the block's two planes
-        const unsigned char* lat = slot + sj * (4 * kPair) + lane * 16;
-        const unsigned char* rope = slot + kLatBytes + sj * 2048 + lane * 16;
-#pragma unroll
-        for (int blk = 0; blk < 4; ++blk) {
-          const uint4 c0 = *reinterpret_cast<const uint4*>(lat + blk * kPair);
-          const uint4 c1 = *reinterpret_cast<const uint4*>(lat + blk * kPair + kPlane);
-          kf[sj][blk] = i32x8{(int)c0.x, (int)c0.y, (int)c0.z, (int)c0.w, (int)c1.x, (int)c1.y, (int)c1.z, (int)c1.w};
-        }
-        rf[sj][0] = *reinterpret_cast<const bf16x8*>(rope);
-        rf[sj][1] = *reinterpret_cast<const bf16x8*>(rope + 1024);
-      }
+      rf[sj][0] = *reinterpret_cast<const bf16x8*>(rope);
+      rf[sj][1] = *reinterpret_cast<const bf16x8*>(rope + 1024);
     };
+    constexpr int kOne = 0x7f7f7f7f;                // operand exponent bytes of 2^0: the key bytes enter the products unscaled
 
     // scores and probabilities of tile tau (whose K operands are in registers) -> P(tau) in LDS;
     // `next`: tile tau+1 exists (it has landed)
@@ -394,100 +372,66 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
 #pragma unroll
         for (int sj = 0; sj < 2; ++sj) kk[sj] = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * sj + 4 * kg);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      // exponent bytes of this lane's key rows, and whether any row of the tile has a mantissa part
-      int kexp[2];
-      bool plain = true;
-#pragma unroll
-      for (int sj = 0; sj < 2; ++sj) {
-        kexp[sj] = 0;
-#pragma unroll
-        for (int blk = 0; blk < 4; ++blk) {
-          const unsigned sc = __float_as_uint(own[sj][(blk * nblk) >> 2]);
-          kexp[sj] |= (int)(((sc >> 23) & 0xffu) << (8 * blk));
-          plain = plain && ((sc & 0x807fffffu) == 0u);
-        }
-      }
-      const bool all_plain = __ballot(!plain) == 0ull;       // (uniform)
-      float ksc[2][4][nblk];                        // scales of keys 16 sj + 4 kg + i: their mantissa parts multiply the partial sums
-      if (!all_plain) {
-#pragma unroll
-        for (int sj = 0; sj < 2; ++sj) {
-          const float* sclc = scl_base + (16 * sj + 4 * kg) * nblk;
-          if (nblk == 4) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float4 v4 = *reinterpret_cast<const float4*>(sclc + 4 * i);
-              ksc[sj][i][0] = v4.x; ksc[sj][i][1 % nblk] = v4.y; ksc[sj][i][2 % nblk] = v4.z; ksc[sj][i][3 % nblk] = v4.w;
-            }
-          } else if (nblk == 2) {
-            const float4 a = *reinterpret_cast<const float4*>(sclc), bq = *reinterpret_cast<const float4*>(sclc + 4);
-            ksc[sj][0][0] = a.x; ksc[sj][0][1 % nblk] = a.y; ksc[sj][1][0] = a.z; ksc[sj][1][1 % nblk] = a.w;
-            ksc[sj][2][0] = bq.x; ksc[sj][2][1 % nblk] = bq.y; ksc[sj][3][0] = bq.z; ksc[sj][3][1 % nblk] = bq.w;
-          } else {
-            const float4 a = *reinterpret_cast<const float4*>(sclc);
-            ksc[sj][0][0] = a.x; ksc[sj][1][0] = a.y; ksc[sj][2][0] = a.z; ksc[sj][3][0] = a.w;
-          }
-        }
-      }
-      f32x4 st[2];
-      st[0] = f32x4{0.f, 0.f, 0.f, 0.f};
-      st[1] = st[0];
-      if (all_plain) {
-        // one sub-tile after the other: the second one's operands are still landing
-#pragma unroll
-        for (int sj = 0; sj < 2; ++sj) {
-          mfma_s8<0>(st[sj], kf[sj][0], qh[0], kexp[sj], qexp);
-          mfma_s8<0>(st[sj], kf[sj][0], ql[0], kexp[sj], qexp);
-          mfma_s8<1>(st[sj], kf[sj][1], qh[1], kexp[sj], qexp);
-          mfma_s8<1>(st[sj], kf[sj][1], ql[1], kexp[sj], qexp);
-          mfma_s8<2>(st[sj], kf[sj][2], qh[2], kexp[sj], qexp);
-          mfma_s8<2>(st[sj], kf[sj][2], ql[2], kexp[sj], qexp);
-          mfma_s8<3>(st[sj], kf[sj][3], qh[3], kexp[sj], qexp);
-          mfma_s8<3>(st[sj], kf[sj][3], ql[3], kexp[sj], qexp);
-          mfma_s(st[sj], rf[sj][0], qr[0]);
-          mfma_s(st[sj], rf[sj][1], qr[1]);
-        }
-      } else {
-        // each block is accumulated apart and enters the score times its keys' mantissa factors; the
-        // two sub-tiles alternate so that a block's factors are applied under the other's products
-        auto block = [&](auto blk_c) {
-          constexpr int blk = decltype(blk_c)::value;
-          f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0;
-          mfma_s8<blk>(a0, kf[0][blk], qh[blk], kexp[0], qexp);
-          mfma_s8<blk>(a1, kf[1][blk], qh[blk], kexp[1], qexp);
-          mfma_s8<blk>(a0, kf[0][blk], ql[blk], kexp[0], qexp);
-          mfma_s8<blk>(a1, kf[1][blk], ql[blk], kexp[1], qexp);
+      // scales of keys 16 sj + 4 kg + i, one per block: they multiply the block's partial sums here and
+      // the probabilities that go to the value product of that block
+      float ksc[4][nblk];                           // of one sub-tile at a time
+      auto load_scales = [&](int sj) {
+        const float* sclc = scl_base + (16 * sj + 4 * kg) * nblk;
+        if (nblk == 4) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            st[0][i] += scale_mant(ksc[0][i][(blk * nblk) >> 2]) * a0[i];
-            st[1][i] += scale_mant(ksc[1][i][(blk * nblk) >> 2]) * a1[i];
+            const float4 v4 = *reinterpret_cast<const float4*>(sclc + 4 * i);
+            ksc[i][0] = v4.x; ksc[i][1 % nblk] = v4.y; ksc[i][2 % nblk] = v4.z; ksc[i][3 % nblk] = v4.w;
           }
+        } else if (nblk == 2) {
+          const float4 a = *reinterpret_cast<const float4*>(sclc), bq = *reinterpret_cast<const float4*>(sclc + 4);
+          ksc[0][0] = a.x; ksc[0][1 % nblk] = a.y; ksc[1][0] = a.z; ksc[1][1 % nblk] = a.w;
+          ksc[2][0] = bq.x; ksc[2][1 % nblk] = bq.y; ksc[3][0] = bq.z; ksc[3][1 % nblk] = bq.w;
+        } else {
+          const float4 a = *reinterpret_cast<const float4*>(sclc);
+          ksc[0][0] = a.x; ksc[1][0] = a.y; ksc[2][0] = a.z; ksc[3][0] = a.w;
+        }
+      };
+      load_k(tau, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      // per sub-tile: the rope part first (it needs no scale); then each latent block is accumulated
+      // apart, from zero, and enters the score times its keys' block scales.  Two blocks alternate so
+      // that a block's scales are applied under the next products.
+      f32x4 st[2];
+      auto subtile = [&](auto sj_c) {
+        constexpr int sj = decltype(sj_c)::value;
+        load_scales(sj);
+        st[sj] = f32x4{0.f, 0.f, 0.f, 0.f};
+        mfma_s(st[sj], rf[sj][0], qr[0]);
+        mfma_s(st[sj], rf[sj][1], qr[1]);
+        auto pair = [&](auto b_c) {
+          constexpr int b0 = decltype(b_c)::value, b1 = b0 + 1;
+          f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0;
+          mfma_s8<b0>(a0, kf[sj][b0], qh[b0], kOne, qexp);
+          mfma_s8<b1>(a1, kf[sj][b1], qh[b1], kOne, qexp);
+          mfma_s8<b0>(a0, kf[sj][b0], ql[b0], kOne, qexp);
+          mfma_s8<b1>(a1, kf[sj][b1], ql[b1], kOne, qexp);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st[sj][i] = __builtin_fmaf(ksc[i][(b0 * nblk) >> 2], a0[i], st[sj][i]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st[sj][i] = __builtin_fmaf(ksc[i][(b1 * nblk) >> 2], a1[i], st[sj][i]);
         };
-        block(std::integral_constant<int, 0>{});
-        block(std::integral_constant<int, 1>{});
-        block(std::integral_constant<int, 2>{});
-        block(std::integral_constant<int, 3>{});
-        mfma_s(st[0], rf[0][0], qr[0]);
-        mfma_s(st[1], rf[1][0], qr[0]);
-        mfma_s(st[0], rf[0][1], qr[1]);
-        mfma_s(st[1], rf[1][1], qr[1]);
-      }
+        pair(std::integral_constant<int, 0>{});
+        pair(std::integral_constant<int, 2>{});
+      };
+      subtile(std::integral_constant<int, 0>{});
+      asm volatile("" ::: "memory");
+      subtile(std::integral_constant<int, 1>{});
 
       __builtin_amdgcn_sched_barrier(0);
-      // The scale reads issued before the products have long landed: say so before the next batch of
-      // reads.  (The LDS counter holds 15 at most; without this the compiler, unable to name "all
-      // but the last 22", makes the first use of a scale wait for most of that batch.)
-      __builtin_amdgcn_s_waitcnt(0xc07f);           // lgkmcnt(0)
-      if (next) load_k(tau + 1);                    // (the fragment registers are free again)
+      // (the scales are read again for the probabilities rather than kept: the registers go to the next tile's operands)
+      if (next) load_k(tau + 1, 0);                 // (the fragment registers are free again)
       __builtin_amdgcn_sched_barrier(0);
       // ---- softmax: this lane holds head n, keys 16 sj + 4 kg + i ----
       float mx;
       float mul = qk_scale;                         // what turns a held sum into a base-2 score
       if (all_valid) {
         // no skipped key: the maximum is taken on the raw sums (qk_scale > 0 on this path)
-        // (fmaxf, not the raw instruction: the compiler pads the wait states a vector instruction
-        // needs before it may read matrix results only for instructions it can see)
         mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
                    fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
       } else {
@@ -520,20 +464,26 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       }
       // exp2(-inf - m) is 0 for a finite m; a head with no valid key yet keeps m_run = -inf
       const float neg_m = -vmax(m_run, -1.0e30f);
-      unsigned char* pdst = smem + kPOff + spar * kPBytes;
+      // P -> LDS in the B-operand layout of the 32x32x16 product: lane (head of a 32-head block,
+      // key/8) owns 16 bytes = 8 keys; this lane holds keys 4kg..4kg+3.  One plane per scale block:
+      // plane b is P times the keys' scales of block b (fp32 product, rounded to bf16 once), so the
+      // value product of block b takes V's bytes unscaled.
+      unsigned char* pdst = smem + kPOff + spar * kPBytes + ((role >> 1) * 64 + (role & 1) * 16 + n + (kg >> 1) * 32) * 16 + (kg & 1) * 8;
 #pragma unroll
       for (int sj = 0; sj < 2; ++sj) {
+        asm volatile("" ::: "memory");
+        load_scales(sj);
         float pr[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           pr[i] = fast_exp2(__builtin_fmaf(st[sj][i], mul, neg_m));
           l_run += pr[i];
         }
-        // P -> LDS in the B-operand layout of the 32x32x16 product: lane (head of a 32-head block,
-        // key/8) owns 16 bytes = 8 keys; this lane holds keys 4kg..4kg+3.  (V's block scales are
-        // applied by the consumers, each for its own channel block.)
-        unsigned char* dst = pdst + ((sj * 2 + (role >> 1)) * 64 + (role & 1) * 16 + n + (kg >> 1) * 32) * 16 + (kg & 1) * 8;
-        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(pr[0], pr[1]), pack_bf16(pr[2], pr[3]));
+#pragma unroll
+        for (int pb = 0; pb < nblk; ++pb) {
+          *reinterpret_cast<uint2*>(pdst + pb * kPPlane + sj * 2048) =
+              make_uint2(pack_bf16(pr[0] * ksc[0][pb], pr[1] * ksc[1][pb]), pack_bf16(pr[2] * ksc[2][pb], pr[3] * ksc[3][pb]));
+        }
       }
     };
 
@@ -542,7 +492,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     for (int t = -1; t < n_tiles; ++t) {
       __syncthreads();
       // (the first barrier only promises tile 0: tile 1's operands are read a round late, once)
-      if (t <= 0 && t + 1 < n_tiles) load_k(t + 1);
+      if (t <= 0 && t + 1 < n_tiles) load_k(t + 1, 0);
       if (t + 1 < n_tiles) produce(t + 1, t >= 0 && t + 2 < n_tiles);
     }
     l_run += xor16(l_run);
@@ -569,17 +519,14 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   //            128 c + 32 kg + 16 j .. + 15 of key 16 sj + n
   //   rope   : plane (sj = c / 2, s = c % 2): lane (n, kq) fetches bytes 64 s + 16 kq .. + 15 of the rope row
   //   scales : element 64c + lane of [32 rows][nblk]
-  //   scales, transposed : (nblk > 1) the wavefronts after those: element 64 (c - nblk/2) + lane of [nblk][32 rows]
   const bool scale_op = has_scale && 64 * role < kTK * nblk;
-  const bool tr_op = has_scale && nblk > 1 && !scale_op && 64 * (role - nblk / 2) < kTK * nblk;
-  const int tr_elem = 64 * (role - nblk / 2) + lane;          // (block, row) = (tr_elem / 32, tr_elem % 32)
   const size_t group_row0 = ((size_t)b * p.Skv_pitch) * p.G + g;     // cache row of key 0; key k is G rows further per step
   const int sc_elem = 64 * role + lane;
   const int sc_row = min(sc_elem / nblk, kTK - 1);
   const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + 128 * role + 32 * (lane >> 4);
   const unsigned char* rope_src = (const unsigned char*)p.rope + group_row0 * (kRope * 2) + 64 * (role & 1) + 16 * (lane >> 4);
   const unsigned char* sc_src = (const unsigned char*)p.kv_scale +
-                                (group_row0 * nblk + (unsigned)(tr_op ? (tr_elem >> 5) & (nblk - 1) : sc_elem % nblk)) * 4;
+                                (group_row0 * nblk + (unsigned)(sc_elem % nblk)) * 4;
   const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = (unsigned)p.G * nblk * 4;
   auto dma16 = [&](const unsigned char* src, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
@@ -597,7 +544,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     dma_slot = smem_base + (unsigned)(tau % kRing) * kSlotBytes;
     const int* tk = keys + tau * kTK;
     const int k0 = tk[lane & 15], k1 = tk[16 + (lane & 15)];        // this lane's key of sub-tile 0 / 1
-    const int ksc_row = scale_op ? tk[sc_row] : tr_op ? tk[tr_elem & 31] : 0;
+    const int ksc_row = scale_op ? tk[sc_row] : 0;
     dma_r0 = (size_t)(unsigned)max(k0, 0);
     dma_r1 = (size_t)(unsigned)max(k1, 0);
     dma_rs = (size_t)(unsigned)max(ksc_row, 0);
@@ -610,8 +557,6 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     else if (i == 4) dma16(rope_src + ((role >> 1) ? dma_r1 : dma_r0) * rope_step, dma_slot + kLatBytes + role * 1024);
     else if (scale_op) {
       if (sc_elem < kTK * nblk) dma4(sc_src + dma_rs * sc_step, dma_slot + kLatBytes + kRopeBytes + 256 * role);
-    } else if (tr_op) {
-      dma4(sc_src + dma_rs * sc_step, dma_slot + kLatBytes + kRopeBytes + kScaleT + 256 * (role - nblk / 2));
     }
   };
   auto issue_tile = [&](int tau) {
@@ -621,7 +566,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   };
   // wait until at most `tiles` of the most recently issued tiles are still in flight
   auto wait_outstanding = [&](int tiles) {
-    const int per = (scale_op || tr_op) ? 6 : 5;
+    const int per = scale_op ? 6 : 5;
     switch (min(tiles, 5) * per) {
       case 30: asm volatile("s_waitcnt vmcnt(30)" ::: "memory"); break;
       case 25: asm volatile("s_waitcnt vmcnt(25)" ::: "memory"); break;
@@ -667,23 +612,12 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   auto consume = [&](int tv, bool next, bool dma) {
     const int vpar = tv & 1;
     if (dma) dma_prepare(tv + kAhead);
-    const unsigned char* pfrag = smem + kPOff + vpar * kPBytes + lane * 16;
+    const unsigned char* pfrag = smem + kPOff + vpar * kPBytes + pvar * kPPlane + lane * 16;
     bf16x8 pb[2][2];
 #pragma unroll
     for (int kstep = 0; kstep < 2; ++kstep)
 #pragma unroll
       for (int hb = 0; hb < 2; ++hb) pb[kstep][hb] = *reinterpret_cast<const bf16x8*>(pfrag + (kstep * 2 + hb) * 1024);
-    // V's scales of this wavefront's channel block for the lane's eight keys of each step
-    float4 vs[2][2];
-    if (has_scale) {
-      const float* tr = reinterpret_cast<const float*>(smem + (tv % kRing) * kSlotBytes + kLatBytes + kRopeBytes + (nblk > 1 ? kScaleT : 0)) +
-                        pvar * kTK + 8 * (lane >> 5);
-#pragma unroll
-      for (int kstep = 0; kstep < 2; ++kstep) {
-        vs[kstep][0] = *reinterpret_cast<const float4*>(tr + 16 * kstep);
-        vs[kstep][1] = *reinterpret_cast<const float4*>(tr + 16 * kstep + 4);
-      }
-    }
     const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
     i32x2 v1[4];
     load_v(tv, 1, v1);
@@ -698,24 +632,6 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
         for (int dvb = 0; dvb < 4; ++dvb)
 #pragma unroll
           for (int j = 0; j < 16; ++j) o[dvb][hb][j] *= fsc;
-      }
-    }
-    if (has_scale) {
-      // P times V's block scale (fp32 product, rounded to bf16 again): V itself is converted unscaled
-#pragma unroll
-      for (int kstep = 0; kstep < 2; ++kstep) {
-        const float sc[8] = {vs[kstep][0].x, vs[kstep][0].y, vs[kstep][0].z, vs[kstep][0].w,
-                             vs[kstep][1].x, vs[kstep][1].y, vs[kstep][1].z, vs[kstep][1].w};
-#pragma unroll
-        for (int hb = 0; hb < 2; ++hb) {
-          const uint4 w = __builtin_bit_cast(uint4, pb[kstep][hb]);
-          const unsigned in[4] = {w.x, w.y, w.z, w.w};
-          unsigned outw[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            outw[i] = pack_bf16(__uint_as_float(in[i] << 16) * sc[2 * i], __uint_as_float(in[i] & 0xffff0000u) * sc[2 * i + 1]);
-          pb[kstep][hb] = __builtin_bit_cast(bf16x8, make_uint4(outw[0], outw[1], outw[2], outw[3]));
-        }
       }
     }
     bf16x8 a[4];
