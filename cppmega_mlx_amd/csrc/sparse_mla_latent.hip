@@ -156,6 +156,12 @@ __device__ __forceinline__ float vmax(float a, float b) {
   return r;
 }
 
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // maximum over lanes l, l^16, l^32, l^48 (every lane gets it): a row swap leaves each value next
 // to its partner's
 __device__ __forceinline__ float max_rows(float v) {
@@ -360,22 +366,20 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     };
     constexpr int kOne = 0x7f7f7f7f;                // operand exponent bytes of 2^0: the key bytes enter the products unscaled
 
-    // scores and probabilities of tile tau (whose K operands are in registers) -> P(tau) in LDS;
-    // `next`: tile tau+1 exists (it has landed)
-    auto produce = [&](int tau, bool next) {
+    // scores and probabilities of tile tau (the operands of its first sub-tile are in registers) ->
+    // P(tau) in LDS.  The common tile - every key valid, no head's maximum above its reference by
+    // more than 2^kLazy - is written straight away, a sub-tile's probabilities under the other's
+    // products, with its block scales still in registers; the maxima are looked at afterwards, and
+    // a tile that moves a reference, or holds skipped keys, is written again the careful way.
+    auto produce = [&](int tau) {
       const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
       const int spar = tau & 1;
       const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
       const bool all_valid = tvalid[tau] != 0;      // (uniform) no skipped key in this tile
-      int4 kk[2] = {make_int4(0, 0, 0, 0), make_int4(0, 0, 0, 0)};
-      if (!all_valid) {
-#pragma unroll
-        for (int sj = 0; sj < 2; ++sj) kk[sj] = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * sj + 4 * kg);
-      }
+      load_k(tau, 1);
       // scales of keys 16 sj + 4 kg + i, one per block: they multiply the block's partial sums here and
       // the probabilities that go to the value product of that block
-      float ksc[4][nblk];                           // of one sub-tile at a time
-      auto load_scales = [&](int sj) {
+      auto load_scales = [&](int sj, float (&ksc)[4][nblk]) {
         const float* sclc = scl_base + (16 * sj + 4 * kg) * nblk;
         if (nblk == 4) {
 #pragma unroll
@@ -392,15 +396,15 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
           ksc[0][0] = a.x; ksc[1][0] = a.y; ksc[2][0] = a.z; ksc[3][0] = a.w;
         }
       };
-      load_k(tau, 1);
-      __builtin_amdgcn_sched_barrier(0);
+      float ks0[4][nblk], ks1[4][nblk];
+      load_scales(0, ks0);
+      load_scales(1, ks1);
       // per sub-tile: the rope part first (it needs no scale); then each latent block is accumulated
       // apart, from zero, and enters the score times its keys' block scales.  Two blocks alternate so
       // that a block's scales are applied under the next products.
       f32x4 st[2];
-      auto subtile = [&](auto sj_c) {
+      auto subtile = [&](auto sj_c, const float (&ksc)[4][nblk]) {
         constexpr int sj = decltype(sj_c)::value;
-        load_scales(sj);
         st[sj] = f32x4{0.f, 0.f, 0.f, 0.f};
         mfma_s(st[sj], rf[sj][0], qr[0]);
         mfma_s(st[sj], rf[sj][1], qr[1]);
@@ -419,22 +423,44 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
         pair(std::integral_constant<int, 0>{});
         pair(std::integral_constant<int, 2>{});
       };
-      subtile(std::integral_constant<int, 0>{});
-      asm volatile("" ::: "memory");
-      subtile(std::integral_constant<int, 1>{});
-
-      __builtin_amdgcn_sched_barrier(0);
-      // (the scales are read again for the probabilities rather than kept: the registers go to the next tile's operands)
-      if (next) load_k(tau + 1, 0);                 // (the fragment registers are free again)
-      __builtin_amdgcn_sched_barrier(0);
-      // ---- softmax: this lane holds head n, keys 16 sj + 4 kg + i ----
+      // P -> LDS in the B-operand layout of the 32x32x16 product: lane (head of a 32-head block,
+      // key/8) owns 16 bytes = 8 keys; this lane holds keys 4kg..4kg+3.  One plane per scale block:
+      // plane b is P times the keys' scales of block b (fp32 product, rounded to bf16 once), so the
+      // value product of block b takes V's bytes unscaled.
+      unsigned char* pdst = smem + kPOff + spar * kPBytes + ((role >> 1) * 64 + (role & 1) * 16 + n + (kg >> 1) * 32) * 16 + (kg & 1) * 8;
+      float l_add = 0.0f;
+      auto emit = [&](int sj, const float (&ksc)[4][nblk], float mul, float neg_m) {
+        float pr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pr[i] = fast_exp2(__builtin_fmaf(st[sj][i], mul, neg_m));
+          l_add += pr[i];
+        }
+#pragma unroll
+        for (int pb = 0; pb < nblk; ++pb) {
+          *reinterpret_cast<uint2*>(pdst + pb * kPPlane + sj * 2048) =
+              make_uint2(pack_bf16(pr[0] * ksc[0][pb], pr[1] * ksc[1][pb]), pack_bf16(pr[2] * ksc[2][pb], pr[3] * ksc[3][pb]));
+        }
+      };
+      // (a head with no valid key yet has m_run = -inf: its tile is always written the careful way)
+      const float neg_m0 = -vmax(m_run, -1.0e30f);
+      subtile(std::integral_constant<int, 0>{}, ks0);
+      subtile(std::integral_constant<int, 1>{}, ks1);
+      load_k(tau + 1, 0);                           // (the fragment registers are free again; a tile that does not exist reads as garbage nobody uses)
+      if (all_valid) {
+        emit(0, ks0, qk_scale, neg_m0);
+        emit(1, ks1, qk_scale, neg_m0);
+      }
+      // ---- the tile's maxima: this lane holds head n, keys 16 sj + 4 kg + i ----
       float mx;
       float mul = qk_scale;                         // what turns a held sum into a base-2 score
       if (all_valid) {
         // no skipped key: the maximum is taken on the raw sums (qk_scale > 0 on this path)
-        mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
-                   fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
+        mx = vmax3(vmax3(st[0][0], st[0][1], st[0][2]), vmax3(st[0][3], st[1][0], st[1][1]), vmax(st[1][2], st[1][3]));
       } else {
+        int4 kk[2];
+#pragma unroll
+        for (int sj = 0; sj < 2; ++sj) kk[sj] = *reinterpret_cast<const int4*>(keys + tau * kTK + 16 * sj + 4 * kg);
         mx = -INFINITY;
 #pragma unroll
         for (int sj = 0; sj < 2; ++sj) {
@@ -448,11 +474,12 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
         mul = 1.0f;
       }
       mx = max_rows(mx) * mul;                 // over the four key quarters (lanes n, n+16, n+32, n+48)
-      {
-        const bool grow = mx > m_run + kLazy;
+      const bool grow = mx > m_run + kLazy;
+      const bool any_grow = __ballot(grow) != 0ull;           // (uniform)
+      bool any_rescale = false;
+      if (any_grow) {
         // accumulators of a head whose reference was -inf are still zero: nothing to rescale
-        const bool rescale = grow && m_run != -INFINITY;
-        const bool any_rescale = __ballot(rescale) != 0ull;
+        any_rescale = __ballot(grow && m_run != -INFINITY) != 0ull;
         float fac = 1.0f;
         if (grow) {
           fac = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - mx);
@@ -460,31 +487,16 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
           m_run = mx;
         }
         if (any_rescale && lane < 16) facbuf[(spar * 4 + role) * 16 + n] = fac;
-        if (lane == 0) flagbuf[spar * 4 + role] = any_rescale ? 1 : 0;
       }
-      // exp2(-inf - m) is 0 for a finite m; a head with no valid key yet keeps m_run = -inf
-      const float neg_m = -vmax(m_run, -1.0e30f);
-      // P -> LDS in the B-operand layout of the 32x32x16 product: lane (head of a 32-head block,
-      // key/8) owns 16 bytes = 8 keys; this lane holds keys 4kg..4kg+3.  One plane per scale block:
-      // plane b is P times the keys' scales of block b (fp32 product, rounded to bf16 once), so the
-      // value product of block b takes V's bytes unscaled.
-      unsigned char* pdst = smem + kPOff + spar * kPBytes + ((role >> 1) * 64 + (role & 1) * 16 + n + (kg >> 1) * 32) * 16 + (kg & 1) * 8;
-#pragma unroll
-      for (int sj = 0; sj < 2; ++sj) {
-        asm volatile("" ::: "memory");
-        load_scales(sj);
-        float pr[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pr[i] = fast_exp2(__builtin_fmaf(st[sj][i], mul, neg_m));
-          l_run += pr[i];
-        }
-#pragma unroll
-        for (int pb = 0; pb < nblk; ++pb) {
-          *reinterpret_cast<uint2*>(pdst + pb * kPPlane + sj * 2048) =
-              make_uint2(pack_bf16(pr[0] * ksc[0][pb], pr[1] * ksc[1][pb]), pack_bf16(pr[2] * ksc[2][pb], pr[3] * ksc[3][pb]));
-        }
+      if (lane == 0) flagbuf[spar * 4 + role] = any_rescale ? 1 : 0;
+      if (any_grow || !all_valid) {
+        // the careful way: exp2(-inf - m) is 0 for a finite m; a head with no valid key yet keeps m_run = -inf
+        const float neg_m = -vmax(m_run, -1.0e30f);
+        l_add = 0.0f;
+        emit(0, ks0, mul, neg_m);
+        emit(1, ks1, mul, neg_m);
       }
+      l_run += l_add;
     };
 
     // t = -1: [X] tile 0 has landed.  t >= 0: [B_t] tile t+2 has landed, P(t) is complete, the value
@@ -493,7 +505,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       __syncthreads();
       // (the first barrier only promises tile 0: tile 1's operands are read a round late, once)
       if (t <= 0 && t + 1 < n_tiles) load_k(t + 1, 0);
-      if (t + 1 < n_tiles) produce(t + 1, t >= 0 && t + 2 < n_tiles);
+      if (t + 1 < n_tiles) produce(t + 1);
     }
     l_run += xor16(l_run);
     l_run += xor32(l_run);
