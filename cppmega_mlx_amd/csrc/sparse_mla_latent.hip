@@ -523,75 +523,60 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   stage_keys();
   __syncthreads();                                // keys[] is complete
   const int n_tiles = count_tiles();
-  // HBM -> LDS: this wavefront brings rows 8c .. 8c+7 of a tile.  A skipped key fetches cache
-  // row 0 instead (its probability is zero), so every tile is the same number of load
-  // instructions and the in-order load counter can be waited on by count.  The loads are inline
-  // assembly: the compiler would otherwise order every later LDS read behind them.
+  // HBM -> LDS.  A skipped key fetches cache row 0 instead (its probability is zero), so every
+  // tile is the same six load instructions per wavefront and the in-order load counter can be
+  // waited on by count.  The loads are inline assembly (the compiler would otherwise order every
+  // later LDS read behind them) with a uniform 64-bit base and a 32-bit byte offset per lane:
   //   latent : block c of both sub-tiles, two planes each: lane (n, kg) of plane j fetches bytes
   //            128 c + 32 kg + 16 j .. + 15 of key 16 sj + n
   //   rope   : plane (sj = c / 2, s = c % 2): lane (n, kq) fetches bytes 64 s + 16 kq .. + 15 of the rope row
-  //   scales : element 64c + lane of [32 rows][nblk]
-  const bool scale_op = has_scale && 64 * role < kTK * nblk;
+  //   scales : elements 8 nblk c .. 8 nblk (c + 1) - 1 of [32 rows][nblk], one per lane (without
+  //            scales in memory: a word nobody reads, so that the count stays six)
   const size_t group_row0 = ((size_t)b * p.Skv_pitch) * p.G + g;     // cache row of key 0; key k is G rows further per step
-  const int sc_elem = 64 * role + lane;
+  const unsigned char* lat_base = (const unsigned char*)p.kv + group_row0 * kLat;
+  const unsigned char* rope_base = (const unsigned char*)p.rope + group_row0 * (kRope * 2);
+  const unsigned char* sc_base = has_scale ? (const unsigned char*)p.kv_scale + group_row0 * nblk * 4 : (const unsigned char*)p.kv;
+  const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = has_scale ? (unsigned)p.G * nblk * 4 : 0u;
+  const unsigned lat_lane = 128u * role + 32u * (lane >> 4), rope_lane = 64u * (role & 1) + 16u * (lane >> 4);
+  const int sc_elem = 8 * nblk * role + lane;                         // (lanes below 8 nblk)
+  const unsigned sc_lane = has_scale ? 4u * (unsigned)(sc_elem % nblk) : 0u;
   const int sc_row = min(sc_elem / nblk, kTK - 1);
-  const unsigned char* lat_src = (const unsigned char*)p.kv + group_row0 * kLat + 128 * role + 32 * (lane >> 4);
-  const unsigned char* rope_src = (const unsigned char*)p.rope + group_row0 * (kRope * 2) + 64 * (role & 1) + 16 * (lane >> 4);
-  const unsigned char* sc_src = (const unsigned char*)p.kv_scale +
-                                (group_row0 * nblk + (unsigned)(sc_elem % nblk)) * 4;
-  const unsigned lat_step = (unsigned)p.G * kLat, rope_step = (unsigned)p.G * (kRope * 2), sc_step = (unsigned)p.G * nblk * 4;
-  auto dma16 = [&](const unsigned char* src, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+  const bool sc_active = lane < 8 * nblk;
+  const unsigned sc_dst = kLatBytes + kRopeBytes + (has_scale ? 32u * nblk * role : 256u);
+  auto dma16 = [&](const unsigned char* base, unsigned off, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
   };
-  auto dma4 = [&](const unsigned char* src, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src) : "memory", "m0");
+  auto dma4 = [&](const unsigned char* base, unsigned off, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
   };
   const unsigned smem_base = (unsigned)(size_t)(lds_void*)smem;                 // LDS byte address of the ring
-  // one tile is six load instructions (five without a scale instruction): prepare computes the
-  // row numbers, part(i) issues instruction i.  The value product spreads the parts between its
-  // matrix instructions: issuing blocks while the load unit's queue is full.
-  unsigned dma_slot = 0;
-  size_t dma_r0 = 0, dma_r1 = 0, dma_rs = 0;
-  auto dma_prepare = [&](int tau) {
-    dma_slot = smem_base + (unsigned)(tau % kRing) * kSlotBytes;
+  // prepare computes the lanes' byte offsets of a tile, part(i) issues instruction i of it into the
+  // slot at `dma_slot`.  The value product spreads the parts between its matrix instructions:
+  // issuing blocks while the load unit's queue is full.
+  unsigned dma_slot = 0;                          // (uniform) LDS address of the slot being filled
+  unsigned off_l0 = 0, off_l1 = 0, off_r = 0, off_s = 0;
+  auto dma_prepare = [&](int tau, unsigned slot_off) {
+    dma_slot = smem_base + slot_off;
     const int* tk = keys + tau * kTK;
-    const int k0 = tk[lane & 15], k1 = tk[16 + (lane & 15)];        // this lane's key of sub-tile 0 / 1
-    const int ksc_row = scale_op ? tk[sc_row] : 0;
-    dma_r0 = (size_t)(unsigned)max(k0, 0);
-    dma_r1 = (size_t)(unsigned)max(k1, 0);
-    dma_rs = (size_t)(unsigned)max(ksc_row, 0);
+    const unsigned k0 = (unsigned)max(tk[lane & 15], 0), k1 = (unsigned)max(tk[16 + (lane & 15)], 0);   // this lane's key of sub-tile 0 / 1
+    const unsigned ks = (unsigned)max(tk[sc_row], 0);
+    off_l0 = __umul24(k0, lat_step) + lat_lane;
+    off_l1 = __umul24(k1, lat_step) + lat_lane;
+    off_r = __umul24((role >> 1) ? k1 : k0, rope_step) + rope_lane;
+    off_s = __umul24(ks, sc_step) + sc_lane;
   };
   auto dma_part = [&](int i) {
-    if (i == 0) dma16(lat_src + dma_r0 * lat_step, dma_slot + role * kPair);
-    else if (i == 1) dma16(lat_src + dma_r0 * lat_step + 16, dma_slot + role * kPair + kPlane);
-    else if (i == 2) dma16(lat_src + dma_r1 * lat_step, dma_slot + (4 + role) * kPair);
-    else if (i == 3) dma16(lat_src + dma_r1 * lat_step + 16, dma_slot + (4 + role) * kPair + kPlane);
-    else if (i == 4) dma16(rope_src + ((role >> 1) ? dma_r1 : dma_r0) * rope_step, dma_slot + kLatBytes + role * 1024);
-    else if (scale_op) {
-      if (sc_elem < kTK * nblk) dma4(sc_src + dma_rs * sc_step, dma_slot + kLatBytes + kRopeBytes + 256 * role);
-    }
+    if (i == 0) dma16(lat_base, off_l0, dma_slot + role * kPair);
+    else if (i == 1) dma16(lat_base, off_l0 + 16u, dma_slot + role * kPair + kPlane);
+    else if (i == 2) dma16(lat_base, off_l1, dma_slot + (4 + role) * kPair);
+    else if (i == 3) dma16(lat_base, off_l1 + 16u, dma_slot + (4 + role) * kPair + kPlane);
+    else if (i == 4) dma16(rope_base, off_r, dma_slot + kLatBytes + role * 1024);
+    else if (sc_active) dma4(sc_base, off_s, dma_slot + sc_dst);
   };
   auto issue_tile = [&](int tau) {
-    dma_prepare(tau);
+    dma_prepare(tau, (unsigned)(tau % kRing) * kSlotBytes);
 #pragma unroll
     for (int i = 0; i < 6; ++i) dma_part(i);
-  };
-  // wait until at most `tiles` of the most recently issued tiles are still in flight
-  auto wait_outstanding = [&](int tiles) {
-    const int per = scale_op ? 6 : 5;
-    switch (min(tiles, 5) * per) {
-      case 30: asm volatile("s_waitcnt vmcnt(30)" ::: "memory"); break;
-      case 25: asm volatile("s_waitcnt vmcnt(25)" ::: "memory"); break;
-      case 24: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
-      case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
-      case 18: asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); break;
-      case 15: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
-      case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-      case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-      case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-      case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
-      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    }
   };
 
   // ---- value side state: o[dvb][hb] = O^T[32 channels x 32 heads] ----
@@ -603,28 +588,31 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
 #pragma unroll
       for (int j = 0; j < 16; ++j) o[i][hb][j] = 0.0f;
   const int pvar = (role * nblk) >> 2;                         // scale block of channels 128c..
-  int pv_off[4];                                               // transposing-read offsets per 32-channel block
+  // transposing reads of V^T: lanes t = 0..15 of a group read 8 bytes each from eight consecutive
+  // keys' 16-byte pieces (128 contiguous bytes); half selects the plane, kq2 the upper eight keys of
+  // the step; the four 32-channel blocks are 256 bytes apart
+  const unsigned char* pv_lane;
   {
-    // lanes t = 0..15 of a group read 8 bytes each from eight consecutive keys' 16-byte pieces (128
-    // contiguous bytes); half selects the plane, kq2 the upper eight keys of the step
     const int t = lane & 15, half = (lane >> 4) & 1, kq2 = lane >> 5;
     const int r = 8 * kq2 + (t >> 1);                          // key within the 16-key step
-#pragma unroll
-    for (int dvb = 0; dvb < 4; ++dvb) pv_off[dvb] = role * kPair + half * kPlane + (dvb * 16 + r) * 16 + 8 * (t & 1);
+    pv_lane = smem + role * kPair + half * kPlane + r * 16 + 8 * (t & 1);
   }
-  // V^T fragments of one 16-key step (four 32-channel blocks), raw
-  auto load_v = [&](int tau, int kstep, i32x2 (&vr)[4]) {
-    const unsigned char* vslot = smem + (tau % kRing) * kSlotBytes + kstep * (4 * kPair);
+  // V^T fragments of one 16-key step (four 32-channel blocks) of the tile in the slot at `slot_off`, raw
+  auto load_v = [&](unsigned slot_off, int kstep, i32x2 (&vr)[4]) {
+    const unsigned char* vslot = pv_lane + slot_off;
 #pragma unroll
     for (int dvb = 0; dvb < 4; ++dvb)
-      vr[dvb] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(vslot + pv_off[dvb]));
+      vr[dvb] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(vslot + kstep * (4 * kPair) + dvb * 256));
   };
+  const unsigned char* p_lane = smem + kPOff + pvar * kPPlane + lane * 16;
   i32x2 v0[4];                                    // first step of the tile about to be consumed (read ahead of the barrier)
-  // value product of tile tv; `next`: tile tv+1 exists (it has landed: the producers are reading it)
-  auto consume = [&](int tv, bool next, bool dma) {
+  // value product of tile tv (in the slot at `cur`); NEXT: tile tv+1 exists (in the slot at `nxt`; it
+  // has landed: the producers are reading it); DMA: tile tv + kAhead exists and goes to the slot at `prv`
+  auto consume = [&](int tv, unsigned cur, unsigned nxt, unsigned prv, auto next_c, auto dma_c) {
+    constexpr bool next = decltype(next_c)::value, dma = decltype(dma_c)::value;
     const int vpar = tv & 1;
-    if (dma) dma_prepare(tv + kAhead);
-    const unsigned char* pfrag = smem + kPOff + vpar * kPBytes + pvar * kPPlane + lane * 16;
+    if (dma) dma_prepare(tv + kAhead, prv);
+    const unsigned char* pfrag = p_lane + vpar * kPBytes;
     bf16x8 pb[2][2];
 #pragma unroll
     for (int kstep = 0; kstep < 2; ++kstep)
@@ -632,7 +620,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       for (int hb = 0; hb < 2; ++hb) pb[kstep][hb] = *reinterpret_cast<const bf16x8*>(pfrag + (kstep * 2 + hb) * 1024);
     const int4 fl = *reinterpret_cast<const int4*>(flagbuf + vpar * 4);
     i32x2 v1[4];
-    load_v(tv, 1, v1);
+    load_v(cur, 1, v1);
     __builtin_amdgcn_sched_barrier(0);
     if (__builtin_amdgcn_readfirstlane(fl.x | fl.y | fl.z | fl.w) != 0) {      // producers moved a reference: rescale (rare)
 #pragma unroll
@@ -656,7 +644,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       mfma_o(o[dvb][1], a[dvb], pb[0][1]);
       if (dma) dma_part(dvb);
     }
-    if (next) load_v(tv + 1, 0, v0);
+    if (next) load_v(nxt, 0, v0);
 #pragma unroll
     for (int dvb = 0; dvb < 4; ++dvb) a[dvb] = cvt8((unsigned)v1[dvb][0], (unsigned)v1[dvb][1]);
     __builtin_amdgcn_sched_barrier(0);
@@ -672,19 +660,42 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   // only the first tile is requested ahead of the first barrier (issuing blocks while the load
   // unit's queue is full, and the producers cannot start before this wavefront gets there)
   if (n_tiles > 0) issue_tile(0);
-  wait_outstanding(0);                            // tile 0 has landed
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // tile 0 has landed
   __syncthreads();                                // [X]
 #pragma unroll
   for (int tau = 1; tau < kAhead; ++tau)
     if (tau < n_tiles) issue_tile(tau);
-  if (n_tiles > 0) load_v(0, 0, v0);
-  wait_outstanding(max(min(kAhead, n_tiles) - 3, 0));   // tile 2 has landed
-  for (int t = 0; t < n_tiles; ++t) {
-    __syncthreads();                              // [B_t]
-    const bool more = t + kAhead < n_tiles;
-    consume(t, t + 1 < n_tiles, more);            // (tile t+4 goes into the slot of tile t-1)
-    // tile t+3 must have landed before the next barrier; the tile issued after it may stay in flight
-    wait_outstanding(max(min(t + kAhead, n_tiles - 1) - (t + 3), 0));
+  if (n_tiles > 0) load_v(0u, 0, v0);
+  // tile 2 has landed (a fourth tile may stay in flight)
+  if (n_tiles >= kAhead) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  {
+    // slots of tile t, t + 1 and t - 1 (= the slot tile t + kAhead goes to), as byte offsets into the ring
+    unsigned cur = 0, nxt = kSlotBytes, prv = (kRing - 1) * kSlotBytes;
+    auto advance = [&]() {
+      prv = cur;
+      cur = nxt;
+      nxt = nxt + kSlotBytes == kRingBytes ? 0u : nxt + kSlotBytes;
+    };
+    const int n_steady = max(n_tiles - kAhead, 0);
+    int t = 0;
+    for (; t < n_steady; ++t) {
+      __syncthreads();                              // [B_t]
+      consume(t, cur, nxt, prv, std::true_type{}, std::true_type{});     // (tile t+4 goes into the slot of tile t-1)
+      // tile t+3 must have landed before the next barrier; the tile just issued may stay in flight
+      asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+      advance();
+    }
+    for (; t < n_tiles - 1; ++t) {
+      __syncthreads();                              // [B_t]
+      consume(t, cur, nxt, prv, std::true_type{}, std::false_type{});
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      advance();
+    }
+    if (t < n_tiles) {
+      __syncthreads();                              // [B_t], the last tile
+      consume(t, cur, nxt, prv, std::false_type{}, std::false_type{});
+    }
   }
   __syncthreads();                                // [E] statistics are visible; the ring is free
 
@@ -906,6 +917,8 @@ bool sparse_mla_latent_supported(const MlaParams& p) {
   if (((uintptr_t)p.q | (uintptr_t)p.kv | (uintptr_t)p.rope) & 15) return false;
   if (p.kv_scale && ((uintptr_t)p.kv_scale & 3)) return false;
   if ((unsigned long long)p.B * p.Skv_pitch * p.G >= 0x7fffffffull) return false;   // cache rows are counted in 32 bits
+  // a lane's byte offset from the first row of its batch is a 24-bit row number times a 24-bit step, below 2^31
+  if ((unsigned long long)p.Skv_pitch * p.G * kLat >= (1ull << 31) || p.Skv_pitch >= (1 << 24) || (long long)p.G * kLat >= (1 << 24)) return false;
   if (p.topk > 16 * kMaxKeys) return false;       // the combine step merges at most 16 key splits
   return true;
 }
