@@ -298,7 +298,7 @@ class QuantizeArgs(C.Structure):
     ]
 
 
-QUANT_PER_TOKEN, QUANT_PER_TENSOR, QUANT_MXFP8, DEQUANT_PER_TOKEN, DEQUANT_MXFP8 = range(5)
+QUANT_PER_TOKEN, QUANT_PER_TENSOR, QUANT_MXFP8, DEQUANT_PER_TOKEN, DEQUANT_MXFP8, QUANT_UNIT, DEQUANT_UNIT = range(7)
 
 
 class CacheAppendArgs(C.Structure):

@@ -134,6 +134,21 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(const QuantParams 
 }
 
 
+// the bare conversions: codes = rne(clamp(x, +-448)) / recovered = dec(codes)
+template <bool ENCODE>
+__global__ __launch_bounds__(256) void unit_convert_kernel(const QuantParams p) {
+  const size_t n = (size_t)p.rows * p.k;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    if (ENCODE) {
+      const float v = load_as(p.x, i, p.x_dtype);
+      const unsigned code = v != v ? (((__float_as_uint(v) >> 24) & 0x80u) | 0x7fu) : e4m3_encode(fminf(fmaxf(v, -448.0f), 448.0f));
+      p.codes[i] = (unsigned char)code;
+    } else {
+      store_as(p.recovered, i, p.x_dtype, e4m3_to_f32(p.in_codes[i]));
+    }
+  }
+}
+
 // ---- cache append -------------------------------------------------------------------------
 struct AppendParams {
   const void* src;
@@ -248,7 +263,7 @@ int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stre
   if (a.rows < 0 || a.k < 1) return fail(CPPMEGA_MI355_ERR_SHAPE, "fp8_quantize: rows=%lld k=%d", (long long)a.rows, a.k);
   if (a.x_dtype != CPPMEGA_MI355_F32 && a.x_dtype != CPPMEGA_MI355_F16 && a.x_dtype != CPPMEGA_MI355_BF16)
     return fail(CPPMEGA_MI355_ERR_DTYPE, "fp8_quantize: dtype %d is not float32/float16/bfloat16", a.x_dtype);
-  if (a.mode < CPPMEGA_MI355_QUANT_PER_TOKEN || a.mode > CPPMEGA_MI355_DEQUANT_MXFP8)
+  if (a.mode < CPPMEGA_MI355_QUANT_PER_TOKEN || a.mode > CPPMEGA_MI355_DEQUANT_UNIT)
     return fail(CPPMEGA_MI355_ERR_SHAPE, "fp8_quantize: unknown mode %d", a.mode);
   const bool mx = a.mode == CPPMEGA_MI355_QUANT_MXFP8 || a.mode == CPPMEGA_MI355_DEQUANT_MXFP8;
   if (mx && a.k % 32 != 0) return fail(CPPMEGA_MI355_ERR_SHAPE, "fp8_quantize: MXFP8 last dim must be divisible by 32, got %d", a.k);
@@ -256,6 +271,16 @@ int fp8_quantize_launch(const cppmega_mi355_quantize_args_t& a, hipStream_t stre
   QuantParams p;
   p.x = a.x; p.codes = a.codes; p.scale = a.scale; p.recovered = a.recovered; p.in_codes = a.codes;
   p.rows = a.rows; p.k = a.k; p.x_dtype = a.x_dtype; p.mode = a.mode;
+  if (a.mode == CPPMEGA_MI355_QUANT_UNIT || a.mode == CPPMEGA_MI355_DEQUANT_UNIT) {
+    const bool enc = a.mode == CPPMEGA_MI355_QUANT_UNIT;
+    if (!a.codes || (enc ? !a.x : !a.recovered)) return fail(CPPMEGA_MI355_ERR_NULL, "fp8_quantize: the bare conversions need codes and %s", enc ? "x" : "recovered");
+    const size_t n = (size_t)a.rows * a.k;
+    const unsigned blocks = (unsigned)min((n + 255) / 256, (size_t)65535 * 16);
+    if (enc) hipLaunchKernelGGL(unit_convert_kernel<true>, dim3(blocks), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(unit_convert_kernel<false>, dim3(blocks), dim3(256), 0, stream, p);
+    CM_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
   if (a.mode >= CPPMEGA_MI355_DEQUANT_PER_TOKEN) {
     if (!a.codes || !a.scale || !a.recovered) return fail(CPPMEGA_MI355_ERR_NULL, "fp8_dequantize: codes/scale/recovered is NULL");
     const size_t n = (size_t)a.rows * a.k;

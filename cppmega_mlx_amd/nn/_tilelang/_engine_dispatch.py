@@ -116,7 +116,34 @@ def _launch_mla(q_kind: int, kv_kind: int, block: int):
     return run
 
 
+def _launch_float_mla(bufs: dict, attrs: dict):
+    B, S, H, G, Skv, topk, K, dv = (int(attrs[n]) for n in ("B", "S", "H", "G", "Skv", "topk", "K", "d_v"))
+    ops.sparse_mla_forward(
+        bufs["q"].view(B, S, H, K), bufs["kv"].view(B, Skv, G, K), bufs["indices"].view(B, S, G, topk),
+        sm_scale=bufs["sm_scale_buf"], d_v=dv, out=bufs["out"].view(B, S, H, dv), lse=bufs["lse"].view(B, S, H))
+
+
+def _launch_float_mla_bwd(bufs: dict, attrs: dict):
+    B, S, H, G, Skv, topk, K, dv = (int(attrs[n]) for n in ("B", "S", "H", "G", "Skv", "topk", "K", "d_v"))
+    ops.sparse_mla_backward(
+        bufs["q"].view(B, S, H, K), bufs["kv"].view(B, Skv, G, K), bufs["d_out"].view(B, S, H, dv),
+        bufs["indices"].view(B, S, G, topk), sm_scale=bufs["sm_scale_buf"], d_v=dv,
+        dq=bufs["dq"].view(B, S, H, K), dkv=bufs["dkv"].view(B, Skv, G, K), clear_dkv=bool(attrs.get("clear_dkv", True)))
+
+
+def _launch_latent_mla(bufs: dict, attrs: dict):
+    B, S, H, G, Skv, topk, K, R, dv, block = (int(attrs[n]) for n in ("B", "S", "H", "G", "Skv", "topk", "K", "R", "d_v", "scale_block"))
+    ops.sparse_mla_forward(
+        bufs["q"].view(B, S, H, K + R), bufs["kv_fp8"].view(B, Skv, G, K), bufs["indices"].view(B, S, G, topk),
+        sm_scale=bufs["sm_scale_buf"], d_v=dv, out=bufs["out"].view(B, S, H, dv), lse=bufs["lse"].view(B, S, H),
+        kv_spec=ops.QuantSpec(_lib.SCALE_F32_BLOCK, bufs["kv_scale"].view(B, Skv, G, K // block), block),
+        kv_rope=bufs["kv_rope"].view(B, Skv, G, R), sinks=bufs.get("sinks"), has_sinks=bufs.get("has_sinks"))
+
+
 _LAUNCHERS: dict[str, Callable[[dict, dict], None]] = {
+    "sparse_mla_float": _launch_float_mla,
+    "sparse_mla_float_bwd": _launch_float_mla_bwd,
+    "sparse_mla_latent": _launch_latent_mla,
     "topk_selector": _launch_topk,
     "fp8_vecmat": _launch_vecmat,
     "sparse_mla_blockscaled": _launch_mla(_lib.SCALE_E8M0, _lib.SCALE_E8M0, 32),
@@ -147,6 +174,32 @@ def fp8_mla_spec(**shape) -> KernelSpec:
     return KernelSpec("sparse_mla_fp8",
                       ("q_fp8", "q_scale", "kv_fp8", "kv_scale", "indices", "sm_scale_buf", "sinks", "has_sinks",
                        "out", "lse"), (8, 9), shape)
+
+
+def float_mla_spec(**shape) -> KernelSpec:
+    """kernel(indices, kv, lse, out, q, sm_scale_buf), out_idx=[2, 3]: the float-carrier forward
+    (sparse_mla_fwd_direct, sparse_mla_path_c.py:2291-2299, compiled with out_idx=[2, 3] at :3068 and called
+    as kernel(indices, kv, q, sm_scale_buf, out=(lse, out)) at :3282-3288).  Carriers: float16 (the
+    reference's), bfloat16 or float32."""
+    return KernelSpec("sparse_mla_float", ("indices", "kv", "lse", "out", "q", "sm_scale_buf"), (2, 3), shape)
+
+
+def float_mla_bwd_spec(**shape) -> KernelSpec:
+    """kernel(d_out, dkv, dq, indices, kv, q, sm_scale_buf), out_idx=[1, 2]: the float-carrier backward
+    (sparse_mla_bwd_direct, sparse_mla_path_c.py:2670-2678, out_idx=[1, 2] at :3159); dkv is float32 and is
+    cleared first unless ``clear_dkv=False`` (the reference clears it with a kernel of its own, :3163-3230)."""
+    return KernelSpec("sparse_mla_float_bwd", ("d_out", "dkv", "dq", "indices", "kv", "q", "sm_scale_buf"), (1, 2), shape)
+
+
+def latent_mla_spec(**shape) -> KernelSpec:
+    """kernel(q, kv_fp8, kv_scale, kv_rope, indices, sm_scale_buf, sinks, has_sinks, out, lse), out_idx=[8, 9]: the
+    block-scaled forward over a latent cache - bfloat16 q [.., K + R], e4m3 latent [.., K] with one float32 scale
+    per ``scale_block`` channels, bfloat16 rope tail [.., R].  The reference has no PrimFunc for this layout; the
+    order is that of its per-token FP8 kernel (sparse_mla_fp8_path_c.py:1821-1835) with the rope tail after the
+    key scales and no query scale."""
+    return KernelSpec("sparse_mla_latent",
+                      ("q", "kv_fp8", "kv_scale", "kv_rope", "indices", "sm_scale_buf", "sinks", "has_sinks", "out", "lse"),
+                      (8, 9), shape)
 
 
 class NativeHipKernel:

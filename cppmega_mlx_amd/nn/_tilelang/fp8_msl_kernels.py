@@ -17,7 +17,7 @@ import torch
 
 from ... import _lib, ops
 
-__all__ = ["FP8MSLKernelStatus", "fp8_msl_status", "fp8_scaled_vecmat"]
+__all__ = ["FP8MSLKernelStatus", "fp8_msl_status", "fp8_scaled_vecmat", "fp8_to_half", "half_to_fp8"]
 
 
 @dataclass(frozen=True)
@@ -33,6 +33,26 @@ def fp8_msl_status() -> FP8MSLKernelStatus:
 def _check_dtype(name: str, arr: torch.Tensor, expected: torch.dtype) -> None:
     if arr.dtype != expected:
         raise TypeError(f"fp8_msl_kernels.{name}: expected dtype {expected}, got {arr.dtype}")
+
+
+def fp8_to_half(fp8_uchar: torch.Tensor) -> torch.Tensor:
+    """uint8 e4m3fn storage -> float16 (cppmega_mlx/nn/_tilelang/fp8_msl_kernels.py:65-71).  Allocates
+    its result, as the reference does."""
+    _check_dtype("fp8_to_half", fp8_uchar, torch.uint8)
+    out = torch.zeros(fp8_uchar.shape, dtype=torch.float16, device=fp8_uchar.device)
+    if fp8_uchar.numel() == 0:
+        return out
+    return ops.e4m3_convert(fp8_uchar.contiguous(), out=out)
+
+
+def half_to_fp8(half_arr: torch.Tensor) -> torch.Tensor:
+    """float16 -> e4m3fn bytes, round to nearest even, saturating at +-448
+    (cppmega_mlx/nn/_tilelang/fp8_msl_kernels.py:74-81)."""
+    _check_dtype("half_to_fp8", half_arr, torch.float16)
+    out = torch.zeros(half_arr.shape, dtype=torch.uint8, device=half_arr.device)
+    if half_arr.numel() == 0:
+        return out
+    return ops.e4m3_convert(half_arr.contiguous(), out=out)
 
 
 def _resolve_scale(scale, *, length: int, name: str, device) -> Tuple[torch.Tensor, int]:

@@ -190,10 +190,10 @@ class _SparseMLAPathCFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, cotangent):
         q, kv, indices = ctx.saved_tensors
-        grads = sparse_mla_bwd_path_c(q, kv, cotangent.to(q.dtype).contiguous(), indices)
-        if grads is None:
-            raise SparseMLAPathCDirectError("sparse-MLA backward kernels are unavailable")
-        dq, dkv = grads
+        # (the direct form: a carrier or shape error surfaces as what it is instead of as "unavailable")
+        shapes = _resolve_shapes(q, kv, indices, d_v=None)
+        buf = torch.tensor([shapes.qk_dim ** -0.5], dtype=torch.float32, device=q.device)
+        dq, dkv = _sparse_mla_bwd_path_c_direct(q, kv, cotangent.to(q.dtype).contiguous(), indices, sm_scale_buf=buf, d_v=shapes.d_v)
         return dq, dkv.to(kv.dtype), None
 
 

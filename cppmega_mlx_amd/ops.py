@@ -454,7 +454,15 @@ def sparse_mla_backward(q: torch.Tensor, kv: torch.Tensor, d_out: torch.Tensor, 
     if q.ndim != 4 or kv.ndim != 4 or indices.ndim != 4:
         raise ValueError("sparse_mla: q, kv and indices must be rank 4")
     B, S, H, D = q.shape
-    _, Skv, G, _ = kv.shape
+    Bk, Skv, G, Dk = kv.shape
+    if Bk != B or Dk != D:
+        raise ValueError(f"kv must have shape ({B}, Skv, G, {D}) to go with q {tuple(q.shape)}; got {tuple(kv.shape)}")
+    if G < 1 or H % G:
+        raise ValueError(f"heads {H} not divisible by kv_group {G}")
+    if tuple(indices.shape[:3]) != (B, S, G):
+        raise ValueError(f"indices shape {tuple(indices.shape)} does not match (B,S,G,topk)=({B},{S},{G},*)")
+    if not 0 < int(d_v) <= D:
+        raise ValueError(f"d_v must be in (0, {D}], got {int(d_v)}")
     if tuple(d_out.shape) != (B, S, H, int(d_v)):
         raise ValueError(f"d_out must have shape {(B, S, H, int(d_v))}; got {tuple(d_out.shape)}")
     if tuple(dq.shape) != (B, S, H, D):
@@ -665,6 +673,32 @@ def fp8_dequantize(codes: torch.Tensor, scale: torch.Tensor, *, out: torch.Tenso
     with torch.cuda.device(codes.device):
         rc = _lib.load().cppmega_mi355_fp8_quantize(C.byref(a), C.sizeof(a), _lib.current_stream(codes.device))
     _lib.check(rc, "fp8_dequantize")
+    return out
+
+
+def e4m3_convert(src: torch.Tensor, *, out: torch.Tensor) -> torch.Tensor:
+    """The bare e4m3 conversions into a caller-owned buffer of the same shape: float16 / bfloat16 /
+    float32 ``src`` -> uint8 codes (round to nearest even, saturating at +-448), or uint8 codes ->
+    their float values in ``out``'s dtype."""
+    _lib.require_device_tensor(src, "src", None)
+    _lib.require_device_tensor(out, "out", src)
+    if tuple(src.shape) != tuple(out.shape) or not (src.is_contiguous() and out.is_contiguous()):
+        raise ValueError("e4m3_convert: src and out must be contiguous tensors of one shape")
+    a = _lib.QuantizeArgs()
+    a.struct_size = C.sizeof(a)
+    if src.dtype == torch.uint8:
+        a.mode, a.x_dtype = _lib.DEQUANT_UNIT, _dtype_or_raise(out, "out", (_lib.F32, _lib.F16, _lib.BF16))
+        a.codes, a.recovered = src.data_ptr(), out.data_ptr()
+    else:
+        if out.dtype != torch.uint8:
+            raise TypeError(f"e4m3_convert: codes must be uint8, got {out.dtype}")
+        a.mode, a.x_dtype = _lib.QUANT_UNIT, _dtype_or_raise(src, "src", (_lib.F32, _lib.F16, _lib.BF16))
+        a.x, a.codes = src.data_ptr(), out.data_ptr()
+    a.rows, a.k = src.numel(), 1
+    if src.numel():
+        with torch.cuda.device(src.device):
+            rc = _lib.load().cppmega_mi355_fp8_quantize(C.byref(a), C.sizeof(a), _lib.current_stream(src.device))
+        _lib.check(rc, "e4m3_convert")
     return out
 
 

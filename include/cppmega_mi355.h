@@ -472,6 +472,10 @@ int cppmega_mi355_dequant_block_fp8(const cppmega_mi355_dequant_block_args_t* ar
  *               codes saturate at +-448
  *   DEQUANT_*   _from_fp8_with_scale (sparse_mla_fp8.py:148-157) / _dequantize_mxfp8
  *               (sparse_mla_blockscaled.py:79-87): recovered = dec(codes) * scale
+ *   QUANT_UNIT / DEQUANT_UNIT   half_to_fp8 / fp8_to_half
+ *               (cppmega_mlx/nn/_tilelang/fp8_msl_kernels.py:65-81): the bare conversions,
+ *               code = rne(clamp(x, +-448)) (NaN -> the NaN code of its sign) and
+ *               recovered = dec(codes); no scale is read or written
  * x is [rows, k] float32/float16/bfloat16, dense.  Any of codes / scale / recovered may be
  * NULL in a quantise call (at least one is not); `recovered` receives dec(code) * scale in
  * x's dtype.  PER_TENSOR needs `scratch`, 4 bytes of device memory. */
@@ -480,7 +484,9 @@ enum {
   CPPMEGA_MI355_QUANT_PER_TENSOR = 1,
   CPPMEGA_MI355_QUANT_MXFP8 = 2,
   CPPMEGA_MI355_DEQUANT_PER_TOKEN = 3,   /* codes + float32 scale[rows] -> recovered */
-  CPPMEGA_MI355_DEQUANT_MXFP8 = 4        /* codes + uint8 scale[rows, k/32] -> recovered */
+  CPPMEGA_MI355_DEQUANT_MXFP8 = 4,       /* codes + uint8 scale[rows, k/32] -> recovered */
+  CPPMEGA_MI355_QUANT_UNIT = 5,          /* x -> codes, scale 1                           */
+  CPPMEGA_MI355_DEQUANT_UNIT = 6         /* codes -> recovered, scale 1                   */
 };
 
 typedef struct cppmega_mi355_quantize_args {

@@ -193,3 +193,104 @@ def test_dispatched_kernels_replay_from_a_hip_graph(device):
         np.testing.assert_array_equal(
             captured["idx"].cpu().numpy(),
             otk.topk_selector_oracle(scores.cpu().numpy(), k, starts=starts.cpu().numpy(), ends=ends.cpu().numpy(), order="value"))
+
+
+def test_float_carrier_mla_kernels_from_dispatch_lower(device):
+    """The float-carrier forward in the reference's order kernel(indices, kv, lse, out, q, sm_scale_buf) with
+    out_idx=[2, 3] (sparse_mla_path_c.py:2291-2299, 3068, 3282-3288) and the backward kernel(d_out, dkv, dq,
+    indices, kv, q, sm_scale_buf) with out_idx=[1, 2] (:2670-2678, 3159), float16 carriers as in the reference."""
+    rng = np.random.default_rng(46)
+    B, S, H, G, Skv, topk, K, dv = 2, 3, 8, 2, 80, 20, 64, 32
+    shape = dict(B=B, S=S, H=H, G=G, Skv=Skv, topk=topk, K=K, d_v=dv)
+    q16 = rng.standard_normal((B, S, H, K)).astype(np.float16)
+    kv16 = rng.standard_normal((B, Skv, G, K)).astype(np.float16)
+    idx = sparse_indices(rng, B, S, G, Skv, topk, causal_offset=30)
+    idx[:, :, :, -2:] = -1
+    q, kv, ind = to_dev(q16, device).reshape(-1), to_dev(kv16, device).reshape(-1), to_dev(idx.astype(np.int32), device).reshape(-1)
+    sm = torch.tensor([0.2], dtype=torch.float32, device=device)
+    fwd = ed.dispatch_lower(ed.float_mla_spec(**shape), "gfx950")
+    assert fwd.result_indices == (2, 3)
+    lse = torch.zeros(B * S * H, dtype=torch.float32, device=device)
+    out = torch.zeros(B * S * H * dv, dtype=torch.float16, device=device)
+    got = fwd(ind, kv, q, sm, out=(lse, out))
+    torch.cuda.synchronize()
+    assert got[0] is lse and got[1] is out
+    want_out, want_lse = om.sparse_mla_oracle(q16.astype(np.float64), kv16.astype(np.float64), idx, sm_scale=0.2, d_v=dv)
+    _check_mla(out, lse, want_out, want_lse)
+
+    bwd = ed.dispatch_lower(ed.float_mla_bwd_spec(**shape), "gfx950")
+    assert bwd.result_indices == (1, 2)
+    d_out16 = rng.standard_normal((B, S, H, dv)).astype(np.float16)
+    dkv = torch.full((B * Skv * G * K,), 7.0, dtype=torch.float32, device=device)      # cleared by the call
+    dq = torch.zeros(B * S * H * K, dtype=torch.float16, device=device)
+    got = bwd(to_dev(d_out16, device).reshape(-1), ind, kv, q, sm, out=(dkv, dq))
+    torch.cuda.synchronize()
+    assert got[0] is dkv and got[1] is dq
+    want_dq, want_dkv = om.sparse_mla_bwd_oracle(q16.astype(np.float64), kv16.astype(np.float64), idx, d_out16.astype(np.float64),
+                                                 sm_scale=0.2, d_v=dv)
+    assert np.abs(dq.float().cpu().numpy().reshape(want_dq.shape) - want_dq).max() <= 2e-2 * np.abs(want_dq).max()
+    assert np.abs(dkv.cpu().numpy().reshape(want_dkv.shape) - want_dkv).max() <= 1e-3 * np.abs(want_dkv).max()
+
+
+def test_latent_cache_mla_kernel_from_dispatch_lower_and_graph_replay(device):
+    """The latent-cache layout (bfloat16 q, e4m3 latent + float32 scales per 128 channels + bfloat16 rope tail)
+    through dispatch_lower on the 64-head kernel with key splits, eager and replayed from a HIP graph with the
+    scale buffer rewritten in between."""
+    from tests._inputs import bf16_pair, latent_cache
+    rng = np.random.default_rng(47)
+    B, S, H, G, Skv, topk = 2, 1, 128, 1, 3000, 1024
+    shape = dict(B=B, S=S, H=H, G=G, Skv=Skv, topk=topk, K=512, R=64, d_v=512, scale_block=128)
+    q, qf = bf16_pair(rng.standard_normal((B, S, H, 576)), device)
+    codes, scale, rope, rows = latent_cache(rng, B, Skv, G, 512, 64, device, pow2=False)
+    idx = sparse_indices(rng, B, S, G, Skv, topk)
+    ind = to_dev(idx.astype(np.int32), device)
+    kernel = ed.dispatch_lower(ed.latent_mla_spec(**shape), "gfx950")
+    assert kernel.result_indices == (8, 9)
+    sm = torch.tensor([576 ** -0.5], dtype=torch.float32, device=device)
+    out = torch.zeros(B * S * H * 512, dtype=torch.bfloat16, device=device)
+    lse = torch.zeros(B * S * H, dtype=torch.float32, device=device)
+    args = (q.reshape(-1), codes.reshape(-1), scale.reshape(-1), rope.reshape(-1), ind.reshape(-1), sm, None, None)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        assert kernel(*args, out=(out, lse))[0] is out
+    stream.synchronize()
+    _check_mla(out, lse, *om.sparse_mla_oracle(qf, rows, idx, sm_scale=576 ** -0.5, d_v=512))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        kernel(*args, out=(out, lse))
+    for scale_value in (0.03, 576 ** -0.5, 0.05):
+        sm.fill_(scale_value)
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _check_mla(out, lse, *om.sparse_mla_oracle(qf, rows, idx, sm_scale=scale_value, d_v=512))
+
+
+def test_bare_e4m3_conversions(device):
+    """fp8_to_half / half_to_fp8 (cppmega_mlx/nn/_tilelang/fp8_msl_kernels.py:65-81): every byte decodes to the
+    oracle's table value; float16 inputs round to nearest even and saturate at +-448; a decode of an encode is
+    the identity on the non-NaN codes."""
+    from cppmega_mlx_amd.nn._tilelang import fp8_msl_kernels as fk
+    codes = np.arange(256, dtype=np.uint8)
+    got = fk.fp8_to_half(to_dev(codes, device))
+    torch.cuda.synchronize()
+    want = fp8.e4m3_decode(codes).astype(np.float32)
+    got_np = got.float().cpu().numpy()
+    ok = ~np.isnan(want)
+    assert got.dtype == torch.float16 and np.array_equal(got_np[ok], want[ok]) and np.isnan(got_np[~ok]).all()
+    rng = np.random.default_rng(48)
+    x = np.concatenate([rng.standard_normal(4000) * 3, rng.standard_normal(500) * 300, fp8.e4m3_decode(codes[ok]),
+                        [0.0, -0.0, 448.0, 449.0, -1000.0, 2.0 ** -10, 2.0 ** -9 * 1.5, 0.0009765625 * 3]]).astype(np.float16)
+    enc = fk.half_to_fp8(to_dev(x, device))
+    torch.cuda.synchronize()
+    assert enc.dtype == torch.uint8
+    np.testing.assert_array_equal(enc.cpu().numpy(), fp8.e4m3_encode(x.astype(np.float64)))
+    back = fk.half_to_fp8(fk.fp8_to_half(to_dev(codes[ok], device)))
+    torch.cuda.synchronize()
+    keep = codes[ok] != 0x80                                    # -0 encodes as it is; compare values for it
+    np.testing.assert_array_equal(back.cpu().numpy()[keep], codes[ok][keep])
+    assert fk.fp8_to_half(torch.zeros((0, 4), dtype=torch.uint8, device=device)).shape == (0, 4)
+    with pytest.raises(TypeError):
+        fk.half_to_fp8(torch.zeros(4, dtype=torch.float32, device=device))
