@@ -108,94 +108,70 @@ struct BinHit {
   unsigned bin, above, cnt, total;
 };
 
+// Inclusive prefix sum over the first N (a power of two, at most 16) lanes of every row of 16.
+template <int N>
+__device__ __forceinline__ unsigned row_inclusive_sum_dpp(unsigned v) {
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);                  // row_shr:1
+  if constexpr (N > 2) v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);   // row_shr:2
+  if constexpr (N > 4) v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);   // row_shr:4
+  if constexpr (N > 8) v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);   // row_shr:8
+  return v;
+}
+
+// Given every wavefront's total in smem[at .. at + WAVES), returns the sum over the wavefronts
+// before this one and the sum over all of them: lanes 0 .. WAVES-1 scan the totals, two lane reads
+// pick the results (a handful of instructions where a loop over the wavefronts costs two each).
+template <int WAVES>
+__device__ __forceinline__ void waves_before_and_total(const unsigned* smem, int at, int lane, int wave, unsigned& before, unsigned& total) {
+  static_assert(WAVES >= 2 && WAVES <= 16 && (WAVES & (WAVES - 1)) == 0, "wavefronts per workgroup");
+  const unsigned incl = row_inclusive_sum_dpp<WAVES>(smem[at + (lane & (WAVES - 1))]);
+  total = (unsigned)__builtin_amdgcn_readlane((int)incl, WAVES - 1);
+  const unsigned upto = (unsigned)__builtin_amdgcn_readlane((int)incl, wave > 0 ? wave - 1 : 0);
+  before = wave > 0 ? upto : 0u;
+}
+
 // Finds the bin at which the running count, walking from the largest value
-// down, first reaches `need`.  All THREADS threads call it.  The NB bins are
-// read as NB/4 aligned quads, thread t taking quads t, t+THREADS, ... so that
-// the 16-byte LDS reads of a wavefront are consecutive (no bank conflicts).
-// Quads [s*THREADS, (s+1)*THREADS) form "segment" s; the walk visits whole
-// segments in a mode-dependent order, ascending or descending inside each.
+// down, first reaches `need`.  All THREADS threads call it.  The walk visits the
+// kHistBins bins in a mode-dependent order; the thread at walk position t takes
+// the run of kHistBins / THREADS consecutive bins that the walk reaches t-th,
+// front to back or back to front as the walk goes: one scan over the threads'
+// run sums finds the thread, which then walks its own run.
 template <int NB, int THREADS>
 __device__ BinHit find_bin(unsigned* smem, unsigned need, int mode) {
-  constexpr int SEGS = NB / 4 / THREADS;
+  static_assert(NB == kHistBins, "the scan walks the whole histogram");
+  constexpr int BPT = NB / THREADS;               // 16, 8 or 4 bins per thread
   constexpr int WAVES = THREADS / 64;
-  static_assert(SEGS >= 1 && SEGS <= 4 && NB == SEGS * 4 * THREADS, "segments");
-  static_assert(SEGS * WAVES <= 16, "scan scratch");
+  static_assert(BPT >= 4 && BPT % 4 == 0 && BPT * THREADS == NB, "bins per thread");
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-  uint4 quad[SEGS];
-  unsigned qsum[SEGS], incl[SEGS];
+  // kSigned: bins 2047..0 (the non-negative values, largest first), then 2048..4095
+  const bool desc = mode == kDescending || (mode == kSigned && tid < THREADS / 2);
+  const int run = mode == kAscending ? tid : mode == kDescending ? THREADS - 1 - tid : (desc ? THREADS / 2 - 1 - tid : tid);
+  unsigned c[BPT];
+  unsigned sum = 0;
 #pragma unroll
-  for (int s = 0; s < SEGS; ++s) {
-    quad[s] = reinterpret_cast<const uint4*>(smem)[s * THREADS + tid];
-    qsum[s] = quad[s].x + quad[s].y + quad[s].z + quad[s].w;
-    incl[s] = wave_inclusive_sum_dpp(qsum[s]);
-    if (lane == 63) smem[kWaveTot + s * WAVES + wave] = incl[s];
+  for (int i = 0; i < BPT / 4; ++i) {
+    const uint4 q = reinterpret_cast<const uint4*>(smem)[run * (BPT / 4) + i];
+    c[4 * i] = q.x; c[4 * i + 1] = q.y; c[4 * i + 2] = q.z; c[4 * i + 3] = q.w;
+    sum += q.x + q.y + q.z + q.w;
   }
+  const unsigned incl = wave_inclusive_sum_dpp(sum);
+  if (lane == 63) smem[kWaveTot + wave] = incl;
   __syncthreads();
-  unsigned wtot[SEGS][WAVES], segtot[SEGS], total = 0;
+  unsigned before, total;
+  waves_before_and_total<WAVES>(smem, kWaveTot, lane, wave, before, total);
+  before += incl - sum;
+  if (before < need && need <= before + sum) {      // exactly one thread when need <= total
+    unsigned walked = before;
 #pragma unroll
-  for (int s = 0; s < SEGS; ++s) {
-    segtot[s] = 0;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      wtot[s][w] = smem[kWaveTot + s * WAVES + w];
-      segtot[s] += wtot[s][w];
-    }
-    total += segtot[s];
-  }
-  // walk step m visits segment seg(m), descending (larger quad index first) when desc(m)
-  unsigned walked = 0;   // elements in segments the walk has finished
-#pragma unroll
-  for (int m = 0; m < SEGS; ++m) {
-    int s; bool desc;
-    if (mode == kAscending) { s = m; desc = false; }
-    else if (mode == kDescending) { s = SEGS - 1 - m; desc = true; }
-    else if constexpr (SEGS == 1) {  // kSigned inside one segment: the lower half of the threads holds bins 2047..0
-      s = 0; desc = tid < THREADS / 2;
-    }
-    else {  // kSigned: bins 2047..0 then 2048..4095 (SEGS is even here)
-      if (m < SEGS / 2) { s = SEGS / 2 - 1 - m; desc = true; } else { s = m; desc = false; }
-    }
-    // (one segment, signed walk: the wavefronts of the other half count as wholly before or after)
-    const bool split_walk = SEGS == 1 && mode == kSigned;
-    // (the loop is unrolled and `s` selects among registers: keep it branch-free over s)
-    unsigned my_sum = 0, my_incl = 0, my_wave_tot = 0, waves_before = 0;
-    uint4 my_quad = make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int ss = 0; ss < SEGS; ++ss) {
-      if (ss == s) {
-        my_sum = qsum[ss]; my_incl = incl[ss]; my_quad = quad[ss]; my_wave_tot = wtot[ss][0];
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) {
-          if (w == wave) my_wave_tot = wtot[ss][w];
-          if (split_walk) {
-            if (desc ? (w > wave && w < WAVES / 2) : (w < wave)) waves_before += wtot[ss][w];
-          } else if (desc ? (w > wave) : (w < wave)) {
-            waves_before += wtot[ss][w];
-          }
-        }
+    for (int i = 0; i < BPT; ++i) {
+      const unsigned n = desc ? c[BPT - 1 - i] : c[i];
+      if (walked < need && need <= walked + n) {
+        smem[kHit + 0] = (unsigned)(run * BPT + (desc ? BPT - 1 - i : i));
+        smem[kHit + 1] = walked;
+        smem[kHit + 2] = n;
       }
+      walked += n;
     }
-    const unsigned lanes_before = desc ? (my_wave_tot - my_incl) : (my_incl - my_sum);
-    const unsigned before = walked + waves_before + lanes_before;
-    if (before < need && need <= before + my_sum) {      // exactly one (thread, m) when need <= total
-      const unsigned cs[4] = {my_quad.x, my_quad.y, my_quad.z, my_quad.w};
-      unsigned run = before;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int slot = desc ? 3 - i : i;
-        const unsigned c = cs[slot];
-        if (run < need && need <= run + c) {
-          smem[kHit + 0] = (unsigned)((s * THREADS + tid) * 4 + slot);
-          smem[kHit + 1] = run;
-          smem[kHit + 2] = c;
-        }
-        run += c;
-      }
-    }
-    walked += (s == 0 ? segtot[0] : 0);
-#pragma unroll
-    for (int ss = 1; ss < SEGS; ++ss) walked += (s == ss ? segtot[ss] : 0);
   }
   __syncthreads();
   BinHit hit;
@@ -224,15 +200,26 @@ __device__ __forceinline__ unsigned order_key(float x) {
 // ---------------------------------------------------------------------------
 constexpr int kTileThreads = 256;
 constexpr int kTileScratch = kHistBins + 64;            // words: histogram + scan scratch
-__host__ __device__ constexpr int tile_pad(int E) { return E == 4 ? 0 : 4; }
+// The row tile is not padded (8192 columns are 32 KiB: four such workgroups fit a CU, and the
+// allocation of a padded tile let only three in).  A thread's run of E columns is E/4 pieces of 16
+// bytes; piece i of thread t sits at position (i + rot(t)) mod E/4 of the run, with rot chosen so
+// that the sixteen lanes of one LDS cycle read sixteen different 16-byte bank groups.
+template <int E>
+__device__ __forceinline__ int tile_piece_slot(int t, int i) {
+  constexpr int PP = E / 4;                               // pieces per thread: 1, 2, 4 or 8
+  if constexpr (PP == 1) return t;
+  constexpr int SH = PP == 2 ? 3 : PP == 4 ? 2 : 1;       // log2(16 / PP)
+  return PP * t + ((i + (t >> SH)) & (PP - 1));
+}
+// both histograms fit the tile's allocation of the widest shape with 64 words to spare
+__host__ __device__ constexpr bool tile_two_hists(int E, int threads) { return threads * E >= 2 * kHistBins; }
 
 // MODE 0: a row per workgroup.  MODE 1: stage 1 of a wide row (a segment per workgroup, candidates
 // out).  MODE 2: stage 2 (a row of candidates per workgroup, positions translated through index_map).
 template <typename ScoreT, int E, int VEC, int THREADS = kTileThreads, int MODE = 0>
-__global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) {
+__global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(const TopkParams p) {
   constexpr int ITEMS = E / VEC;                        // loads per thread
   constexpr int CHUNK = THREADS * VEC;                  // columns covered by one load per thread
-  constexpr int PITCH = E + tile_pad(E);                // words between the runs of consecutive threads
   extern __shared__ __align__(16) unsigned smem[];
   float* tile = reinterpret_cast<float*>(smem);
   unsigned* hist = smem;
@@ -259,7 +246,7 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
     const int chunk_lo = j * CHUNK;
     const int col = chunk_lo + tid * VEC;
     if (chunk_lo >= end || chunk_lo + CHUNK <= start || col >= T) continue;
-    float* dst = tile + col + (col / E) * tile_pad(E);
+    float* dst = tile + 4 * tile_piece_slot<E>(col / E, (col % E) >> 2) + (col & 3);
     if constexpr (VEC == 4) {
       float t4[4];
       ScoreLoad<ScoreT>::vec4(src + col, t4);
@@ -273,12 +260,12 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
   float v[E];
 #pragma unroll
   for (int i = 0; i < E / 4; ++i) {
-    const float4 t4 = *reinterpret_cast<const float4*>(tile + tid * PITCH + 4 * i);
+    const float4 t4 = *reinterpret_cast<const float4*>(tile + 4 * tile_piece_slot<E>(tid, i));
     v[4 * i] = t4.x; v[4 * i + 1] = t4.y; v[4 * i + 2] = t4.z; v[4 * i + 3] = t4.w;
   }
   __syncthreads();
   // two cleared histograms: pass 1 uses the first, pass 2 the second (no clear + barrier in between)
-  constexpr int kHist2 = (THREADS * PITCH >= 2 * kHistBins + 64) ? kHistBins + 64 : 0;
+  constexpr int kHist2 = tile_two_hists(E, THREADS) ? kHistBins + 64 : 0;
   zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
   __syncthreads();
 
@@ -338,8 +325,8 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
       if (rem == h2.cnt) {
         lo_bits = (p2 << 8) | (neg ? 0xffu : 0u);
       } else {
-        // ---- pass 3: bits[7:0] (256 of 1024 cleared slots are used) ------------------
-        constexpr int NB3 = 4 * THREADS > 1024 ? 4 * THREADS : 1024;   // the scan wants one quad per thread at least
+        // ---- pass 3: bits[7:0] (256 of the cleared slots are used) -------------------------
+        constexpr int NB3 = kHistBins;                      // (the scan walks the whole histogram)
         zero_hist<THREADS>(hist, NB3);
         __syncthreads();
 #pragma unroll
@@ -371,13 +358,9 @@ __global__ __launch_bounds__(THREADS) void topk_tile_kernel(const TopkParams p) 
   const unsigned incl = wave_inclusive_sum_dpp(packed);
   if (lane == 63) smem[kWaveTot + wave] = incl;
   __syncthreads();
-  unsigned before = incl - packed, totals = 0;
-#pragma unroll
-  for (int w = 0; w < THREADS / 64; ++w) {
-    const unsigned t = smem[kWaveTot + w];
-    if (w < wave) before += t;
-    totals += t;
-  }
+  unsigned before, totals;
+  waves_before_and_total<THREADS / 64>(smem, kWaveTot, lane, wave, before, totals);
+  before += incl - packed;
   unsigned run_g = before & 0xffffu, run_e = before >> 16;
   const unsigned n_sel = (totals & 0xffffu) + min(totals >> 16, rem);
   const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
@@ -649,8 +632,6 @@ int launch_kernel(K kernel, const TopkParams& p, int threads, size_t smem, hipSt
   return 0;
 }
 
-static int wide_threads() { return 512; }
-
 template <typename ScoreT, int MODE = 0>
 int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* smem_out) {
   const int T = p.segs > 1 ? p.seg_width : p.width;      // columns one workgroup looks at
@@ -658,8 +639,8 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
   const size_t out_words = sorted ? (size_t)p.sort_len * 2 : (size_t)p.k;
   if (T <= 32768) {
     auto tile_smem = [&](int E, int threads) {
-      const size_t tile_words = (size_t)threads * (E + tile_pad(E));
-      const size_t need = (size_t)kTileScratch + out_words;
+      const size_t tile_words = (size_t)threads * E;
+      const size_t need = (size_t)kTileScratch + (tile_two_hists(E, threads) && out_words < (size_t)kHistBins ? (size_t)kHistBins : out_words);
       return (need > tile_words ? need : tile_words) * 4;
     };
 #define CM_TOPK_TILE(E, THR)                                                              \
@@ -678,11 +659,7 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
     if (T <= 4096) CM_TOPK_TILE(16, kTileThreads);
     // the widest rows: 512 threads x 16 columns (twice the wavefronts per row shorten every phase
     // of the row's pipeline, and the narrower runs need fewer registers)
-    if (T <= 8192) {
-      if (wide_threads() == 1024) CM_TOPK_TILE(8, 1024);
-      if (wide_threads() == 512) CM_TOPK_TILE(16, 512);
-      CM_TOPK_TILE(32, kTileThreads);
-    }
+    if (T <= 8192) CM_TOPK_TILE(16, 512);
     // up to 32768 columns: the same kernel on 1024 threads (half the time of the keyed-bin kernel below)
     if (T <= 16384) CM_TOPK_TILE(16, 1024);
     CM_TOPK_TILE(32, 1024);
