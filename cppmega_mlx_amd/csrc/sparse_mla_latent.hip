@@ -194,7 +194,9 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   long long qg;
   int chunk, split;
   {
-    const long long id = blockIdx.x;
+    // (several queries per sequence: the last ones first - under a causal selection they hold the
+    // longest key lists, and the short ones then fill the end of the launch)
+    const long long id = p.S > 1 ? (long long)gridDim.x - 1 - blockIdx.x : (long long)blockIdx.x;
     long long r;
     if (id < nq8 * per_q) {
       const long long slot = id >> 3;
