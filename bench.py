@@ -639,7 +639,8 @@ PROFILE_RUNS = {
     "sq_decode": _PMC.format("sq_decode", "decode_general", 3, _SQ),
     "sq_prefill": _PMC.format("sq_prefill", "prefill_general", 2, _SQ),
 }
-# summary file -> (trace run, (fetch run, write run) or None, SQ run or None, kernel-name fragments, workload text)
+# summary file -> (trace run, (fetch run, write run) or None, SQ run or None, kernel-name fragments, workload text
+#                  [, grid size in threads: only dispatches of that size count])
 PROFILE_WORKLOADS = [
     ("sparse_mla_decode", "trace_main", ("fetch_main", "write_main"), "sq_decode", ("sparse_mla_latent",),
      "decode B=32 S_q=1 H=128 topk=2048 Skv=65536 (e4m3 latent + general fp32/128 scales (amax/448) + bf16 rope)"),
@@ -660,9 +661,10 @@ PROFILE_WORKLOADS = [
     ("fp8_vecmat_m32", "trace_main", ("fetch_main", "write_main"), None, ("skinny_mfma_kernel<2>", "skinny_reduce"),
      "W e4m3[7168,16384] + fp32 scale/128, x bf16[32,16384] (split-K kernel + reduce kernel)"),
     ("topk_selector", "trace_main", ("fetch_main", "write_main"), None, ("topk_tile_kernel<float, 16, 4, 512, 0>",),
-     "scores fp32[4096 rows,8192] -> int32[4096,2048], indices in ascending order"),
+     "scores fp32[4096 rows,8192] -> int32[4096,2048], indices in ascending order (the dispatches of 4096 workgroups only: "
+     "the same kernel also selects for the indexer and for the prefill rows of the same run)", 4096 * 512),
     ("topk_selector_value_order", "trace_alt", None, None, ("topk_tile_kernel<float, 16, 4, 512, 0>",),
-     "scores fp32[4096 rows,8192] -> int32[4096,2048], indices by descending value (same kernel, sorted in LDS)"),
+     "scores fp32[4096 rows,8192] -> int32[4096,2048], indices by descending value (same kernel, sorted in LDS)", 4096 * 512),
     ("topk_selector_decode_shape", "trace_main", ("fetch_main", "write_main"), None,
      ("topk_tile_kernel<float, 16, 4, 512, 1>", "topk_tile_kernel<float, 16, 4, 1024, 2>", "topk_wide_kernel"),
      "scores fp32[32,65536] -> int32[32,2048]: the two-stage path (segment kernel, then candidate kernel) and, for "
@@ -733,10 +735,34 @@ def summarise_profiles(src: str) -> int:
     def short(name):
         return name.replace("(anonymous namespace)::", "")
 
+    trace_cache = {}
+
+    def dispatch_stats(run, name, grid):
+        """Calls / average / min / max (ns) over the dispatches of `name` with `grid` threads."""
+        if run not in trace_cache:
+            trace_cache[run] = rows(f"{run}/t_kernel_trace.csv")
+        ns = [float(r["End_Timestamp"]) - float(r["Start_Timestamp"]) for r in trace_cache[run]
+              if r["Kernel_Name"] == name and int(r["Grid_Size_X"]) == grid]
+        if not ns:
+            return None
+        return {"Calls": str(len(ns)), "AverageNs": sum(ns) / len(ns), "MinNs": min(ns), "MaxNs": max(ns)}
+
+    def counters_by_grid(run, grid):
+        agg = collections.defaultdict(lambda: collections.defaultdict(list))
+        for r in rows(f"{run}/c_counter_collection.csv"):
+            if int(r["Grid_Size"]) == grid:
+                agg[r["Kernel_Name"]][r["Counter_Name"]].append(float(r["Counter_Value"]))
+        return agg
+
     traffic, missing = {}, []
-    for fname, trace_run, pmc_runs, sq_run, frags, workload in PROFILE_WORKLOADS:
+    for entry in PROFILE_WORKLOADS:
+        fname, trace_run, pmc_runs, sq_run, frags, workload = entry[:6]
+        grid = entry[6] if len(entry) > 6 else None
         stats = stats_of(trace_run)
         names = [n for n in stats if "cm::" in n and any(f in n for f in frags)]
+        if grid is not None:
+            stats = {n: dispatch_stats(trace_run, n, grid) for n in names}
+            names = [n for n in names if stats[n]]
         if not names:
             missing.append(fname)
             continue
@@ -749,6 +775,8 @@ def summarise_profiles(src: str) -> int:
                                                               float(r["MinNs"]) / 1e3, float(r["MaxNs"]) / 1e3))
         if pmc_runs:
             fetch, write = counters_of(pmc_runs[0]), counters_of(pmc_runs[1])
+            if grid is not None:
+                fetch, write = counters_by_grid(pmc_runs[0], grid), counters_by_grid(pmc_runs[1], grid)
             (scale_f, copy_f), (scale_w, copy_w) = copy_scale(pmc_runs[0], "FETCH_SIZE"), copy_scale(pmc_runs[1], "WRITE_SIZE")
             text += ["", "## HBM traffic per dispatch (`--pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, KiB)", "",
                      "Commands: " + cmd(pmc_runs[0]) + " and " + cmd(pmc_runs[1]) + ".", "",
