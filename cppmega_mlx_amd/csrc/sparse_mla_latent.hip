@@ -352,11 +352,13 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     // the first one's products.
     i32x8 kf[2][4];
     bf16x8 rf[2][2];
-    auto load_k = [&](int tau, int sj) {
-      const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
+    // (a tile's slot is passed as its byte offset into the ring, a running value: one address
+    // register per slot then reaches every operand of the tile with an immediate offset)
+    auto load_k = [&](unsigned slot_off, int sj) {
+      const unsigned char* slot = smem + (slot_off + (unsigned)lane * 16u);
       // the lane's 32 bytes of a block are its 16 bytes of the block's two planes
-      const unsigned char* lat = slot + sj * (4 * kPair) + lane * 16;
-      const unsigned char* rope = slot + kLatBytes + sj * 2048 + lane * 16;
+      const unsigned char* lat = slot + sj * (4 * kPair);
+      const unsigned char* rope = slot + kLatBytes + sj * 2048;
 #pragma unroll
       for (int blk = 0; blk < 4; ++blk) {
         const uint4 c0 = *reinterpret_cast<const uint4*>(lat + blk * kPair);
@@ -373,12 +375,12 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
     // more than 2^kLazy - is written straight away, a sub-tile's probabilities under the other's
     // products, with its block scales still in registers; the maxima are looked at afterwards, and
     // a tile that moves a reference, or holds skipped keys, is written again the careful way.
-    auto produce = [&](int tau) {
-      const unsigned char* slot = smem + (tau % kRing) * kSlotBytes;
+    auto produce = [&](int tau, unsigned slot_off, unsigned next_off) {
+      const unsigned char* slot = smem + slot_off;
       const int spar = tau & 1;
       const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
       const bool all_valid = tvalid[tau] != 0;      // (uniform) no skipped key in this tile
-      load_k(tau, 1);
+      load_k(slot_off, 1);
       // scales of keys 16 sj + 4 kg + i, one per block: they multiply the block's partial sums here and
       // the probabilities that go to the value product of that block
       auto load_scales = [&](int sj, float (&ksc)[4][nblk]) {
@@ -448,7 +450,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       const float neg_m0 = -vmax(m_run, -1.0e30f);
       subtile(std::integral_constant<int, 0>{}, ks0);
       subtile(std::integral_constant<int, 1>{}, ks1);
-      load_k(tau + 1, 0);                           // (the fragment registers are free again; a tile that does not exist reads as garbage nobody uses)
+      load_k(next_off, 0);                          // (the fragment registers are free again; a tile that does not exist reads as garbage nobody uses)
       if (all_valid) {
         emit(0, ks0, qk_scale, neg_m0);
         emit(1, ks1, qk_scale, neg_m0);
@@ -503,11 +505,14 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
 
     // t = -1: [X] tile 0 has landed.  t >= 0: [B_t] tile t+2 has landed, P(t) is complete, the value
     // product of tile t-1 is done.
+    unsigned s_cur = 0, s_nxt = kSlotBytes;       // ring offsets of the tile produced in this round and of the next one
     for (int t = -1; t < n_tiles; ++t) {
       __syncthreads();
       // (the first barrier only promises tile 0: tile 1's operands are read a round late, once)
-      if (t <= 0 && t + 1 < n_tiles) load_k(t + 1, 0);
-      if (t + 1 < n_tiles) produce(t + 1);
+      if (t <= 0 && t + 1 < n_tiles) load_k(s_cur, 0);
+      if (t + 1 < n_tiles) produce(t + 1, s_cur, s_nxt);
+      s_cur = s_nxt;
+      s_nxt = s_nxt + kSlotBytes == kRingBytes ? 0u : s_nxt + kSlotBytes;
     }
     l_run += xor16(l_run);
     l_run += xor32(l_run);
