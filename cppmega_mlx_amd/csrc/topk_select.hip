@@ -4,13 +4,17 @@
 // with 16-byte loads, and stays in registers for the rest of the kernel; a
 // 4096-bin histogram of the row lives in LDS.
 //
-// Rows of up to 8192 columns (topk_tile_kernel) are staged through LDS once so
-// that every thread ends up owning a contiguous run of columns: a thread's
-// selected columns are then a bit mask, one block-wide prefix sum of the
-// popcounts gives every thread its output offset, and the indices come out in
-// ascending order.  Wider rows (topk_row_kernel, up to 65536 columns) do not
-// fit in LDS; they keep the interleaved ownership of the coalesced loads and
-// compact with per-chunk ballots.
+// In topk_tile_kernel (rows of up to 32768 columns) every thread owns a
+// contiguous run of columns: a thread's selected columns are then a bit mask,
+// one block-wide prefix sum of the popcounts gives every thread its output
+// offset, and the indices come out in ascending order.  Rows whose address and
+// pitch allow 16-byte loads are fetched that way by the owning thread itself,
+// the pieces of a run one load after the other (a wavefront's first load
+// brings in the lines its next ones hit): the histogram can be cleared while
+// the loads travel and no barrier precedes the first pass.  Other rows are
+// loaded a column per lane and reach their owners through an LDS tile.  Wider
+// rows (topk_wide_kernel, up to 65536 columns) keep the interleaved ownership
+// of coalesced loads and compact with per-chunk ballots.
 //
 // Selection (k largest, ties toward the lower index):
 //   pass 1  LDS-atomic histogram of bits[31:20] (sign, exponent, 3 mantissa
@@ -30,8 +34,8 @@
 // Float compares give the ordering: -0.0 == +0.0, and NaN (which also stands
 // for "outside [start,end)") never compares true, so it is never selected.
 // After `x + 0.0f` every NaN is quiet, so NaNs fall into histogram bins no
-// real number can reach (0x7f9..0x7ff, 0xff9..0xfff); those bins are cleared
-// before the scan instead of testing every element.
+// real number can reach (0x7f9..0x7ff, 0xff9..0xfff); the first scan counts
+// those bins as empty instead of every element being tested.
 
 
 #include "common.h"
@@ -136,8 +140,10 @@ __device__ __forceinline__ void waves_before_and_total(const unsigned* smem, int
 // the run of kHistBins / THREADS consecutive bins that the walk reaches t-th,
 // front to back or back to front as the walk goes: one scan over the threads'
 // run sums finds the thread, which then walks its own run.
+// `skip_nan_bins` (first pass only): the bins 0x7f9..0x7ff and 0xff9..0xfff, which no number but only
+// NaN patterns reach, count as empty.
 template <int NB, int THREADS>
-__device__ BinHit find_bin(unsigned* smem, unsigned need, int mode) {
+__device__ BinHit find_bin(unsigned* smem, unsigned need, int mode, bool skip_nan_bins = false) {
   static_assert(NB == kHistBins, "the scan walks the whole histogram");
   constexpr int BPT = NB / THREADS;               // 16, 8 or 4 bins per thread
   constexpr int WAVES = THREADS / 64;
@@ -153,6 +159,14 @@ __device__ BinHit find_bin(unsigned* smem, unsigned need, int mode) {
     const uint4 q = reinterpret_cast<const uint4*>(smem)[run * (BPT / 4) + i];
     c[4 * i] = q.x; c[4 * i + 1] = q.y; c[4 * i + 2] = q.z; c[4 * i + 3] = q.w;
     sum += q.x + q.y + q.z + q.w;
+  }
+  if (skip_nan_bins && ((run * BPT + BPT - 1) & 0x7ff) >= 0x7f9) {      // (two threads, or four)
+    sum = 0;
+#pragma unroll
+    for (int i = 0; i < BPT; ++i) {
+      if (((run * BPT + i) & 0x7ff) >= 0x7f9) c[i] = 0;
+      sum += c[i];
+    }
   }
   const unsigned incl = wave_inclusive_sum_dpp(sum);
   if (lane == 63) smem[kWaveTot + wave] = incl;
@@ -216,8 +230,12 @@ __host__ __device__ constexpr bool tile_two_hists(int E, int threads) { return t
 
 // MODE 0: a row per workgroup.  MODE 1: stage 1 of a wide row (a segment per workgroup, candidates
 // out).  MODE 2: stage 2 (a row of candidates per workgroup, positions translated through index_map).
-template <typename ScoreT, int E, int VEC, int THREADS = kTileThreads, int MODE = 0>
+// DIRECT: a thread fetches its own run of columns from memory, 16 bytes at a time, the pieces of
+// a run one load after the other (the lines a wavefront touches with its first load serve its
+// next ones from the cache): no trip through an LDS tile and no barriers before the first pass.
+template <typename ScoreT, int E, int VEC, int THREADS = kTileThreads, int MODE = 0, bool DIRECT = false>
 __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(const TopkParams p) {
+  static_assert(!DIRECT || VEC == 4, "direct loads are 16-byte loads");
   constexpr int ITEMS = E / VEC;                        // loads per thread
   constexpr int CHUNK = THREADS * VEC;                  // columns covered by one load per thread
   extern __shared__ __align__(16) unsigned smem[];
@@ -240,6 +258,17 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   const float kNegInf = __uint_as_float(0xff800000u);
   const unsigned k = (unsigned)p.k;
 
+  float v[E];
+  if constexpr (DIRECT) {
+    const int c0 = tid * E;
+    const bool any = c0 < end && c0 + E > start;          // (a run with nothing selectable is not read)
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) {
+      float t4[4] = {kNaN, kNaN, kNaN, kNaN};
+      if (any && c0 + 4 * i < T) ScoreLoad<ScoreT>::vec4(src + c0 + 4 * i, t4);
+      v[4 * i] = t4[0]; v[4 * i + 1] = t4[1]; v[4 * i + 2] = t4[2]; v[4 * i + 3] = t4[3];
+    }
+  } else {
   // ---- HBM -> LDS, coalesced; chunks with nothing selectable are not read ----------
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
@@ -257,13 +286,13 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   }
   __syncthreads();
   // ---- LDS -> registers: my contiguous run ------------------------------------------
-  float v[E];
 #pragma unroll
   for (int i = 0; i < E / 4; ++i) {
     const float4 t4 = *reinterpret_cast<const float4*>(tile + 4 * tile_piece_slot<E>(tid, i));
     v[4 * i] = t4.x; v[4 * i + 1] = t4.y; v[4 * i + 2] = t4.z; v[4 * i + 3] = t4.w;
   }
   __syncthreads();
+  }
   // two cleared histograms: pass 1 uses the first, pass 2 the second (no clear + barrier in between)
   constexpr int kHist2 = tile_two_hists(E, THREADS) ? kHistBins + 64 : 0;
   zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
@@ -290,10 +319,8 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
     }
   }
   __syncthreads();
-  if (tid < 7) { hist[0x7f9 + tid] = 0u; hist[0xff9 + tid] = 0u; }   // bins only NaN patterns reach
-  __syncthreads();
 
-  BinHit h1 = find_bin<kHistBins, THREADS>(smem, k, kSigned);
+  BinHit h1 = find_bin<kHistBins, THREADS>(smem, k, kSigned, true);
   float thr;
   unsigned rem = 0;
   bool tie = false;
@@ -648,8 +675,8 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
     const size_t smem = tile_smem(E, THR);                                                \
     *smem_out = smem;                                                                     \
     if (smem > 160 * 1024) return -3;                                                     \
-    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4, THR, MODE>, p, THR, smem, stream) \
-                : launch_kernel(topk_tile_kernel<ScoreT, E, 1, THR, MODE>, p, THR, smem, stream); \
+    return vec4 ? launch_kernel(topk_tile_kernel<ScoreT, E, 4, THR, MODE, true>, p, THR, smem, stream) \
+                : launch_kernel(topk_tile_kernel<ScoreT, E, 1, THR, MODE, false>, p, THR, smem, stream); \
   } while (0)
     if constexpr (MODE == 1) {                            // a segment is always kSegWidth columns wide
       CM_TOPK_TILE(16, 512);
