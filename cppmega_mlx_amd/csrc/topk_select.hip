@@ -373,14 +373,25 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   }
 
   // ---- emission: bit masks, one block-wide prefix sum, ascending indices --------------
-  unsigned gmask = 0, emask = 0;
+  // (the common case - index order, no duplicated threshold - only counts here and compares again
+  // when it writes: a compare and an add-with-carry per element instead of building a mask and
+  // taking it apart)
+  const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
+  const bool plain = !sorted && !tie;
+  unsigned gmask = 0, emask = 0, cg = 0, ce = 0;
+  if (plain) {
 #pragma unroll
-  for (int i = 0; i < E; ++i) {
-    const float x = v[i];
-    gmask |= ((tie ? (x > thr) : (x >= thr)) ? 1u : 0u) << i;
-    if (tie) emask |= ((x == thr) ? 1u : 0u) << i;
+    for (int i = 0; i < E; ++i) cg += (v[i] >= thr) ? 1u : 0u;
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      const float x = v[i];
+      gmask |= ((tie ? (x > thr) : (x >= thr)) ? 1u : 0u) << i;
+      if (tie) emask |= ((x == thr) ? 1u : 0u) << i;
+    }
+    cg = (unsigned)__popc(gmask);
+    ce = (unsigned)__popc(emask);
   }
-  const unsigned cg = (unsigned)__popc(gmask), ce = (unsigned)__popc(emask);
   const unsigned packed = cg | (ce << 16);               // both counts fit in 16 bits (<= 8192)
   const unsigned incl = wave_inclusive_sum_dpp(packed);
   if (lane == 63) smem[kWaveTot + wave] = incl;
@@ -390,13 +401,14 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   before += incl - packed;
   unsigned run_g = before & 0xffffu, run_e = before >> 16;
   const unsigned n_sel = (totals & 0xffffu) + min(totals >> 16, rem);
-  const bool sorted = p.order == CPPMEGA_MI355_TOPK_ORDER_VALUE;
   int* stage = reinterpret_cast<int*>(smem + kTileScratch);
   unsigned long long* pairs = reinterpret_cast<unsigned long long*>(smem + kTileScratch);
-  if (!sorted && !tie) {
+  if (plain) {
 #pragma unroll
     for (int i = 0; i < E; ++i) {
-      if ((gmask >> i) & 1u) stage[run_g++] = col0 + i;
+      const bool g = v[i] >= thr;
+      if (g) stage[run_g] = col0 + i;
+      run_g += g ? 1u : 0u;
     }
   } else {
 #pragma unroll
