@@ -660,13 +660,13 @@ PROFILE_WORKLOADS = [
      "W e4m3[7168,16384] + fp32 scale/128, x bf16[16,16384] (one kernel, no K split, no workspace)"),
     ("fp8_vecmat_m32", "trace_main", ("fetch_main", "write_main"), None, ("skinny_mfma_kernel<2>", "skinny_reduce"),
      "W e4m3[7168,16384] + fp32 scale/128, x bf16[32,16384] (split-K kernel + reduce kernel)"),
-    ("topk_selector", "trace_main", ("fetch_main", "write_main"), None, ("topk_tile_kernel<float, 16, 4, 512, 0>",),
+    ("topk_selector", "trace_main", ("fetch_main", "write_main"), None, ("topk_tile_kernel<float, 16, 4, 512, 0,",),
      "scores fp32[4096 rows,8192] -> int32[4096,2048], indices in ascending order (the dispatches of 4096 workgroups only: "
      "the same kernel also selects for the indexer and for the prefill rows of the same run)", 4096 * 512),
-    ("topk_selector_value_order", "trace_alt", None, None, ("topk_tile_kernel<float, 16, 4, 512, 0>",),
+    ("topk_selector_value_order", "trace_alt", None, None, ("topk_tile_kernel<float, 16, 4, 512, 0,",),
      "scores fp32[4096 rows,8192] -> int32[4096,2048], indices by descending value (same kernel, sorted in LDS)", 4096 * 512),
     ("topk_selector_decode_shape", "trace_main", ("fetch_main", "write_main"), None,
-     ("topk_tile_kernel<float, 16, 4, 512, 1>", "topk_tile_kernel<float, 16, 4, 1024, 2>", "topk_wide_kernel"),
+     ("topk_tile_kernel<float, 16, 4, 512, 1,", "topk_tile_kernel<float, 16, 4, 1024, 2,", "topk_wide_kernel"),
      "scores fp32[32,65536] -> int32[32,2048]: the two-stage path (segment kernel, then candidate kernel) and, for "
      "comparison, the one-workgroup-per-row kernel; the indexer's decode row runs the two-stage kernels as well"),
     ("indexer_scores_topk", "trace_main", ("fetch_main", "write_main"), None, ("indexer_scores_kernel", "indexer_qw_kernel"),
