@@ -380,6 +380,9 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
       const int spar = tau & 1;
       const float* scl_base = reinterpret_cast<const float*>(slot + kLatBytes + kRopeBytes);
       const bool all_valid = tvalid[tau] != 0;      // (uniform) no skipped key in this tile
+      // "no head of this tile moves its reference": written first, so that the common tile ends
+      // without an LDS write the barrier would have to wait for
+      if (lane == 0) flagbuf[spar * 4 + role] = 0;
       load_k(slot_off, 1);
       // scales of keys 16 sj + 4 kg + i, one per block: they multiply the block's partial sums here and
       // the probabilities that go to the value product of that block
@@ -492,7 +495,7 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
         }
         if (any_rescale && lane < 16) facbuf[(spar * 4 + role) * 16 + n] = fac;
       }
-      if (lane == 0) flagbuf[spar * 4 + role] = any_rescale ? 1 : 0;
+      if (any_rescale && lane == 0) flagbuf[spar * 4 + role] = 1;
       if (any_grow || !all_valid) {
         // the careful way: exp2(-inf - m) is 0 for a finite m; a head with no valid key yet keeps m_run = -inf
         const float neg_m = -vmax(m_run, -1.0e30f);
