@@ -59,6 +59,11 @@ struct IndexerParams {
   int b_begin, nb, s_begin, s_count;
   int keys_per_wg;           // multiple of kKeysPerIter
   int q_vec, k_vec, s_vec;   // 16-byte accesses allowed for q rows / k rows / score rows
+  // Selection bounds of the pass's rows (row (b - b_begin) * s_count + (s - s_begin); null = none).
+  // A workgroup scores only the keys some row of its query tile can select: under a causal bound
+  // that is half the matrix.  Not used when the caller asked for the whole score matrix.
+  const int* starts;
+  const int* ends;
   float sm_scale;
 };
 
@@ -127,6 +132,71 @@ __global__ __launch_bounds__(kThreads) void indexer_qw_kernel(const IndexerParam
                  lo[6] | ((unsigned)lo[7] << 16));
 }
 
+// The same head sum with one wavefront per query row, for bf16 rows whose padded width is 32, 64,
+// 128 or 256 channels: a load instruction fetches 1 KiB of the row (64 / chunks heads, neighbouring
+// lanes neighbouring 16 bytes), sixteen of them in flight per lane; the lanes that hold the same
+// channels of different heads meet through lane exchanges in a fixed order.  No LDS, no barrier:
+// a row is a 16 KiB stream at 64 heads of 128 channels, and a CU keeps 32 of them in flight.
+// q is read once, so the loads are non-temporal: with ordinary loads the same kernel streams
+// 128 MiB of query rows at 2.9 TB/s (the lines it allocates in the caches displace each other),
+// with the hint at 5.1 TB/s.
+constexpr int kQwWaves = 4;
+__device__ __forceinline__ uint4 load_once(const uint4* src) {
+  typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
+  return make_uint4(t[0], t[1], t[2], t[3]);
+}
+__global__ __launch_bounds__(kQwWaves * 64) void indexer_qw_wave_kernel(const IndexerParams p) {
+  const int D = p.D, H = p.H;
+  const int Dp = (D + 31) & ~31;
+  const int chunks = Dp / 8;                      // 4, 8, 16 or 32 lanes per head
+  const int hp = 64 / chunks;                     // heads per load instruction
+  const int rows = p.nb * p.s_count;
+  const int lane = (int)threadIdx.x & 63;
+  const int r = (int)blockIdx.x * kQwWaves + ((int)threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int c = lane & (chunks - 1), hs = lane / chunks;
+  const size_t row = (size_t)(p.b_begin + r / p.s_count) * p.Sq + (size_t)(p.s_begin + r % p.s_count);
+  const bool live = 8 * c < D;
+  const uint4* src = reinterpret_cast<const uint4*>((const unsigned short*)p.q + row * H * D + 8 * (live ? c : 0));
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto add = [&](const uint4& t, float wh) {
+    const unsigned u[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc[2 * i] = fmaf(wh, __uint_as_float(u[i] << 16), acc[2 * i]);
+      acc[2 * i + 1] = fmaf(wh, __uint_as_float(u[i] & 0xffff0000u), acc[2 * i + 1]);
+    }
+  };
+  int h = hs;
+  for (; h + 15 * hp < H; h += 16 * hp) {         // sixteen loads in flight
+    uint4 t[16];
+    float wh[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      t[j] = load_once(src + (size_t)(h + j * hp) * (D / 8));
+      wh[j] = load_as(p.w, row * H + h + j * hp, p.w_dtype);
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) add(t[j], wh[j]);
+  }
+  for (; h < H; h += hp) add(load_once(src + (size_t)h * (D / 8)), load_as(p.w, row * H + h, p.w_dtype));
+  for (int off = 32; off >= chunks; off >>= 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], off, 64);
+  }
+  if (lane >= chunks) return;
+  unsigned short hi[8], lo[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) split_bf16(live ? acc[i] : 0.0f, hi[i], lo[i]);
+  const size_t at = (size_t)r * Dp + 8 * c;
+  *reinterpret_cast<uint4*>(p.qw + at) = make_uint4(hi[0] | ((unsigned)hi[1] << 16), hi[2] | ((unsigned)hi[3] << 16),
+                                                    hi[4] | ((unsigned)hi[5] << 16), hi[6] | ((unsigned)hi[7] << 16));
+  *reinterpret_cast<uint4*>(p.qw + (size_t)rows * Dp + at) =
+      make_uint4(lo[0] | ((unsigned)lo[1] << 16), lo[2] | ((unsigned)lo[3] << 16), lo[4] | ((unsigned)lo[5] << 16),
+                 lo[6] | ((unsigned)lo[7] << 16));
+}
+
 // Keys are the MFMA's A rows and 16 queries its B columns: lane (n, kg) holds C rows
 // 4 kg .. 4 kg + 3 of tile j, i.e. four consecutive keys key0 + 16 j + 4 kg + i of query n, and
 // writes them as one 16-byte store; the four lanes of a query cover 64 contiguous bytes.
@@ -175,8 +245,20 @@ __global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerP
   __syncthreads();
 
   const int n = lane & 15, kg = lane >> 4;
-  const int key_begin = (int)blockIdx.x * p.keys_per_wg;
-  const int key_end = min(p.Skv, key_begin + p.keys_per_wg);
+  int key_begin = (int)blockIdx.x * p.keys_per_wg;
+  int key_end = min(p.Skv, key_begin + p.keys_per_wg);
+  if (p.starts || p.ends) {                            // (rows_here <= 64: a lane per row, every wavefront the same)
+    int lo = lane < rows_here && p.starts ? p.starts[out_row0 + lane] : (lane < rows_here ? 0 : p.Skv);
+    int hi = lane < rows_here ? (p.ends ? p.ends[out_row0 + lane] : p.Skv) : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      lo = min(lo, __shfl_xor(lo, off, 64));
+      hi = max(hi, __shfl_xor(hi, off, 64));
+    }
+    lo = max(lo, 0);
+    if (lo > key_begin) key_begin += (lo - key_begin) / kKeysPerIter * kKeysPerIter;
+    key_end = min(key_end, (hi + 63) & ~63);
+  }
   // bf16 keys with 16-byte loads: the next 64 keys are requested before the current ones are used
   constexpr bool kPrefetch = !K_F32 && KSTEPS > 0;
   constexpr int kBuf = kPrefetch ? KSTEPS : 1;
@@ -493,6 +575,7 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
 
   IndexerParams p;
   p.q = a.q; p.w = a.weights; p.k = a.k; p.mask = a.mask; p.scores = scores;
+  p.starts = nullptr; p.ends = nullptr;
   p.qw = (unsigned short*)((char*)a.workspace + pl.score_bytes);
   p.q_dtype = a.q_dtype; p.w_dtype = a.w_dtype; p.k_dtype = a.k_dtype; p.mask_dtype = a.mask_dtype;
   p.B = a.batch; p.Sq = a.seq_q; p.H = a.heads; p.D = a.head_dim; p.Skv = a.seq_kv;
@@ -506,7 +589,17 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
     for (int s_begin = 0; s_begin < a.seq_q; s_begin += pl.rows_per_pass) {
       const int s_count = a.seq_q - s_begin < pl.rows_per_pass ? a.seq_q - s_begin : pl.rows_per_pass;
       p.b_begin = b0; p.nb = nb; p.s_begin = s_begin; p.s_count = s_count;
-      hipLaunchKernelGGL(indexer_qw_kernel, dim3((unsigned)(nb * s_count)), dim3(kThreads), 0, stream, p);
+      if (!a.scores_out) {
+        const size_t first = (size_t)b0 * a.seq_q + (size_t)s_begin;
+        p.starts = a.starts ? a.starts + first : nullptr;
+        p.ends = a.ends ? a.ends + first : nullptr;
+      }
+      const int dp8 = ((a.head_dim + 31) & ~31) / 8;
+      if (p.q_vec && (dp8 & (dp8 - 1)) == 0)
+        hipLaunchKernelGGL(indexer_qw_wave_kernel, dim3((unsigned)((nb * s_count + kQwWaves - 1) / kQwWaves)), dim3(kQwWaves * 64), 0,
+                           stream, p);
+      else
+        hipLaunchKernelGGL(indexer_qw_kernel, dim3((unsigned)(nb * s_count)), dim3(kThreads), 0, stream, p);
       const int qt = (s_count >= 4 * kQRows && a.head_dim <= 128) ? 4 : 1;     // query tiles per workgroup
       const int tiles = (s_count + kQRows * qt - 1) / (kQRows * qt);
       const int max_splits = (a.seq_kv + kKeysPerIter - 1) / kKeysPerIter;
