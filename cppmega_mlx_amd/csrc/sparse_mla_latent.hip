@@ -855,8 +855,11 @@ __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const Ml
     for (int u = 0; u < 4; ++u) {
       const int s = min(s0 + u, p.num_splits - 1);             // a repeated last split gets weight 0
 #pragma unroll
-      for (int i2 = 0; i2 < 2; ++i2)
-        raw[u][i2] = *reinterpret_cast<const uint4*>(src0 + (size_t)s * (HG * kPartFloats) + (size_t)i2 * 512);
+      for (int i2 = 0; i2 < 2; ++i2) {                          // (read once: non-temporal, 0.7 us of the decode step)
+        typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+        const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src0 + (size_t)s * (HG * kPartFloats) + (size_t)i2 * 512));
+        raw[u][i2] = make_uint4(t[0], t[1], t[2], t[3]);
+      }
     }
     float4 v[4][4];
 #pragma unroll
