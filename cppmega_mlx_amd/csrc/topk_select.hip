@@ -438,7 +438,8 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
       return;
     }
     const int* map = MODE == 2 ? p.index_map + (long long)row * p.width : nullptr;
-    for (unsigned i = tid; i < k; i += THREADS) out_row[i] = (i < n_sel) ? (MODE == 2 ? map[stage[i]] : stage[i]) : -1;
+    for (unsigned i = tid; i < k; i += THREADS)             // (written once, not read again here: non-temporal)
+      __builtin_nontemporal_store((i < n_sel) ? (MODE == 2 ? map[stage[i]] : stage[i]) : -1, out_row + i);
     return;
   }
   const int* map = MODE == 2 ? p.index_map + (long long)row * p.width : nullptr;
