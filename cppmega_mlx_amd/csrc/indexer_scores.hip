@@ -299,6 +299,22 @@ __global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerP
         const int row = 16 * jj + n, c = 4 * ks + kg;
         a_off[jj][ks] = (row * PPR + (c ^ ((row / RP) % PPR))) * 16;
       }
+    // The query operands do not change over the keys: they are read from LDS once (128 registers at
+    // four query tiles of 128 channels; one workgroup per CU).  Read inside the loop they were 128 KiB
+    // of LDS traffic per wavefront and 64-key step: 76 -> 71 us at 8192 x 8192 under a causal bound.
+    // (One query tile - the decode-time shape, bound by the key stream - keeps reading them from LDS.)
+    constexpr bool kHoist = QT > 1;
+    bf16x8 bq[kHoist ? QT : 1][kHoist ? KSTEPS : 1][2];
+    if constexpr (kHoist) {
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int d0 = 32 * ks + 8 * kg;
+          bq[qt][ks][0] = *reinterpret_cast<const bf16x8*>(&q_hi[(16 * qt + n) * pitch + d0]);
+          bq[qt][ks][1] = *reinterpret_cast<const bf16x8*>(&q_lo[(16 * qt + n) * pitch + d0]);
+        }
+    }
     if (key_begin + 64 * wave < key_end) fetch_rows(key_begin + 64 * wave, kc);
     for (int key0 = key_begin + 64 * wave; key0 < key_end; key0 += kKeysPerIter) {
       f32x4 acc[QT][4];
@@ -321,11 +337,17 @@ __global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerP
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) {
             const bf16x8 ka = *reinterpret_cast<const bf16x8*>(stage + a_off[jj][ks]);
-            const int d0 = 32 * ks + 8 * kg;
 #pragma unroll
             for (int qt = 0; qt < QT; ++qt) {
-              const bf16x8 b_hi = *reinterpret_cast<const bf16x8*>(&q_hi[(16 * qt + n) * pitch + d0]);
-              const bf16x8 b_lo = *reinterpret_cast<const bf16x8*>(&q_lo[(16 * qt + n) * pitch + d0]);
+              bf16x8 b_hi, b_lo;
+              if constexpr (kHoist) {
+                b_hi = bq[qt][ks][0];
+                b_lo = bq[qt][ks][1];
+              } else {
+                const int d0 = 32 * ks + 8 * kg;
+                b_hi = *reinterpret_cast<const bf16x8*>(&q_hi[(16 * qt + n) * pitch + d0]);
+                b_lo = *reinterpret_cast<const bf16x8*>(&q_lo[(16 * qt + n) * pitch + d0]);
+              }
               acc[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, b_hi, acc[qt][j], 0, 0, 0);
               acc[qt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, b_lo, acc[qt][j], 0, 0, 0);
             }
