@@ -669,7 +669,7 @@ PROFILE_WORKLOADS = [
      ("topk_tile_kernel<float, 16, 4, 512, 1,", "topk_tile_kernel<float, 16, 4, 1024, 2,", "topk_wide_kernel"),
      "scores fp32[32,65536] -> int32[32,2048]: the two-stage path (segment kernel, then candidate kernel) and, for "
      "comparison, the one-workgroup-per-row kernel; the indexer's decode row runs the two-stage kernels as well"),
-    ("indexer_scores_topk", "trace_main", ("fetch_main", "write_main"), None, ("indexer_scores_kernel", "indexer_qw_kernel"),
+    ("indexer_scores_topk", "trace_main", ("fetch_main", "write_main"), None, ("indexer_scores_kernel", "indexer_qw_"),
      "indexer_topk q bf16[B,Sq,64,128], k bf16[B,Skv,128]: prefill (1, 8192, 8192) and decode (32, 1, 65536) dispatches"),
     ("mla_absorb_head_gemm", "trace_main", ("fetch_main", "write_main"), None, ("head_gemm_kernel",),
      "head_gemm x bf16[32,128,128] . W bf16[128,512,128] and x bf16[32,128,512] . W bf16[128,128,512]"),

@@ -38,6 +38,8 @@
 // those bins as empty instead of every element being tested.
 
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace cm {
@@ -175,17 +177,28 @@ __device__ BinHit find_bin(unsigned* smem, unsigned need, int mode, bool skip_na
   waves_before_and_total<WAVES>(smem, kWaveTot, lane, wave, before, total);
   before += incl - sum;
   if (before < need && need <= before + sum) {      // exactly one thread when need <= total
-    unsigned walked = before;
+    // The walk direction is the same for a whole wavefront (a mode, or the half of the workgroup
+    // in the signed pass): a scalar branch picks one of two walks with constant register indices,
+    // and one write follows the walk (with the direction as a per-lane value every step was an
+    // eight-way register select: ~150 instructions that the rest of the row waits for).
+    unsigned hit_i = 0, hit_walked = before, hit_n = 0, walked = before;
+    auto walk = [&](auto dir) {
+      constexpr bool D = decltype(dir)::value;
 #pragma unroll
-    for (int i = 0; i < BPT; ++i) {
-      const unsigned n = desc ? c[BPT - 1 - i] : c[i];
-      if (walked < need && need <= walked + n) {
-        smem[kHit + 0] = (unsigned)(run * BPT + (desc ? BPT - 1 - i : i));
-        smem[kHit + 1] = walked;
-        smem[kHit + 2] = n;
+      for (int i = 0; i < BPT; ++i) {
+        const unsigned n = c[D ? BPT - 1 - i : i];
+        const bool here = walked < need && need <= walked + n;
+        hit_i = here ? (unsigned)(D ? BPT - 1 - i : i) : hit_i;
+        hit_walked = here ? walked : hit_walked;
+        hit_n = here ? n : hit_n;
+        walked += n;
       }
-      walked += n;
-    }
+    };
+    if (__builtin_amdgcn_readfirstlane((int)desc)) walk(std::true_type{});
+    else walk(std::false_type{});
+    smem[kHit + 0] = (unsigned)(run * BPT) + hit_i;
+    smem[kHit + 1] = hit_walked;
+    smem[kHit + 2] = hit_n;
   }
   __syncthreads();
   BinHit hit;
@@ -680,7 +693,8 @@ int launch_for_type(const TopkParams& p, bool vec4, hipStream_t stream, size_t* 
   if (T <= 32768) {
     auto tile_smem = [&](int E, int threads) {
       const size_t tile_words = (size_t)threads * E;
-      const size_t need = (size_t)kTileScratch + (tile_two_hists(E, threads) && out_words < (size_t)kHistBins ? (size_t)kHistBins : out_words);
+      // (with two histograms the second one's scan scratch, 64 words, lies behind it)
+      const size_t need = (size_t)kTileScratch + (tile_two_hists(E, threads) && out_words < (size_t)kHistBins + 64 ? (size_t)kHistBins + 64 : out_words);
       return (need > tile_words ? need : tile_words) * 4;
     };
 #define CM_TOPK_TILE(E, THR)                                                              \
