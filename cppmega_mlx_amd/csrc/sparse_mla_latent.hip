@@ -187,32 +187,36 @@ __global__ __launch_bounds__(512, 2) void sparse_mla_latent_kernel(const MlaPara
   //      the same XCD and share its L2: every workgroup of one (query, KV group) gets such ids, so
   //      the gathered key rows are fetched from HBM once for both head chunks and the query rows
   //      once for all key splits ----
-  const int chunks = (p.heads_per_group + kHeadsWg - 1) / kHeadsWg;
-  const long long per_q = (long long)p.num_splits * chunks;    // workgroups of one (query, KV group)
-  const long long nq = (long long)p.B * p.S * p.G;
-  const long long nq8 = nq & ~7ll;
-  long long qg;
+  // (all of it in 32-bit unsigned arithmetic - the launcher checks that the grid fits: the same
+  // decoding with 64-bit divisions was a dependent chain of ~1000 scalar instructions in front of
+  // the first load of every workgroup)
+  const unsigned chunks = (unsigned)(p.heads_per_group + kHeadsWg - 1) / (unsigned)kHeadsWg;
+  const unsigned per_q = (unsigned)p.num_splits * chunks;      // workgroups of one (query, KV group)
+  const unsigned nq = (unsigned)p.B * (unsigned)p.S * (unsigned)p.G;
+  const unsigned nq8 = nq & ~7u;
+  unsigned qg;
   int chunk, split;
   {
     // (several queries per sequence: the last ones first - under a causal selection they hold the
     // longest key lists, and the short ones then fill the end of the launch)
-    const long long id = p.S > 1 ? (long long)gridDim.x - 1 - blockIdx.x : (long long)blockIdx.x;
-    long long r;
+    const unsigned id = p.S > 1 ? gridDim.x - 1u - blockIdx.x : blockIdx.x;
+    unsigned r;
     if (id < nq8 * per_q) {
-      const long long slot = id >> 3;
-      qg = (slot / per_q) * 8 + (id & 7);
-      r = slot % per_q;
+      const unsigned slot = id >> 3, sq = slot / per_q;
+      qg = sq * 8u + (id & 7u);
+      r = slot - sq * per_q;
     } else {
-      const long long rest = id - nq8 * per_q;
-      qg = nq8 + rest / per_q;
-      r = rest % per_q;
+      const unsigned rest = id - nq8 * per_q, rq = rest / per_q;
+      qg = nq8 + rq;
+      r = rest - rq * per_q;
     }
     split = (int)(r / chunks);
-    chunk = (int)(r % chunks);
+    chunk = (int)(r - (unsigned)split * chunks);
   }
-  const int g = (int)(qg % p.G);
-  const size_t bs = (size_t)(qg / p.G);           // b*S + s
-  const int b = (int)(bs / p.S);
+  const unsigned bs32 = qg / (unsigned)p.G;       // b*S + s
+  const int g = (int)(qg - bs32 * (unsigned)p.G);
+  const size_t bs = bs32;
+  const int b = (int)(bs32 / (unsigned)p.S);
   const int head0 = g * p.heads_per_group + chunk * kHeadsWg;
   const int heads_here = min(kHeadsWg, p.heads_per_group - chunk * kHeadsWg);
   const size_t idx_base = (bs * p.G + g) * (size_t)p.topk;
@@ -810,10 +814,11 @@ __global__ __launch_bounds__(256) void sparse_mla_latent_combine_kernel(const Ml
   const int chunks = (p.heads_per_group + 32 * HG - 1) / (32 * HG);
   const int w = (int)blockIdx.y / HG, hg = (int)blockIdx.y % HG;
   const size_t unit = blockIdx.x;                              // (b*S + s, g, chunk)
-  const int chunk = (int)(unit % chunks);
-  const size_t qg = unit / chunks;
-  const int g = (int)(qg % p.G);
-  const size_t bs = qg / p.G;
+  const unsigned qg = blockIdx.x / (unsigned)chunks;           // (32-bit divisions: the 64-bit ones are long scalar chains)
+  const int chunk = (int)(blockIdx.x - qg * (unsigned)chunks);
+  const unsigned bs32 = qg / (unsigned)p.G;
+  const int g = (int)(qg - bs32 * (unsigned)p.G);
+  const size_t bs = bs32;
   const int head0 = g * p.heads_per_group + chunk * 32 * HG;
   const int heads_here = min(32 * HG, p.heads_per_group - chunk * 32 * HG);
   const int hd = lane & 31, half = lane >> 5;

@@ -70,6 +70,38 @@ def test_integer_inputs_select_exactly_the_oracle_set(device, case, order):
         np.testing.assert_array_equal(out2.cpu().numpy(), want)
 
 
+BOUND_CASES = [
+    # B, Sq, H, D, Skv, topk: bf16 rows, so that the wavefront-per-row head sum runs
+    (1, 300, 64, 128, 2048, 64),       # sixteen heads-of-four in flight, no tail
+    (1, 200, 100, 128, 1536, 48),      # one full round of heads and a tail of 36
+    (2, 150, 8, 64, 1300, 40),         # eight heads per load: the tail loop only
+    (1, 90, 6, 256, 1024, 32),         # two heads per load
+]
+
+
+@pytest.mark.parametrize("case", BOUND_CASES, ids=lambda c: "B%d_S%d_H%d_D%d_T%d_k%d" % c)
+def test_tight_bounds_leave_unscored_keys_unread(device, case):
+    """Sliding causal windows: a query tile scores only the keys between the smallest start and the
+    largest end of its rows.  The workspace is poisoned first (NaN patterns and huge values), so a
+    selection that looked at a key nobody scored would show."""
+    B, Sq, H, D, Skv, topk = case
+    rng = np.random.default_rng(Sq + H + D)
+    q, k, w = _int_inputs(rng, B, Sq, H, D, Skv)
+    pos = (np.arange(Sq) * (Skv - 1) // max(Sq - 1, 1)).astype(np.int64)
+    ends = np.tile(pos + 1, B).astype(np.int32)
+    starts = np.maximum(ends - 400, 0).astype(np.int32)
+    want = oi.indexer_topk_oracle(q, k, w, sm_scale=0.125, index_topk=topk, starts=starts, ends=ends, order="index")
+    qt, kt, wt = (to_dev(a, device).to(torch.bfloat16) for a in (q, k, w))
+    need = ops.indexer_topk_workspace_bytes(qt, kt, wt, topk=topk)
+    for poison in (0x7fc00000, 0x7f000000):
+        ws = torch.full(((need + 3) // 4,), poison, dtype=torch.int32, device=device).view(torch.uint8)
+        out = torch.full((B, Sq, topk), -9, dtype=torch.int32, device=device)
+        ops.indexer_topk(qt, kt, wt, sm_scale=0.125, topk=topk, out=out, starts=to_dev(starts, device),
+                         ends=to_dev(ends, device), order="index", workspace=ws)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
 def test_additive_mask_and_masked_positions(device):
     rng = np.random.default_rng(5)
     B, Sq, H, D, Skv, topk = 2, 24, 4, 32, 64, 20
