@@ -168,12 +168,14 @@ struct AppendParams {
 template <bool PREPARED>
 __global__ __launch_bounds__(256) void cache_append_kernel(const AppendParams p) {
   const int lane = lane_id();
-  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);       // (b * S + s) * G + g
-  const long long rows = (long long)p.B * p.S * p.G;
+  // (32-bit arithmetic, the launcher checks that the row count fits: 64-bit divisions per
+  // wavefront were most of this kernel's instructions)
+  const unsigned row = blockIdx.x * 4u + (threadIdx.x >> 6);                  // (b * S + s) * G + g
+  const unsigned rows = (unsigned)p.B * (unsigned)p.S * (unsigned)p.G;
   if (row >= rows) return;
-  const int g = (int)(row % p.G);
-  const long long bs = row / p.G;
-  const int s = (int)(bs % p.S), b = (int)(bs / p.S);
+  const unsigned bs = row / (unsigned)p.G;
+  const int g = (int)(row - bs * (unsigned)p.G);
+  const int b = (int)(bs / (unsigned)p.S), s = (int)(bs - (unsigned)b * (unsigned)p.S);
   const int pos = (p.positions ? p.positions[b] : p.position) + s;
   if (pos < 0 || pos >= p.cap) return;                                         // (checked on the host when positions is NULL)
   const size_t crow = ((size_t)b * p.cap + pos) * p.G + g;                     // cache row
@@ -341,6 +343,7 @@ int kv_cache_append_launch(const cppmega_mi355_cache_append_args_t& a, hipStream
   p.B = a.batch; p.S = a.new_tokens; p.G = a.groups; p.D = a.dim; p.R = a.rope_dim; p.cap = a.capacity;
   p.src_dtype = a.src_dtype; p.rope_dtype = a.rope_dtype; p.scale_block = a.scale_block; p.pow2 = a.pow2_scales;
   const long long rows = (long long)a.batch * a.new_tokens * a.groups;
+  if (rows > 0x7fffffffll) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "kv_cache_append: %lld rows in one call", rows);
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   if (prepared) hipLaunchKernelGGL(cache_append_kernel<true>, grid, block, 0, stream, p);
   else hipLaunchKernelGGL(cache_append_kernel<false>, grid, block, 0, stream, p);

@@ -107,11 +107,14 @@ __device__ __forceinline__ unsigned valid16(const MaskParams& p, const unsigned 
 template <int DT>
 __global__ __launch_bounds__(256) void mask_indices_kernel(const MaskParams p) {
   const int lane = lane_id();
-  const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);           // (b * S + s) * G + g
-  if (r >= (long long)p.B * p.S * p.G) return;
-  const int g = (int)(r % p.G);
-  const long long bs = r / p.G;
-  const int s = (int)(bs % p.S), b = (int)(bs / p.S);
+  // (32-bit arithmetic, the launcher checks that the row count fits: the 64-bit divisions were
+  // several hundred instructions per wavefront)
+  const unsigned r32 = blockIdx.x * 4u + (threadIdx.x >> 6);                    // (b * S + s) * G + g
+  if (r32 >= (unsigned)p.B * (unsigned)p.S * (unsigned)p.G) return;
+  const unsigned bs = r32 / (unsigned)p.G;
+  const int g = (int)(r32 - bs * (unsigned)p.G);
+  const int b = (int)(bs / (unsigned)p.S), s = (int)(bs - (unsigned)b * (unsigned)p.S);
+  const long long r = r32;
   constexpr int ES = DT == CPPMEGA_MI355_MASK_BOOL ? 1 : (DT == CPPMEGA_MI355_MASK_F32 ? 4 : 2);
   const unsigned char* row = (const unsigned char*)p.mask + ((long long)b * p.sb + (long long)g * p.sg + (long long)s * p.ss) * ES;
   const bool vec_ok = (((size_t)row) & 15) == 0;
@@ -205,6 +208,7 @@ int mask_indices_launch(const cppmega_mi355_mask_indices_args_t& a, hipStream_t 
   p.mask = a.mask; p.sb = a.stride_b; p.sg = a.stride_g; p.ss = a.stride_s; p.out = a.indices;
   p.B = a.batch; p.S = a.seq; p.G = a.groups; p.K = a.key_length; p.n = min(a.topk, a.key_length); p.dtype = a.mask_dtype;
   const long long rows = (long long)a.batch * a.seq * a.groups;
+  if (rows > 0x7fffffffll) return fail(CPPMEGA_MI355_ERR_UNSUPPORTED, "sparse_indices_from_attention_mask: %lld rows in one call", rows);
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   switch (a.mask_dtype) {
     case CPPMEGA_MI355_MASK_BOOL: hipLaunchKernelGGL(mask_indices_kernel<CPPMEGA_MI355_MASK_BOOL>, grid, block, 0, stream, p); break;
