@@ -272,7 +272,10 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   const unsigned k = (unsigned)p.k;
 
   float v[E];
+  constexpr int kHist2 = tile_two_hists(E, THREADS) ? kHistBins + 64 : 0;
   if constexpr (DIRECT) {
+    // (no tile in LDS on this path: the histograms are cleared before the row's bounds have arrived)
+    zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
     const int c0 = tid * E;
     const bool any = c0 < end && c0 + E > start;          // (a run with nothing selectable is not read)
 #pragma unroll
@@ -307,8 +310,7 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   __syncthreads();
   }
   // two cleared histograms: pass 1 uses the first, pass 2 the second (no clear + barrier in between)
-  constexpr int kHist2 = tile_two_hists(E, THREADS) ? kHistBins + 64 : 0;
-  zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
+  if constexpr (!DIRECT) zero_hist<THREADS>(hist, kHist2 ? kHist2 + kHistBins : kHistBins);
   __syncthreads();
 
   // ---- canonicalise (-0 -> +0, NaN -> quiet NaN, masked -> NaN) + pass 1 -------------
