@@ -453,7 +453,19 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
       return;
     }
     const int* map = MODE == 2 ? p.index_map + (long long)row * p.width : nullptr;
-    for (unsigned i = tid; i < k; i += THREADS)             // (written once, not read again here: non-temporal)
+    // (written once, not read again here: non-temporal; four slots per thread and store where the
+    // row allows it - the stage starts on a 16-byte boundary)
+    if (MODE != 2 && (k & 3u) == 0 && (((size_t)out_row) & 15) == 0) {
+      typedef int i32x4_t __attribute__((ext_vector_type(4)));
+      for (unsigned i = 4 * tid; i < k; i += 4 * THREADS) {
+        i32x4_t q = *reinterpret_cast<const i32x4_t*>(stage + i);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) q[c] = (i + c < n_sel) ? q[c] : -1;
+        __builtin_nontemporal_store(q, reinterpret_cast<i32x4_t*>(out_row + i));
+      }
+      return;
+    }
+    for (unsigned i = tid; i < k; i += THREADS)
       __builtin_nontemporal_store((i < n_sel) ? (MODE == 2 ? map[stage[i]] : stage[i]) : -1, out_row + i);
     return;
   }
