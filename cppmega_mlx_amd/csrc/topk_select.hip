@@ -314,8 +314,20 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
   __syncthreads();
 
   // ---- canonicalise (-0 -> +0, NaN -> quiet NaN, masked -> NaN) + pass 1 -------------
+  // A row with no more selectable columns than k needs no threshold: everything that is a number is
+  // taken (the rows of a causal prefill whose prefix is shorter than k).
   const int col0 = tid * E;
-  if (col0 >= start && col0 + E <= end && !p.neg_inf_masked) {
+  const bool take_all = end - start <= (int)k;      // (uniform)
+  if (take_all) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      float x = v[i] + 0.0f;
+      const int idx = col0 + i;
+      x = (idx >= start && idx < end) ? x : kNaN;
+      if (p.neg_inf_masked) x = (x == kNegInf) ? kNaN : x;
+      v[i] = x;
+    }
+  } else if (col0 >= start && col0 + E <= end && !p.neg_inf_masked) {
 #pragma unroll
     for (int i = 0; i < E; ++i) {
       const float x = v[i] + 0.0f;
@@ -333,12 +345,15 @@ __global__ __launch_bounds__(THREADS, E > 16 ? 4 : 8) void topk_tile_kernel(cons
       if (x == x) atomicAdd(&hist[__float_as_uint(x) >> 20], 1u);
     }
   }
-  __syncthreads();
-
-  BinHit h1 = find_bin<kHistBins, THREADS>(smem, k, kSigned, true);
-  float thr;
+  float thr = kNegInf;
   unsigned rem = 0;
   bool tie = false;
+  BinHit h1;
+  h1.bin = 0; h1.above = 0; h1.cnt = 0; h1.total = 0;
+  if (!take_all) {
+    __syncthreads();
+    h1 = find_bin<kHistBins, THREADS>(smem, k, kSigned, true);
+  }
   if (h1.total <= k) {
     thr = kNegInf;   // every selectable element is taken
   } else {
