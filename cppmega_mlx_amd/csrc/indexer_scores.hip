@@ -212,7 +212,7 @@ constexpr int kCPitch = 68;                        // floats per row of the scor
 static_assert(16 * kCPitch * 4 <= kStageBytes, "the score tile reuses the key tile");
 
 template <bool K_F32, int KSTEPS, int QT, bool STAGED = false>
-__global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerParams p) {
+__global__ __launch_bounds__(kThreads, 2) void indexer_scores_kernel(const IndexerParams p) {
   extern __shared__ __align__(16) unsigned short q_lds[];     // [2][16 QT][Dp + 8]: hi plane, lo plane; then the staging tiles
   const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bz = (int)blockIdx.z;
@@ -303,9 +303,11 @@ __global__ __launch_bounds__(kThreads) void indexer_scores_kernel(const IndexerP
         const int row = 16 * jj + n, c = 4 * ks + kg;
         a_off[jj][ks] = (row * PPR + (c ^ ((row / RP) % PPR))) * 16;
       }
-    // The query operands do not change over the keys: they are read from LDS once (128 registers at
-    // four query tiles of 128 channels; one workgroup per CU).  Read inside the loop they were 128 KiB
-    // of LDS traffic per wavefront and 64-key step: 76 -> 71 us at 8192 x 8192 under a causal bound.
+    // The query operands do not change over the keys: they are read from LDS once (64 registers at
+    // two query tiles of 128 channels).  Two tiles and not four: the kernel then fits 256 registers,
+    // two workgroups share a CU, and one's matrix products run under the other's fetches, staging
+    // and stores - 56 us at 8192 x 8192 under a causal bound against 71 us for four tiles in 380
+    // registers (one workgroup per CU) and 76 us for four tiles with the operands read in the loop.
     // (One query tile - the decode-time shape, bound by the key stream - keeps reading them from LDS.)
     constexpr bool kHoist = QT > 1;
     bf16x8 bq[kHoist ? QT : 1][kHoist ? KSTEPS : 1][2];
@@ -562,7 +564,7 @@ int indexer_topk_workspace_bytes(const cppmega_mi355_indexer_args_t& a, size_t* 
 
 template <bool K_F32, int QT>
 static int launch_scores(const IndexerParams& p, dim3 grid, hipStream_t stream) {
-  const size_t q_bytes = (size_t)2 * kQRows * QT * (((p.D + 31) & ~31) + 8) * sizeof(unsigned short);   // <= 67.6 KB at QT = 4, D = 256: QT = 4 is only used up to D = 128
+  const size_t q_bytes = (size_t)2 * kQRows * QT * (((p.D + 31) & ~31) + 8) * sizeof(unsigned short);   // (two query tiles are only used up to D = 128: 17 KB)
   const int ks = (p.D + 31) / 32;
   if constexpr (!K_F32) {
     if (p.k_vec && p.s_vec && p.D % 32 == 0 && (ks == 1 || ks == 2 || ks == 4)) {
@@ -626,7 +628,7 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
                            stream, p);
       else
         hipLaunchKernelGGL(indexer_qw_kernel, dim3((unsigned)(nb * s_count)), dim3(kThreads), 0, stream, p);
-      const int qt = (s_count >= 4 * kQRows && a.head_dim <= 128) ? 4 : 1;     // query tiles per workgroup
+      const int qt = (s_count >= 4 * kQRows && a.head_dim <= 128) ? 2 : 1;     // query tiles per workgroup (prefill: two)
       const int tiles = (s_count + kQRows * qt - 1) / (kQRows * qt);
       const int max_splits = (a.seq_kv + kKeysPerIter - 1) / kKeysPerIter;
       int splits = (1024 + tiles * nb - 1) / (tiles * nb);
@@ -634,8 +636,8 @@ int indexer_topk_launch(const cppmega_mi355_indexer_args_t& a, hipStream_t strea
       const int per = (a.seq_kv + splits - 1) / splits;
       p.keys_per_wg = (per + kKeysPerIter - 1) / kKeysPerIter * kKeysPerIter;
       const dim3 grid((unsigned)((a.seq_kv + p.keys_per_wg - 1) / p.keys_per_wg), (unsigned)tiles, (unsigned)nb);
-      if (a.k_dtype == CPPMEGA_MI355_F32) rc = qt == 4 ? launch_scores<true, 4>(p, grid, stream) : launch_scores<true, 1>(p, grid, stream);
-      else rc = qt == 4 ? launch_scores<false, 4>(p, grid, stream) : launch_scores<false, 1>(p, grid, stream);
+      if (a.k_dtype == CPPMEGA_MI355_F32) rc = qt == 2 ? launch_scores<true, 2>(p, grid, stream) : launch_scores<true, 1>(p, grid, stream);
+      else rc = qt == 2 ? launch_scores<false, 2>(p, grid, stream) : launch_scores<false, 1>(p, grid, stream);
       if (rc) return rc;
       CM_HIP_CHECK(hipGetLastError());
 

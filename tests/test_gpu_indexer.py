@@ -36,7 +36,7 @@ INT_CASES = [
     (3, 1, 8, 64, 2048, 128, torch.bfloat16),          # decode: one query row per sequence
     (1, 5, 3, 40, 77, 77, torch.float32),              # head_dim and key count off every vector width; topk = Skv
     (1, 9, 2, 20, 130, 9, torch.bfloat16),
-    (1, 100, 8, 64, 512, 32, torch.bfloat16),          # 64 query rows per workgroup, the second one ragged
+    (1, 100, 8, 64, 512, 32, torch.bfloat16),          # 32 query rows per workgroup, the last one ragged
     (2, 70, 4, 128, 300, 16, torch.float32),
     (1, 130, 4, 96, 260, 8, torch.bfloat16),           # three 32-channel steps
 ]
