@@ -154,6 +154,13 @@ __global__ __launch_bounds__(256) void mask_indices_kernel(const MaskParams p) {
     // the step's kept keys go through this wavefront's LDS strip in rank order and leave as
     // whole 256-byte stores (a lane's keys are consecutive ranks: direct stores would scatter)
     const int step_rank0 = before - step_total;                                 // rank of the step's first valid key
+    if (step_total == 64 * 16) {
+      // every key of the step is valid (the body of a causal mask): rank = position within the step,
+      // so the kept keys are the consecutive numbers base + lo .. base + 1023 and need no strip
+      const int lo = max(first - step_rank0, 0);
+      for (int e = lo + lane; e < 64 * 16; e += 64) out[step_rank0 + e - first] = (int)(base + e);
+      continue;
+    }
     unsigned rest = bits;
     int rloc = rank - step_rank0;                                               // 0 .. 1023
     while (rest) {

@@ -66,6 +66,7 @@ def test_mask_indices_reference_known_answer(device, kats):
     ((2, 5), 1000, 64, np.bool_),             # (B,S,K)
     ((2, 3, 4), 257, 300, np.bool_),          # (B,G,S,K), topk > K
     ((2, 1, 4), 4096, 2048, np.bool_),        # (B,1,S,K) group broadcast, more than one 1024-key step
+    ((2, 1, 4), 4096, 1500, np.bool_),        # the window starts inside an all-valid 1024-key step
     ((3,), 77, 10, np.float32),
     ((2, 2), 130, 33, np.float16),
 ])
@@ -75,6 +76,8 @@ def test_mask_indices_match_oracle(device, shape, K, topk, dtype):
     if valid.ndim >= 2:
         valid[(0,) * (valid.ndim - 1)] = False        # a row with nothing valid
         valid[(-1,) * (valid.ndim - 1)] = True        # a row with everything valid
+        if K >= 4096:                                 # a causal row: whole steps valid, then a ragged one, then nothing
+            valid[(0,) * (valid.ndim - 2) + (1,)] = np.arange(K) < 2500
     if dtype == np.bool_:
         mask = valid
         t = to_dev(mask, device)
